@@ -1,0 +1,121 @@
+// Elementwise binary operators with BIDMat's broadcasting rules. Streaming kernels: 12 bytes
+// per element; the equal-shape case uses 128-bit accesses.
+#include "common.hpp"
+#include "kernels.hpp"
+#include <math.h>
+
+namespace bm {
+namespace {
+
+template <int OP>
+__device__ __forceinline__ float binop(float a, float b) {
+    if constexpr (OP == 0) return a + b;
+    else if constexpr (OP == 1) return a - b;
+    else if constexpr (OP == 2) return a * b;
+    else if constexpr (OP == 3) return a / b;
+    else if constexpr (OP == 4) return (a > b) ? 1.0f : 0.0f;
+    else if constexpr (OP == 5) return (a < b) ? 1.0f : 0.0f;
+    else if constexpr (OP == 6) return (a == b) ? 1.0f : 0.0f;
+    else if constexpr (OP == 7) return (a >= b) ? 1.0f : 0.0f;
+    else if constexpr (OP == 8) return (a <= b) ? 1.0f : 0.0f;
+    else if constexpr (OP == 9) return (a != b) ? 1.0f : 0.0f;
+    else if constexpr (OP == 10) return fmaxf(a, b);
+    else if constexpr (OP == 11) return fminf(a, b);
+    else if constexpr (OP == 12) return atan2f(a, b);
+    else if constexpr (OP == 13) return powf(a, b);
+    else return (a > 0) ? b : 0.0f;
+}
+
+// Index modes: how element i (column-major, nrows x ncols) picks its operand.
+enum Mode { FULL = 0, COL = 1, ROW = 2, VAL = 3 };
+
+template <int MODE>
+__device__ __forceinline__ long long pick(long long i, int nrows) {
+    if constexpr (MODE == FULL) return i;
+    else if constexpr (MODE == COL) return i % nrows;      // column vector: one entry per row
+    else if constexpr (MODE == ROW) return i / nrows;      // row vector: one entry per column
+    else return 0;
+}
+
+template <int OP, int MA, int MB>
+__global__ __launch_bounds__(BM_BLOCK) void k_apply(const float* __restrict__ A, const float* __restrict__ B,
+                                                    float* __restrict__ C, long long n, int nrows) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    for (; i < n; i += stride) C[i] = binop<OP>(A[pick<MA>(i, nrows)], B[pick<MB>(i, nrows)]);
+}
+
+template <int OP>
+__global__ __launch_bounds__(BM_BLOCK) void k_apply_full4(const float4* __restrict__ A, const float4* __restrict__ B,
+                                                          float4* __restrict__ C, long long n4) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    for (; i < n4; i += stride) {
+        const float4 a = A[i], b = B[i];
+        C[i] = make_float4(binop<OP>(a.x, b.x), binop<OP>(a.y, b.y), binop<OP>(a.z, b.z), binop<OP>(a.w, b.w));
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+inline unsigned grid_for(long long n) {
+    long long b = (n + BM_BLOCK - 1) / BM_BLOCK;
+    if (b < 1) b = 1;
+    if (b > 16384) b = 16384;
+    return (unsigned)b;
+}
+
+template <int OP>
+hipError_t apply_impl(const float* A, int ma, const float* B, int mb, float* C, long long n, int nrows,
+                      hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (ma == FULL && mb == FULL) {
+        long long n4 = 0;
+        if (aligned16(A) && aligned16(B) && aligned16(C)) {
+            n4 = n / 4;
+            if (n4 > 0) hipLaunchKernelGGL(k_apply_full4<OP>, dim3(grid_for(n4)), dim3(BM_BLOCK), 0, s,
+                                           (const float4*)A, (const float4*)B, (float4*)C, n4);
+        }
+        long long done = n4 * 4;
+        if (done < n) hipLaunchKernelGGL((k_apply<OP, FULL, FULL>), dim3(grid_for(n - done)), dim3(BM_BLOCK), 0, s,
+                                         A + done, B + done, C + done, n - done, nrows);
+        return hipGetLastError();
+    }
+    dim3 grid(grid_for(n)), block(BM_BLOCK);
+#define BM_M(MA_, MB_)                                                                        \
+    if (ma == MA_ && mb == MB_) {                                                             \
+        hipLaunchKernelGGL((k_apply<OP, MA_, MB_>), grid, block, 0, s, A, B, C, n, nrows);    \
+        return hipGetLastError();                                                             \
+    }
+    BM_M(FULL, COL) BM_M(FULL, ROW) BM_M(COL, FULL) BM_M(ROW, FULL) BM_M(FULL, VAL) BM_M(VAL, FULL)
+#undef BM_M
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+// Same case analysis, in the same order, as apply_binop (Operators.cu:529-553).
+hipError_t applyop(const float* A, int Anr, int Anc, const float* B, int Bnr, int Bnc, float* C,
+                   int opn, hipStream_t s) {
+    const int nr = Anr > Bnr ? Anr : Bnr;
+    const int nc = Anc > Bnc ? Anc : Bnc;
+    const long long n = (long long)nr * nc;
+    int ma, mb;
+    if (Anr == Bnr && Anc == Bnc) { ma = FULL; mb = FULL; }
+    else if (Anr == Bnr && Bnc == 1) { ma = FULL; mb = COL; }
+    else if (Anc == Bnc && Bnr == 1) { ma = FULL; mb = ROW; }
+    else if (Anr == Bnr && Anc == 1) { ma = COL; mb = FULL; }
+    else if (Anc == Bnc && Anr == 1) { ma = ROW; mb = FULL; }
+    else if (Bnr == 1 && Bnc == 1) { ma = FULL; mb = VAL; }
+    else if (Anr == 1 && Anc == 1) { ma = VAL; mb = FULL; }
+    else return hipErrorInvalidValue;      // the reference launches nothing for incompatible shapes
+    switch (opn) {
+#define BM_OP(N_) case N_: return apply_impl<N_>(A, ma, B, mb, C, n, nr, s);
+    BM_OP(0) BM_OP(1) BM_OP(2) BM_OP(3) BM_OP(4) BM_OP(5) BM_OP(6) BM_OP(7)
+    BM_OP(8) BM_OP(9) BM_OP(10) BM_OP(11) BM_OP(12) BM_OP(13) BM_OP(14)
+#undef BM_OP
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace bm

@@ -1,0 +1,429 @@
+// C ABI of libbidmathip.so: argument validation, the reference-shaped blocking launchers, the
+// native stream-taking entry points, plan handles + the fingerprint-keyed plan cache used by the
+// reference-shaped entries, and the device-memory helpers.
+#include "../../include/bidmat_hip.h"
+#include "common.hpp"
+#include "kernels.hpp"
+#include "plan.hpp"
+#include "workspace.hpp"
+#include <atomic>
+#include <cstring>
+#include <cstdio>
+#include <cstdlib>
+#include <list>
+#include <mutex>
+
+#define API extern "C" __attribute__((visibility("default")))
+
+namespace bm {
+namespace {
+std::atomic<int> g_seglen{1024};
+std::atomic<int> g_panel_kb{2048};
+}  // namespace
+int opt_seglen() { return g_seglen.load(std::memory_order_relaxed); }
+int opt_panel_kb() { return g_panel_kb.load(std::memory_order_relaxed); }
+}  // namespace bm
+
+namespace {
+
+constexpr int kInvalid = (int)hipErrorInvalidValue;
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Blocking epilogue of the reference-shaped launchers (Arith.cu:57-59).
+inline int finish_blocking(hipError_t launch_err) {
+    hipError_t sync_err = hipStreamSynchronize(nullptr);
+    if (launch_err != hipSuccess) return (int)launch_err;
+    if (sync_err != hipSuccess) return (int)sync_err;
+    return (int)hipGetLastError();
+}
+
+// ---- plan cache for entries that only receive (ir, ic): keyed by a fingerprint of both index
+// arrays, so a caller that refills the same device buffers with another pattern never meets a
+// stale plan.
+struct CacheEntry {
+    int device;
+    int ncols, nnz, nrows, k_hint;
+    unsigned long long fa, fb;
+    bidmat_plan* plan;
+};
+std::mutex g_cache_mu;
+std::list<CacheEntry> g_cache;          // most recently used first
+constexpr size_t kMaxCachedPlans = 4;
+
+hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_hint, bidmat_plan** out) {
+    *out = nullptr;
+    hipError_t err;
+    int dev = 0;
+    if ((err = hipGetDevice(&dev)) != hipSuccess) return err;
+    hipStream_t s = nullptr;
+    unsigned long long* d_misc = (unsigned long long*)bm::ws_get(bm::WS_MISC, 64, &err);
+    if (!d_misc) return err;
+    // misc layout: [0..1] fingerprints, [2] (as int) max row
+    if ((err = bm::fingerprint(ir, nnz, ic, nnz, d_misc, s)) != hipSuccess) return err;
+    int* d_max = reinterpret_cast<int*>(d_misc + 2);
+    if ((err = bm::int_max(ir, nnz, d_max, s)) != hipSuccess) return err;
+    unsigned long long h[3];
+    if ((err = hipMemcpy(h, d_misc, sizeof(h), hipMemcpyDeviceToHost)) != hipSuccess) return err;
+    int maxrow;
+    memcpy(&maxrow, &h[2], sizeof(int));
+    const int nrows = maxrow + 1;
+
+    std::lock_guard<std::mutex> lock(g_cache_mu);
+    for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
+        if (it->device == dev && it->ncols == ncols && it->nnz == nnz && it->nrows == nrows &&
+            it->fa == h[0] && it->fb == h[1]) {
+            g_cache.splice(g_cache.begin(), g_cache, it);
+            *out = g_cache.front().plan;
+            return hipSuccess;
+        }
+    }
+    int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
+    if (!jc) return err;
+    if ((err = bm::coo_compress_cols(ncols, nnz, ic, jc, s)) != hipSuccess) return err;
+    bidmat_plan* p = nullptr;
+    if ((err = bm::plan_build(nrows, ncols, nnz, ir, jc, k_hint, &p)) != hipSuccess) return err;
+    while (g_cache.size() >= kMaxCachedPlans) {
+        (void)bm::plan_free(g_cache.back().plan);
+        g_cache.pop_back();
+    }
+    g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, h[0], h[1], p});
+    *out = p;
+    return hipSuccess;
+}
+
+hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* vals, float* C, int beta,
+                       hipStream_t s) {
+    hipError_t err;
+    if ((err = bm::plan_reserve_partial(plan, k)) != hipSuccess) return err;
+    if ((err = bm::gather_segments(k, plan->nseg, A, vals, plan->pc, plan->perm, plan->segstart,
+                                   plan->partial, s)) != hipSuccess) return err;
+    return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, C, beta, s);
+}
+
+hipError_t run_spsum_rows(bidmat_plan* plan, const float* vals, float* out, int beta, hipStream_t s) {
+    hipError_t err;
+    if ((err = bm::plan_reserve_partial(plan, 1)) != hipSuccess) return err;
+    if ((err = bm::spsum_segments(plan->nseg, vals, plan->perm, plan->segstart, plan->partial, s)) != hipSuccess)
+        return err;
+    return bm::reduce_segments(1, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, out, beta, s);
+}
+
+bool plan_on_current_device(const bidmat_plan* p) {
+    int dev = -1;
+    return p && hipGetDevice(&dev) == hipSuccess && dev == p->device;
+}
+
+}  // namespace
+
+// ======================================================================== reference-shaped
+
+API int bidmat_dsmult(int nrows, int ncols, int nnz, const float* A, const float* Bdata,
+                      const int* Bir, const int* Bic, float* C) {
+    if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
+    if (nrows == 0 || ncols == 0 || nnz == 0) return 0;           // C += 0
+    if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
+    hipError_t err;
+    int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
+    if (!jc) return (int)err;
+    err = bm::coo_compress_cols(ncols, nnz, Bic, jc, nullptr);
+    if (err == hipSuccess) err = bm::dsmult_csc(nrows, ncols, nnz, A, Bdata, Bir, jc, C, 1, nullptr);
+    return finish_blocking(err);
+}
+
+API int bidmat_dsmultT(int nrows, int ncols, int nnz, const float* A, const float* Bdata,
+                       const int* Bir, const int* Bic, float* C) {
+    if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
+    if (nrows == 0 || ncols == 0 || nnz == 0) return 0;
+    if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
+    bidmat_plan* plan = nullptr;
+    hipError_t err = cached_plan(ncols, nnz, Bir, Bic, nrows, &plan);
+    if (err == hipSuccess) err = run_dsmultT(plan, nrows, A, Bdata, C, 1, nullptr);
+    return finish_blocking(err);
+}
+
+API int bidmat_dds(int nrows, int nnz, const float* A, const float* B, const int* Cir,
+                   const int* Cic, float* P) {
+    if (nrows < 0 || nnz < 0) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!Cir || !Cic || !P || (nrows > 0 && (!A || !B))) return kInvalid;
+    // the launcher has no column count: it is max(Cic)+1, and Cic is non-decreasing
+    int last = 0;
+    hipError_t err = hipMemcpy(&last, Cic + (nnz - 1), sizeof(int), hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return (int)err;
+    if (last < 0 || last == 0x7fffffff) return kInvalid;
+    const int ncols = last + 1;
+    int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
+    if (!jc) return (int)err;
+    err = bm::coo_compress_cols(ncols, nnz, Cic, jc, nullptr);
+    if (err == hipSuccess) err = bm::dds_csc(nrows, ncols, nnz, A, B, Cir, jc, P, 1, nullptr);
+    return finish_blocking(err);
+}
+
+API int bidmat_spsum(int nrows, int ncols, int nnz, const int* Air, const int* Aic, const float* P,
+                     float* B, int n) {
+    if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!Air || !Aic || !P || !B) return kInvalid;
+    hipError_t err;
+    if (n == 1) {
+        int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
+        if (!jc) return (int)err;
+        err = bm::coo_compress_cols(ncols, nnz, Aic, jc, nullptr);
+        if (err == hipSuccess) err = bm::spsum_cols(ncols, nnz, P, jc, B, 1, nullptr);
+    } else {
+        bidmat_plan* plan = nullptr;
+        err = cached_plan(ncols, nnz, Air, Aic, 0, &plan);
+        if (err == hipSuccess && plan->nrows > nrows) err = hipErrorInvalidValue;   // row index outside B
+        if (err == hipSuccess) err = run_spsum_rows(plan, P, B, 1, nullptr);
+    }
+    return finish_blocking(err);
+}
+
+API int bidmat_reduce1op(int nrows, int ncols, const float* A, float* B, float initv, int opn) {
+    if (nrows < 0 || ncols < 0) return kInvalid;
+    if (ncols == 0) return 0;
+    if (!B || (nrows > 0 && !A)) return kInvalid;
+    return finish_blocking(bm::reduce1op(nrows, ncols, A, B, initv, opn, nullptr));
+}
+
+API int bidmat_reduce2op(int nrows, int ncols, const float* A, float* B, float initv, int opn) {
+    if (nrows < 0 || ncols < 0) return kInvalid;
+    if (nrows == 0) return 0;
+    if (!B || (ncols > 0 && !A)) return kInvalid;
+    return finish_blocking(bm::reduce2op(nrows, ncols, A, B, initv, opn, nullptr));
+}
+
+API int bidmat_applyop(const float* A, int Anrows, int Ancols, const float* B, int Bnrows, int Bncols,
+                       float* C, int opn) {
+    if (Anrows < 0 || Ancols < 0 || Bnrows < 0 || Bncols < 0) return kInvalid;
+    if (opn < 0 || opn > 14) return kInvalid;
+    if ((long long)(Anrows > Bnrows ? Anrows : Bnrows) * (Ancols > Bncols ? Ancols : Bncols) == 0) return 0;
+    if (!A || !B || !C) return kInvalid;
+    return finish_blocking(bm::applyop(A, Anrows, Ancols, B, Bnrows, Bncols, C, opn, nullptr));
+}
+
+// ======================================================================== native entries
+
+API int bidmat_dsmult_csc(int k, int ncols, int nnz, const float* A, const float* Sdata,
+                          const int* Sir, const int* Sjc, float* C, int beta, void* stream) {
+    if (k < 0 || ncols < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (k == 0 || ncols == 0) return 0;
+    if (!Sjc || !C || (nnz > 0 && (!A || !Sdata || !Sir))) return kInvalid;
+    return (int)bm::dsmult_csc(k, ncols, nnz, A, Sdata, Sir, Sjc, C, beta, as_stream(stream));
+}
+
+API int bidmat_dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* Sir,
+                       const int* Sjc, float* P, int beta, void* stream) {
+    if (k < 0 || ncols < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (ncols == 0 || nnz == 0) return 0;
+    if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
+    return (int)bm::dds_csc(k, ncols, nnz, A, B, Sir, Sjc, P, beta, as_stream(stream));
+}
+
+API int bidmat_plan_create(int nrows, int ncols, int nnz, const int* Sir, const int* Sjc, int k_hint,
+                           bidmat_plan** plan) {
+    if (!plan) return kInvalid;
+    *plan = nullptr;
+    if (nrows < 0 || ncols < 0 || nnz < 0 || k_hint < 0) return kInvalid;
+    if (nnz > 0 && (!Sir || !Sjc)) return kInvalid;
+    return (int)bm::plan_build(nrows, ncols, nnz, Sir, Sjc, k_hint, plan);
+}
+
+API int bidmat_plan_destroy(bidmat_plan* plan) {
+    if (!plan) return 0;
+    return (int)bm::plan_free(plan);
+}
+
+API long long bidmat_plan_bytes(const bidmat_plan* plan) {
+    if (!plan) return 0;
+    return (long long)(plan->index_bytes + plan->partial_floats * sizeof(float));
+}
+
+API int bidmat_plan_segments(const bidmat_plan* plan) { return plan ? plan->nseg : 0; }
+
+API int bidmat_dsmultT_plan(bidmat_plan* plan, int k, const float* A, const float* Sdata, float* C,
+                            int beta, void* stream) {
+    if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (k == 0 || plan->nrows == 0) return 0;
+    if (!C || (plan->nnz > 0 && (!A || !Sdata))) return kInvalid;
+    return (int)run_dsmultT(plan, k, A, Sdata, C, beta, as_stream(stream));
+}
+
+API int bidmat_spsum_cols(int ncols, int nnz, const float* Sdata, const int* Sjc, float* out, int beta,
+                          void* stream) {
+    if (ncols < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (ncols == 0) return 0;
+    if (!Sjc || !out || (nnz > 0 && !Sdata)) return kInvalid;
+    return (int)bm::spsum_cols(ncols, nnz, Sdata, Sjc, out, beta, as_stream(stream));
+}
+
+API int bidmat_spsum_rows_plan(bidmat_plan* plan, const float* Sdata, float* out, int beta, void* stream) {
+    if (!plan || (beta != 0 && beta != 1)) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (plan->nrows == 0) return 0;
+    if (!out || (plan->nnz > 0 && !Sdata)) return kInvalid;
+    return (int)run_spsum_rows(plan, Sdata, out, beta, as_stream(stream));
+}
+
+API int bidmat_csc_expand_cols(int ncols, int nnz, const int* Sjc, int* Sic, void* stream) {
+    if (ncols < 0 || nnz < 0) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!Sjc || !Sic) return kInvalid;
+    return (int)bm::csc_expand_cols(ncols, nnz, Sjc, Sic, as_stream(stream));
+}
+
+API int bidmat_coo_compress_cols(int ncols, int nnz, const int* Sic, int* Sjc, void* stream) {
+    if (ncols < 0 || nnz < 0) return kInvalid;
+    if (!Sjc || (nnz > 0 && !Sic)) return kInvalid;
+    return (int)bm::coo_compress_cols(ncols, nnz, Sic, Sjc, as_stream(stream));
+}
+
+API int bidmat_applyop_flat(const float* A, const float* B, float* C, long long n, int opn, void* stream) {
+    if (n < 0 || opn < 0 || opn > 14) return kInvalid;
+    if (n == 0) return 0;
+    if (!A || !B || !C) return kInvalid;
+    // a flat array is a column vector longer than an int allows: walk it in int-sized pieces
+    const long long piece = 1LL << 30;
+    for (long long off = 0; off < n; off += piece) {
+        const int len = (int)((n - off) < piece ? (n - off) : piece);
+        hipError_t e = bm::applyop(A + off, len, 1, B + off, len, 1, C + off, opn, as_stream(stream));
+        if (e != hipSuccess) return (int)e;
+    }
+    return 0;
+}
+
+// ======================================================================== memory / runtime
+
+API int bidmat_device_count(int* count) { return count ? (int)hipGetDeviceCount(count) : kInvalid; }
+API int bidmat_set_device(int dev) { return (int)hipSetDevice(dev); }
+API int bidmat_get_device(int* dev) { return dev ? (int)hipGetDevice(dev) : kInvalid; }
+
+API int bidmat_malloc(void** dptr, long long bytes) {
+    if (!dptr || bytes < 0) return kInvalid;
+    *dptr = nullptr;
+    hipError_t e = hipMalloc(dptr, bytes > 0 ? (size_t)bytes : 256);
+    if (e == hipSuccess && getenv("BIDMAT_DEBUG_MEM")) {
+        size_t f = 0, t = 0;
+        (void)hipMemGetInfo(&f, &t);
+        fprintf(stderr, "[bidmathip] malloc %lld bytes, free fraction %.3f\n", bytes, t ? (double)f / t : 0.0);
+    }
+    return (int)e;
+}
+API int bidmat_free(void* dptr) { return dptr ? (int)hipFree(dptr) : 0; }
+API int bidmat_memcpy_h2d(void* dst, const void* src, long long bytes) {
+    if (bytes < 0 || (bytes > 0 && (!dst || !src))) return kInvalid;
+    return bytes ? (int)hipMemcpy(dst, src, (size_t)bytes, hipMemcpyHostToDevice) : 0;
+}
+API int bidmat_memcpy_d2h(void* dst, const void* src, long long bytes) {
+    if (bytes < 0 || (bytes > 0 && (!dst || !src))) return kInvalid;
+    return bytes ? (int)hipMemcpy(dst, src, (size_t)bytes, hipMemcpyDeviceToHost) : 0;
+}
+API int bidmat_memcpy_d2d(void* dst, const void* src, long long bytes) {
+    if (bytes < 0 || (bytes > 0 && (!dst || !src))) return kInvalid;
+    return bytes ? (int)hipMemcpy(dst, src, (size_t)bytes, hipMemcpyDeviceToDevice) : 0;
+}
+API int bidmat_memset(void* dptr, int value, long long bytes) {
+    if (bytes < 0 || (bytes > 0 && !dptr)) return kInvalid;
+    if (!bytes) return 0;
+    hipError_t e = hipMemset(dptr, value, (size_t)bytes);
+    if (e != hipSuccess) return (int)e;
+    return (int)hipStreamSynchronize(nullptr);
+}
+API int bidmat_mem_info(long long* free_bytes, long long* total_bytes) {
+    size_t f = 0, t = 0;
+    hipError_t e = hipMemGetInfo(&f, &t);
+    if (free_bytes) *free_bytes = (long long)f;
+    if (total_bytes) *total_bytes = (long long)t;
+    return (int)e;
+}
+API int bidmat_synchronize(void) { return (int)hipDeviceSynchronize(); }
+API int bidmat_host_alloc(void** hptr, long long bytes) {
+    if (!hptr || bytes < 0) return kInvalid;
+    return (int)hipHostMalloc(hptr, bytes > 0 ? (size_t)bytes : 256, hipHostMallocDefault);
+}
+API int bidmat_host_free(void* hptr) { return hptr ? (int)hipHostFree(hptr) : 0; }
+
+API int bidmat_stream_create(void** stream) {
+    if (!stream) return kInvalid;
+    hipStream_t s;
+    hipError_t e = hipStreamCreate(&s);      // default priority
+    *stream = (e == hipSuccess) ? (void*)s : nullptr;
+    return (int)e;
+}
+API int bidmat_stream_destroy(void* stream) { return stream ? (int)hipStreamDestroy(as_stream(stream)) : 0; }
+API int bidmat_stream_synchronize(void* stream) { return (int)hipStreamSynchronize(as_stream(stream)); }
+API int bidmat_event_create(void** event) {
+    if (!event) return kInvalid;
+    hipEvent_t ev;
+    hipError_t e = hipEventCreate(&ev);
+    *event = (e == hipSuccess) ? (void*)ev : nullptr;
+    return (int)e;
+}
+API int bidmat_event_destroy(void* event) { return event ? (int)hipEventDestroy((hipEvent_t)event) : 0; }
+API int bidmat_event_record(void* event, void* stream) {
+    return event ? (int)hipEventRecord((hipEvent_t)event, as_stream(stream)) : kInvalid;
+}
+API int bidmat_event_synchronize(void* event) { return event ? (int)hipEventSynchronize((hipEvent_t)event) : kInvalid; }
+API int bidmat_event_elapsed_ms(void* start, void* stop, float* ms) {
+    if (!start || !stop || !ms) return kInvalid;
+    return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop);
+}
+
+API const char* bidmat_error_string(int err) { return hipGetErrorString((hipError_t)err); }
+
+API const char* bidmat_version(void) { return "bidmathip 0.1 (gfx950, wave64, HIP)"; }
+
+API int bidmat_device_info(char* arch, int arch_len, int* compute_units, long long* total_mem) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return (int)e;
+    if (arch && arch_len > 0) {
+        strncpy(arch, prop.gcnArchName, (size_t)arch_len - 1);
+        arch[arch_len - 1] = 0;
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (total_mem) *total_mem = (long long)prop.totalGlobalMem;
+    return 0;
+}
+
+API int bidmat_set_option(const char* name, long long value) {
+    if (!name) return kInvalid;
+    if (!strcmp(name, "seglen")) {
+        if (value < 64 || value > (1 << 24)) return kInvalid;
+        bm::g_seglen.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "panel_kb")) {
+        if (value < 16 || value > (1 << 22)) return kInvalid;
+        bm::g_panel_kb.store((int)value);
+        return 0;
+    }
+    return kInvalid;
+}
+
+API long long bidmat_get_option(const char* name) {
+    if (!name) return -1;
+    if (!strcmp(name, "seglen")) return bm::opt_seglen();
+    if (!strcmp(name, "panel_kb")) return bm::opt_panel_kb();
+    return -1;
+}
+
+API int bidmat_release_caches(void) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    (void)hipDeviceSynchronize();
+    {
+        std::lock_guard<std::mutex> lock(g_cache_mu);
+        for (auto it = g_cache.begin(); it != g_cache.end();) {
+            if (it->device == dev) { (void)bm::plan_free(it->plan); it = g_cache.erase(it); }
+            else ++it;
+        }
+    }
+    return (int)bm::ws_release();
+}

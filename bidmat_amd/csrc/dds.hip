@@ -1,0 +1,174 @@
+// Sampled dense-dense products on a sparse pattern: P[j] = dot(A[:,ir[j]], B[:,c]) for every
+// stored nonzero j of column c.
+//
+// One wavefront owns a column (long columns: seglen-sized segments, extra waves take the
+// overflow segments; no reduction is needed between segments). The column of B stays in
+// registers for the whole segment. A group of LPN lanes covers one column of A, so a wave
+// gathers 64/LPN columns of A per load instruction; the dot product is finished with a
+// butterfly inside the group (DPP inside 16-lane rows) and each lane keeps the result of
+// "its" nonzero, so a chunk of 64 results is written with one coalesced store.
+#include "common.hpp"
+#include "kernels.hpp"
+#include "workspace.hpp"
+
+namespace bm {
+namespace {
+
+struct DdsArgs {
+    int k;
+    int ncols;
+    int seglen;
+    int beta;
+    const float* A;
+    const float* B;
+    const int* ir;
+    const int* jc;
+    const int* ovf;
+    float* P;
+};
+
+template <int V, int LPN>
+struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw < 1 ? 1 : (raw > LPN ? LPN : raw); };
+
+template <int W, int V, int LPN, bool EXACT, bool FULL>
+__device__ __forceinline__ void dds_chunk(const DdsArgs& a, int j0, int rem, int g, int l,
+                                          const int (&eld)[V], const bool (&ev)[V],
+                                          const Vec<W> (&b)[V], bool accumulate) {
+    constexpr int NG = 64 / LPN;
+    constexpr int U = Unroll<V, LPN>::U;
+    const int q = l * NG + g;            // the nonzero of this chunk whose result this lane keeps
+    int myrow = 0;
+    if (FULL || q < rem) myrow = a.ir[j0 + q];
+    float res = 0.f;
+    const int niter = FULL ? LPN : (rem + NG - 1) / NG;
+    for (int it0 = 0; it0 < niter; it0 += U) {
+        Vec<W> av[U][V];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int it = it0 + u;
+            int r;
+            if constexpr (LPN == 64) r = __builtin_amdgcn_readlane(myrow, it);
+            else r = lane_read(myrow, g * LPN + it);
+            const float* ap = a.A + (size_t)r * (size_t)a.k;
+#pragma unroll
+            for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                Vec<W> x = av[u][i];
+                if (!EXACT) x = ev[i] ? x : Vec<W>::zero();   // lanes past k contribute nothing
+                s = x.dotacc(b[i], s);
+            }
+            s = group_allsum<LPN>(s);
+            res = (l == it0 + u) ? s : res;
+        }
+    }
+    if (FULL || q < rem) {
+        float* o = a.P + j0 + q;
+        *o = accumulate ? (*o + res) : res;
+    }
+}
+
+template <int W, int V, int LPN, bool EXACT>
+__global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
+    constexpr int KT = W * V * LPN;
+    const int lane = threadIdx.x & 63;
+    const long long w = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+    const int g = lane / LPN, l = lane % LPN;
+
+    int c, jstart, jend;
+    if (w < a.ncols) {
+        c = (int)w;
+        const int s = a.jc[c], e = a.jc[c + 1];
+        jstart = s;
+        jend = (e - s > a.seglen) ? s + a.seglen : e;
+    } else {
+        if (a.ovf == nullptr) return;
+        const long long x = w - a.ncols;
+        if (x >= a.ovf[a.ncols]) return;
+        int lo = 0, hi = a.ncols;        // ovf[lo] <= x < ovf[hi]
+        while (hi - lo > 1) {
+            const int mid = (int)(((long long)lo + hi) >> 1);
+            if (a.ovf[mid] <= x) lo = mid; else hi = mid;
+        }
+        c = lo;
+        const long long qseg = x - a.ovf[lo] + 1;
+        const long long s = (long long)a.jc[lo] + qseg * a.seglen;
+        const long long e = a.jc[lo + 1];
+        jstart = (int)s;
+        jend = (int)((e - s > a.seglen) ? s + a.seglen : e);
+    }
+    if (jstart >= jend) return;
+
+    const float* bp = a.B + (size_t)c * (size_t)a.k;
+    for (int k0 = 0; k0 < a.k; k0 += KT) {
+        int eld[V];
+        bool ev[V];
+        Vec<W> b[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const int e = k0 + (i * LPN + l) * W;
+            ev[i] = e < a.k;
+            eld[i] = ev[i] ? e : 0;
+            b[i] = ev[i] ? Vec<W>::load(bp + e) : Vec<W>::zero();
+        }
+        const bool accumulate = (a.beta != 0) || (k0 > 0);
+        int j0 = jstart;
+        for (; j0 + 64 <= jend; j0 += 64)
+            dds_chunk<W, V, LPN, EXACT, true>(a, j0, 64, g, l, eld, ev, b, accumulate);
+        if (j0 < jend) dds_chunk<W, V, LPN, EXACT, false>(a, j0, jend - j0, g, l, eld, ev, b, accumulate);
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+hipError_t launch_dds(const Shape& sh, bool exact, const DdsArgs& a, long long nwaves, hipStream_t s) {
+    if (nwaves <= 0) return hipSuccess;
+    long long nblk = (nwaves + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)nblk), block(BM_BLOCK);
+#define BM_CASE(W_, V_, L_, E_)                                                          \
+    if (sh.W == W_ && sh.V == V_ && sh.LPN == L_ && exact == E_) {                       \
+        hipLaunchKernelGGL((k_dds<W_, V_, L_, E_>), grid, block, 0, s, a);               \
+        return hipGetLastError();                                                        \
+    }
+#define BM_CASES(W_, E_)                                                                 \
+    BM_CASE(W_, 1, 1, E_) BM_CASE(W_, 1, 2, E_) BM_CASE(W_, 1, 4, E_) BM_CASE(W_, 1, 8, E_) \
+    BM_CASE(W_, 1, 16, E_) BM_CASE(W_, 1, 32, E_) BM_CASE(W_, 1, 64, E_) BM_CASE(W_, 2, 64, E_) \
+    BM_CASE(W_, 4, 64, E_)
+    BM_CASES(1, false)
+    BM_CASES(4, false)
+    BM_CASES(4, true)
+#undef BM_CASES
+#undef BM_CASE
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
+                   const int* jc, float* P, int beta, hipStream_t s) {
+    if (ncols <= 0 || nnz <= 0) return hipSuccess;
+    if (k <= 0) {
+        // empty dot products: P = beta*P + 0
+        if (!beta) return fill_f32(P, nnz, 0.f, s);
+        return hipSuccess;
+    }
+    const int seglen = opt_seglen();
+    int* ovf = nullptr;
+    hipError_t err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
+    if (err != hipSuccess) return err;
+    long long novf_max = ovf ? nnz / seglen : 0;
+    Shape sh = pick_shape(k, aligned16(A) && aligned16(B));
+    if (sh.V > 4) sh.V = 4;
+    const bool exact = (sh.W == 4) && (k % (sh.W * sh.V * sh.LPN) == 0);
+    DdsArgs a;
+    a.k = k; a.ncols = ncols; a.seglen = seglen; a.beta = beta;
+    a.A = A; a.B = B; a.ir = ir; a.jc = jc; a.ovf = ovf; a.P = P;
+    return launch_dds(sh, exact, a, (long long)ncols + novf_max, s);
+}
+
+}  // namespace bm

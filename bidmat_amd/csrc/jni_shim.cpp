@@ -1,0 +1,100 @@
+// JNI entry points for a Scala/Java host (class edu.berkeley.bid.HIPMAT). They forward to the
+// C ABI one to one; device addresses travel as jlong, so no JCuda Pointer objects and no cached
+// field ids are needed (the reference unwraps jcuda.Pointer in PointerUtils.cpp:353-363 and
+// caches field ids in JNI_OnLoad, BIDMat_CUMAT.cpp:11-29).
+// Compiled only where a JDK's <jni.h> is on the include path; elsewhere this file is empty.
+#if defined(__has_include)
+#if __has_include(<jni.h>)
+#define BIDMAT_HAVE_JNI 1
+#endif
+#endif
+
+#ifdef BIDMAT_HAVE_JNI
+#include <jni.h>
+#include "../../include/bidmat_hip.h"
+
+#define P(T, x) reinterpret_cast<T*>(static_cast<intptr_t>(x))
+#define JFN(ret, name) extern "C" JNIEXPORT ret JNICALL Java_edu_berkeley_bid_HIPMAT_##name
+
+// replaces Java_edu_berkeley_bid_CUMAT_dsmult (BIDMat_CUMAT.cpp:722-733)
+JFN(jint, dsmult)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong A, jlong Bdata, jlong Bir, jlong Bic, jlong C) {
+    return bidmat_dsmult(nr, nc, nnz, P(const float, A), P(const float, Bdata), P(const int, Bir), P(const int, Bic), P(float, C));
+}
+// replaces Java_edu_berkeley_bid_CUMAT_dsmultT (BIDMat_CUMAT.cpp:761-772)
+JFN(jint, dsmultT)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong A, jlong Bdata, jlong Bir, jlong Bic, jlong C) {
+    return bidmat_dsmultT(nr, nc, nnz, P(const float, A), P(const float, Bdata), P(const int, Bir), P(const int, Bic), P(float, C));
+}
+// replaces Java_edu_berkeley_bid_CUMAT_dds (BIDMat_CUMAT.cpp:774-785)
+JFN(jint, dds)(JNIEnv*, jclass, jint nr, jint nnz, jlong A, jlong B, jlong Cir, jlong Cic, jlong Pv) {
+    return bidmat_dds(nr, nnz, P(const float, A), P(const float, B), P(const int, Cir), P(const int, Cic), P(float, Pv));
+}
+// replaces Java_edu_berkeley_bid_CUMAT_spsum (BIDMat_CUMAT.cpp:873-882)
+JFN(jint, spsum)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong Air, jlong Aic, jlong Pv, jlong B, jint n) {
+    return bidmat_spsum(nr, nc, nnz, P(const int, Air), P(const int, Aic), P(const float, Pv), P(float, B), n);
+}
+// replaces Java_edu_berkeley_bid_CUMAT_reduce1op / reduce2op (BIDMat_CUMAT.cpp:800-808, 838-846)
+JFN(jint, reduce1op)(JNIEnv*, jclass, jint nr, jint nc, jlong A, jlong B, jfloat initv, jint opn) {
+    return bidmat_reduce1op(nr, nc, P(const float, A), P(float, B), initv, opn);
+}
+JFN(jint, reduce2op)(JNIEnv*, jclass, jint nr, jint nc, jlong A, jlong B, jfloat initv, jint opn) {
+    return bidmat_reduce2op(nr, nc, P(const float, A), P(float, B), initv, opn);
+}
+// replaces Java_edu_berkeley_bid_CUMAT_applyop
+JFN(jint, applyop)(JNIEnv*, jclass, jlong A, jint Anr, jint Anc, jlong B, jint Bnr, jint Bnc, jlong C, jint opn) {
+    return bidmat_applyop(P(const float, A), Anr, Anc, P(const float, B), Bnr, Bnc, P(float, C), opn);
+}
+// native entries (column pointer + beta), used by the patched GMat.madd / GSMat.DDS
+JFN(jint, dsmultCsc)(JNIEnv*, jclass, jint k, jint nc, jint nnz, jlong A, jlong Sdata, jlong Sir, jlong Sjc, jlong C, jint beta) {
+    int e = bidmat_dsmult_csc(k, nc, nnz, P(const float, A), P(const float, Sdata), P(const int, Sir), P(const int, Sjc), P(float, C), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jint, ddsCsc)(JNIEnv*, jclass, jint k, jint nc, jint nnz, jlong A, jlong B, jlong Sir, jlong Sjc, jlong Pv, jint beta) {
+    int e = bidmat_dds_csc(k, nc, nnz, P(const float, A), P(const float, B), P(const int, Sir), P(const int, Sjc), P(float, Pv), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jlong, planCreate)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong Sir, jlong Sjc, jint khint) {
+    bidmat_plan* p = nullptr;
+    int e = bidmat_plan_create(nr, nc, nnz, P(const int, Sir), P(const int, Sjc), khint, &p);
+    return e ? -(jlong)e : (jlong)reinterpret_cast<intptr_t>(p);
+}
+JFN(jint, planDestroy)(JNIEnv*, jclass, jlong plan) { return bidmat_plan_destroy(P(bidmat_plan, plan)); }
+JFN(jint, dsmultTPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong Sdata, jlong C, jint beta) {
+    int e = bidmat_dsmultT_plan(P(bidmat_plan, plan), k, P(const float, A), P(const float, Sdata), P(float, C), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jint, cscExpandCols)(JNIEnv*, jclass, jint nc, jint nnz, jlong Sjc, jlong Sic) {
+    int e = bidmat_csc_expand_cols(nc, nnz, P(const int, Sjc), P(int, Sic), nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jlong, malloc)(JNIEnv*, jclass, jlong bytes) {
+    void* p = nullptr;
+    return bidmat_malloc(&p, bytes) ? 0 : (jlong)reinterpret_cast<intptr_t>(p);
+}
+JFN(jint, free)(JNIEnv*, jclass, jlong p) { return bidmat_free(P(void, p)); }
+JFN(jint, memset)(JNIEnv*, jclass, jlong p, jint v, jlong bytes) { return bidmat_memset(P(void, p), v, bytes); }
+JFN(jint, copyFloatsToDevice)(JNIEnv* env, jclass, jlong dst, jfloatArray src, jlong n) {
+    void* h = env->GetPrimitiveArrayCritical(src, nullptr);
+    int e = bidmat_memcpy_h2d(P(void, dst), h, n * 4);
+    env->ReleasePrimitiveArrayCritical(src, h, JNI_ABORT);
+    return e;
+}
+JFN(jint, copyIntsToDevice)(JNIEnv* env, jclass, jlong dst, jintArray src, jlong n) {
+    void* h = env->GetPrimitiveArrayCritical(src, nullptr);
+    int e = bidmat_memcpy_h2d(P(void, dst), h, n * 4);
+    env->ReleasePrimitiveArrayCritical(src, h, JNI_ABORT);
+    return e;
+}
+JFN(jint, copyFloatsFromDevice)(JNIEnv* env, jclass, jfloatArray dst, jlong src, jlong n) {
+    void* h = env->GetPrimitiveArrayCritical(dst, nullptr);
+    int e = bidmat_memcpy_d2h(h, P(const void, src), n * 4);
+    env->ReleasePrimitiveArrayCritical(dst, h, 0);
+    return e;
+}
+JFN(jint, copyIntsFromDevice)(JNIEnv* env, jclass, jintArray dst, jlong src, jlong n) {
+    void* h = env->GetPrimitiveArrayCritical(dst, nullptr);
+    int e = bidmat_memcpy_d2h(h, P(const void, src), n * 4);
+    env->ReleasePrimitiveArrayCritical(dst, h, 0);
+    return e;
+}
+JFN(jstring, errorString)(JNIEnv* env, jclass, jint err) { return env->NewStringUTF(bidmat_error_string(err)); }
+#endif  // BIDMAT_HAVE_JNI

@@ -1,0 +1,59 @@
+// Host-side launchers of the gfx950 kernels (internal to the library; the C ABI in
+// capi.cpp validates arguments and calls these).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace bm {
+
+// ---- tunables (capi.cpp owns the storage)
+int opt_seglen();      // nonzeros per wave segment for long columns / rows
+int opt_panel_kb();    // KiB of A per column panel in a plan
+
+// ---- CSC utilities (csc_util.hip)
+hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);
+hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStream_t s);
+// out[i] = v for i < n (a kernel, so that callers may record it into a HIP graph)
+hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
+hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);
+// max over an int array (result written to *d_out, a device int; empty -> -1)
+hipError_t int_max(const int* d_in, long long n, int* d_out, hipStream_t s);
+// order-sensitive 64-bit fingerprint of two int arrays (device result, 2 x uint64)
+hipError_t fingerprint(const int* a, long long na, const int* b, long long nb,
+                       unsigned long long* d_out, hipStream_t s);
+
+// ---- overflow-segment table shared by dsmult and dds (spmm.hip)
+// Returns in *d_ovf a device table int[ncols+1] (exclusive scan of the number of extra
+// seglen-sized segments of each column), or nullptr when no column can exceed seglen.
+hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, int** d_ovf,
+                                hipStream_t s);
+
+// ---- A*S (spmm.hip)
+hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* vals, const int* ir,
+                      const int* jc, float* C, int beta, hipStream_t s);
+// ---- DDS (dds.hip)
+hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
+                   const int* jc, float* P, int beta, hipStream_t s);
+
+// ---- plan stage kernels (spmm.hip): segment s gathers columns pc[p] of A scaled by
+// vals[perm[p]] for p in [segstart[s], segstart[s+1]) into partial[s*k ..].
+hipError_t gather_segments(int k, int nseg, const float* A, const float* vals, const int* pc,
+                           const int* perm, const int* segstart, float* partial, hipStream_t s);
+// C[:,r] = beta*C[:,r] + sum over q in [rowptr[r], rowptr[r+1]) of partial[rowseg[q]*k ..]
+hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
+                           const float* partial, float* C, int beta, hipStream_t s);
+
+// ---- sums (sums.hip)
+hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, float* out, int beta,
+                      hipStream_t s);
+hipError_t spsum_segments(int nseg, const float* vals, const int* perm, const int* segstart,
+                          float* partial, hipStream_t s);
+hipError_t reduce1op(int nrows, int ncols, const float* A, float* B, float initv, int opn,
+                     hipStream_t s);
+hipError_t reduce2op(int nrows, int ncols, const float* A, float* B, float initv, int opn,
+                     hipStream_t s);
+
+// ---- elementwise (applyop.hip)
+hipError_t applyop(const float* A, int Anr, int Anc, const float* B, int Bnr, int Bnc, float* C,
+                   int opn, hipStream_t s);
+
+}  // namespace bm

@@ -1,0 +1,329 @@
+// Gather-accumulate kernels: C = beta*C + A*S over CSC columns (dsmult) and the segment
+// stage of the row-binned plan (dsmultT).
+//
+// Scheduling: one wavefront owns one column (or one plan segment). A column longer than
+// `seglen` nonzeros is cut into seglen-sized segments; the first stays with the column's
+// wave, the others are "overflow" segments picked up by extra waves that write k-vector
+// partial sums, added to C afterwards in a fixed order (no atomics, deterministic).
+//
+// Data movement: a dense column of k floats is covered by a group of LPN lanes holding V
+// vectors of W floats each (W = 4: 128-bit loads). With LPN < 64 a wave works on 64/LPN
+// nonzeros per load instruction. Index/value arrays are read 64 at a time, coalesced, and
+// handed to the owning group by lane reads; U independent gathers are issued back to back
+// before their FMAs to keep the memory pipeline full.
+#include "common.hpp"
+#include "kernels.hpp"
+#include "scan.hpp"
+#include "workspace.hpp"
+
+namespace bm {
+namespace {
+
+struct GatherArgs {
+    int k;
+    int nfirst;          // columns (CSC mode) or segments (plan mode)
+    int seglen;
+    int beta;
+    const float* A;
+    const float* vals;
+    const int* idx;      // ir (CSC mode) / pc (plan mode): which column of A to gather
+    const int* perm;     // plan mode: position of the value in the original CSC order
+    const int* ptr;      // jc (CSC mode) / segstart (plan mode)
+    const int* ovf;      // CSC mode: overflow table (nullable)
+    float* out;          // C (CSC mode) / partial (plan mode)
+    float* partial;      // CSC mode: partial sums of overflow segments
+};
+
+template <int V, int LPN>
+struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw < 1 ? 1 : (raw > LPN ? LPN : raw); };
+
+template <int W, int V, int LPN, bool PLAN, bool FULL>
+__device__ __forceinline__ void gather_chunk(const GatherArgs& a, int j0, int rem, int g, int l,
+                                             const int (&eld)[V], Vec<W> (&acc)[V]) {
+    constexpr int NG = 64 / LPN;
+    constexpr int U = Unroll<V, LPN>::U;
+    // lane (g,l) holds nonzero q = l*NG + g of the chunk, so group g meets its nonzeros
+    // q = it*NG + g in lane l == it of its own group.
+    const int q = l * NG + g;
+    int myrow = 0;
+    float myval = 0.f;
+    if (FULL || q < rem) {
+        const int p = j0 + q;
+        myrow = a.idx[p];
+        myval = PLAN ? a.vals[a.perm[p]] : a.vals[p];
+    }
+    const int niter = FULL ? LPN : (rem + NG - 1) / NG;
+    for (int it0 = 0; it0 < niter; it0 += U) {
+        Vec<W> av[U][V];
+        float vv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int it = it0 + u;
+            int r;
+            if constexpr (LPN == 64) {
+                r = __builtin_amdgcn_readlane(myrow, it);
+                vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myval), it));
+            } else {
+                const int src = g * LPN + it;
+                r = lane_read(myrow, src);
+                vv[u] = lane_read(myval, src);
+            }
+            const float* ap = a.A + (size_t)r * (size_t)a.k;
+#pragma unroll
+            for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
+            if (!FULL) {
+                // past the end of the segment: lane data is (row 0, value 0); drop the load so
+                // that a non-finite entry of A's column 0 cannot leak in as 0*inf.
+                const bool ok = (it * NG + g) < rem;
+#pragma unroll
+                for (int i = 0; i < V; ++i) av[u][i] = ok ? av[u][i] : Vec<W>::zero();
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i].fma(av[u][i], vv[u]);
+        }
+    }
+}
+
+template <int W>
+__device__ __forceinline__ Vec<W> vec_xor_add(Vec<W> x, int m);
+template <>
+__device__ __forceinline__ Vec<1> vec_xor_add<1>(Vec<1> x, int m) {
+    x.x += __shfl_xor(x.x, m, 64);
+    return x;
+}
+template <>
+__device__ __forceinline__ Vec<4> vec_xor_add<4>(Vec<4> x, int m) {
+    x.v.x += __shfl_xor(x.v.x, m, 64);
+    x.v.y += __shfl_xor(x.v.y, m, 64);
+    x.v.z += __shfl_xor(x.v.z, m, 64);
+    x.v.w += __shfl_xor(x.v.w, m, 64);
+    return x;
+}
+
+template <int W, int V, int LPN, bool PLAN>
+__global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
+    constexpr int KT = W * V * LPN;      // elements of a dense column covered per pass
+    const int lane = threadIdx.x & 63;
+    const long long w = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+    const int g = lane / LPN, l = lane % LPN;
+
+    // ---- which segment does this wave own (all wave-uniform)
+    int jstart, jend;
+    float* outp;
+    bool accumulate;
+    if (PLAN) {
+        if (w >= a.nfirst) return;
+        jstart = a.ptr[w];
+        jend = a.ptr[w + 1];
+        outp = a.out + (size_t)w * (size_t)a.k;
+        accumulate = false;
+    } else if (w < a.nfirst) {
+        const int s = a.ptr[w], e = a.ptr[w + 1];
+        jstart = s;
+        jend = (e - s > a.seglen) ? s + a.seglen : e;
+        outp = a.out + (size_t)w * (size_t)a.k;
+        accumulate = a.beta != 0;
+    } else {
+        if (a.ovf == nullptr) return;
+        const long long x = w - a.nfirst;
+        if (x >= a.ovf[a.nfirst]) return;
+        int lo = 0, hi = a.nfirst;       // ovf[lo] <= x < ovf[hi]
+        while (hi - lo > 1) {
+            const int mid = (int)(((long long)lo + hi) >> 1);
+            if (a.ovf[mid] <= x) lo = mid; else hi = mid;
+        }
+        const long long qseg = x - a.ovf[lo] + 1;
+        const long long s = (long long)a.ptr[lo] + qseg * a.seglen;
+        const long long e = a.ptr[lo + 1];
+        jstart = (int)s;
+        jend = (int)((e - s > a.seglen) ? s + a.seglen : e);
+        outp = a.partial + (size_t)x * (size_t)a.k;
+        accumulate = false;
+    }
+
+    for (int k0 = 0; k0 < a.k; k0 += KT) {
+        int est[V], eld[V];
+        bool ev[V];
+        Vec<W> acc[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            est[i] = k0 + (i * LPN + l) * W;
+            ev[i] = est[i] < a.k;
+            eld[i] = ev[i] ? est[i] : 0;     // lanes past k re-read element 0; never stored
+            acc[i] = Vec<W>::zero();
+        }
+        int j0 = jstart;
+        for (; j0 + 64 <= jend; j0 += 64) gather_chunk<W, V, LPN, PLAN, true>(a, j0, 64, g, l, eld, acc);
+        if (j0 < jend) gather_chunk<W, V, LPN, PLAN, false>(a, j0, jend - j0, g, l, eld, acc);
+
+#pragma unroll
+        for (int m = LPN; m < 64; m <<= 1) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] = vec_xor_add<W>(acc[i], m);
+        }
+        if (g == 0) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                if (ev[i]) {
+                    float* o = outp + est[i];
+                    Vec<W> r = acc[i];
+                    if (accumulate) r.add(Vec<W>::load(o));
+                    r.store(o);
+                }
+            }
+        }
+    }
+}
+
+// C[:,c] += sum of the overflow partials of column c, in segment order.
+__global__ __launch_bounds__(BM_BLOCK) void k_overflow_reduce(int k, int ncols, const int* __restrict__ ovf,
+                                                              const float* __restrict__ partial,
+                                                              float* __restrict__ C) {
+    const int lane = threadIdx.x & 63;
+    const long long w = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + (threadIdx.x >> 6);
+    if (w >= ncols) return;
+    const int s = ovf[w], e = ovf[w + 1];
+    if (s == e) return;
+    for (int el = lane; el < k; el += 64) {
+        float acc = C[(size_t)w * k + el];
+        for (int q = s; q < e; ++q) acc += partial[(size_t)q * k + el];
+        C[(size_t)w * k + el] = acc;
+    }
+}
+
+__global__ __launch_bounds__(BM_BLOCK) void k_extra_segments(int ncols, const int* __restrict__ jc, int seglen,
+                                                             int* __restrict__ extra) {
+    const long long c = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    if (c >= ncols) return;
+    const int len = jc[c + 1] - jc[c];
+    extra[c] = len > seglen ? (len - 1) / seglen : 0;
+}
+
+// Plan stage 2: rows handled by groups of LPR lanes.
+template <int W>
+__global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int nrows, int lpr,
+                                                              const int* __restrict__ rowptr,
+                                                              const int* __restrict__ rowseg,
+                                                              const float* __restrict__ partial,
+                                                              float* __restrict__ C, int beta) {
+    const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long row = t / lpr;
+    const int l = (int)(t % lpr);
+    if (row >= nrows) return;
+    const int s = rowptr[row], e = rowptr[row + 1];
+    for (int el = l * W; el < k; el += lpr * W) {
+        float* o = C + (size_t)row * k + el;
+        Vec<W> acc = beta ? Vec<W>::load(o) : Vec<W>::zero();
+        for (int q = s; q < e; ++q) acc.add(Vec<W>::load(partial + (size_t)rowseg[q] * k + el));
+        acc.store(o);
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <bool PLAN>
+hipError_t launch_gather(const Shape& sh, const GatherArgs& a, long long nwaves, hipStream_t s) {
+    if (nwaves <= 0) return hipSuccess;
+    long long nblk = (nwaves + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)nblk), block(BM_BLOCK);
+#define BM_CASE(W_, V_, L_)                                                              \
+    if (sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                                      \
+        hipLaunchKernelGGL((k_gather_axpy<W_, V_, L_, PLAN>), grid, block, 0, s, a);     \
+        return hipGetLastError();                                                        \
+    }
+#define BM_CASES(W_)                                                                     \
+    BM_CASE(W_, 1, 1) BM_CASE(W_, 1, 2) BM_CASE(W_, 1, 4) BM_CASE(W_, 1, 8) BM_CASE(W_, 1, 16) \
+    BM_CASE(W_, 1, 32) BM_CASE(W_, 1, 64) BM_CASE(W_, 2, 64) BM_CASE(W_, 4, 64)
+    BM_CASES(1)
+    BM_CASES(4)
+#undef BM_CASES
+#undef BM_CASE
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+// Columns wider than 4*64 vectors are processed in passes of V = 4 inside the kernel.
+static Shape clamp_shape(Shape sh) {
+    if (sh.V > 4) sh.V = 4;
+    return sh;
+}
+
+hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, int** d_ovf, hipStream_t s) {
+    *d_ovf = nullptr;
+    if (nnz <= seglen || ncols <= 0) return hipSuccess;
+    hipError_t err;
+    int* buf = (int*)ws_get(WS_OVF, sizeof(int) * (2 * (size_t)ncols + 2), &err);
+    if (!buf) return err;
+    int* tmp = (int*)ws_get(WS_SCAN, sizeof(int) * scan_tmp_ints(ncols), &err);
+    if (!tmp) return err;
+    int* extra = buf;
+    int* ovf = buf + ncols + 1;
+    unsigned nblk = (unsigned)(((long long)ncols + BM_BLOCK - 1) / BM_BLOCK);
+    hipLaunchKernelGGL(k_extra_segments, dim3(nblk), dim3(BM_BLOCK), 0, s, ncols, jc, seglen, extra);
+    err = scan_exclusive_i32(extra, ovf, ncols, tmp, s);
+    if (err != hipSuccess) return err;
+    *d_ovf = ovf;
+    return hipGetLastError();
+}
+
+hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* vals, const int* ir,
+                      const int* jc, float* C, int beta, hipStream_t s) {
+    if (k <= 0 || ncols <= 0) return hipSuccess;
+    const int seglen = opt_seglen();
+    int* ovf = nullptr;
+    hipError_t err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
+    if (err != hipSuccess) return err;
+    float* partial = nullptr;
+    long long novf_max = 0;
+    if (ovf) {
+        novf_max = nnz / seglen;
+        partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err);
+        if (!partial) return err;
+    }
+    Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(C) && aligned16(partial)));
+    GatherArgs a;
+    a.k = k; a.nfirst = ncols; a.seglen = seglen; a.beta = beta;
+    a.A = A; a.vals = vals; a.idx = ir; a.perm = nullptr; a.ptr = jc; a.ovf = ovf;
+    a.out = C; a.partial = partial;
+    err = launch_gather<false>(sh, a, (long long)ncols + novf_max, s);
+    if (err != hipSuccess) return err;
+    if (ovf) {
+        unsigned nblk = (unsigned)(((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK);
+        hipLaunchKernelGGL(k_overflow_reduce, dim3(nblk), dim3(BM_BLOCK), 0, s, k, ncols, ovf, partial, C);
+        err = hipGetLastError();
+    }
+    return err;
+}
+
+hipError_t gather_segments(int k, int nseg, const float* A, const float* vals, const int* pc,
+                           const int* perm, const int* segstart, float* partial, hipStream_t s) {
+    if (k <= 0 || nseg <= 0) return hipSuccess;
+    Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(partial)));
+    GatherArgs a;
+    a.k = k; a.nfirst = nseg; a.seglen = 0; a.beta = 0;
+    a.A = A; a.vals = vals; a.idx = pc; a.perm = perm; a.ptr = segstart; a.ovf = nullptr;
+    a.out = partial; a.partial = nullptr;
+    return launch_gather<true>(sh, a, nseg, s);
+}
+
+hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
+                           const float* partial, float* C, int beta, hipStream_t s) {
+    if (k <= 0 || nrows <= 0) return hipSuccess;
+    const bool al = aligned16(C) && aligned16(partial) && (k % 4 == 0);
+    const int W = al ? 4 : 1;
+    int nv = (k + W - 1) / W;
+    int lpr = pow2ceil(nv) < 64 ? pow2ceil(nv) : 64;
+    long long threads = (long long)nrows * lpr;
+    long long nblk = (threads + BM_BLOCK - 1) / BM_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (al) hipLaunchKernelGGL(k_reduce_segments<4>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, nrows, lpr, rowptr, rowseg, partial, C, beta);
+    else hipLaunchKernelGGL(k_reduce_segments<1>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, nrows, lpr, rowptr, rowseg, partial, C, beta);
+    return hipGetLastError();
+}
+
+}  // namespace bm

@@ -1,0 +1,204 @@
+// Column / row reductions of sparse values and of dense matrices. All are streaming,
+// bandwidth-bound kernels; every sum has a fixed order (two-stage, no atomics).
+#include "common.hpp"
+#include "kernels.hpp"
+#include "workspace.hpp"
+#include <math.h>
+
+namespace bm {
+namespace {
+
+// ------------------------------------------------------------------ sparse
+// 16 lanes per column (or per plan segment): strided partial sums, DPP butterfly inside the row.
+template <bool PERM>
+__global__ __launch_bounds__(BM_BLOCK) void k_spsum_ranges(int nranges, const float* __restrict__ vals,
+                                                           const int* __restrict__ perm,
+                                                           const int* __restrict__ ptr,
+                                                           float* __restrict__ out, int beta) {
+    const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long c = t >> 4;
+    const int l = (int)(t & 15);
+    float acc = 0.f;
+    if (c < nranges) {
+        const int s = ptr[c], e = ptr[c + 1];
+        for (int j = s + l; j < e; j += 16) acc += PERM ? vals[perm[j]] : vals[j];
+    }
+    acc = group_allsum<16>(acc);
+    if (c < nranges && l == 0) out[c] = beta ? out[c] + acc : acc;
+}
+
+// ------------------------------------------------------------------ dense
+template <int OP> __device__ __forceinline__ float op2(float a, float b);
+template <> __device__ __forceinline__ float op2<0>(float a, float b) { return a + b; }
+template <> __device__ __forceinline__ float op2<2>(float a, float b) { return a * b; }
+template <> __device__ __forceinline__ float op2<10>(float a, float b) { return fmaxf(a, b); }
+template <> __device__ __forceinline__ float op2<11>(float a, float b) { return fminf(a, b); }
+template <int OP> __device__ __forceinline__ float op_identity();
+template <> __device__ __forceinline__ float op_identity<0>() { return 0.f; }
+template <> __device__ __forceinline__ float op_identity<2>() { return 1.f; }
+template <> __device__ __forceinline__ float op_identity<10>() { return -INFINITY; }
+template <> __device__ __forceinline__ float op_identity<11>() { return INFINITY; }
+
+// Column reduce. lpc lanes (power of two <= 64) per column; rows [r0, r1) of chunk blockIdx.y.
+// out[chunk*ncols + c].
+template <int OP>
+__global__ __launch_bounds__(BM_BLOCK) void k_reduce_cols(int nrows, int ncols, int lpc, int rows_per_chunk,
+                                                          const float* __restrict__ A,
+                                                          float* __restrict__ out) {
+    const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long c = t / lpc;
+    const int l = (int)(t % lpc);
+    const long long r0 = (long long)blockIdx.y * rows_per_chunk;
+    long long r1 = r0 + rows_per_chunk;
+    if (r1 > nrows) r1 = nrows;
+    float acc = op_identity<OP>();
+    if (c < ncols) {
+        const float* col = A + (size_t)c * nrows;
+        for (long long r = r0 + l; r < r1; r += lpc) acc = op2<OP>(acc, col[r]);
+    }
+    for (int d = 1; d < lpc; d <<= 1) acc = op2<OP>(acc, __shfl_xor(acc, d, 64));
+    if (c < ncols && l == 0) out[(size_t)blockIdx.y * ncols + c] = acc;
+}
+
+// Row reduce, stage 1. Block = rb rows x cl column lanes (rb*cl == 256); blockIdx.y = row tile,
+// blockIdx.x = column chunk. out[chunk*nrows + r].
+template <int OP>
+__global__ __launch_bounds__(BM_BLOCK) void k_reduce_rows(int nrows, int ncols, int rb, int cols_per_chunk,
+                                                          const float* __restrict__ A,
+                                                          float* __restrict__ out) {
+    __shared__ float sm[BM_BLOCK];
+    const int cl = BM_BLOCK / rb;
+    const int tr = threadIdx.x % rb;
+    const int tc = threadIdx.x / rb;
+    const long long r = (long long)blockIdx.y * rb + tr;
+    const long long c0 = (long long)blockIdx.x * cols_per_chunk;
+    long long c1 = c0 + cols_per_chunk;
+    if (c1 > ncols) c1 = ncols;
+    float acc = op_identity<OP>();
+    if (r < nrows) {
+        for (long long c = c0 + tc; c < c1; c += cl) acc = op2<OP>(acc, A[(size_t)c * nrows + r]);
+    }
+    sm[threadIdx.x] = acc;
+    __syncthreads();
+    if (tc == 0 && r < nrows) {
+        for (int q = 1; q < cl; ++q) acc = op2<OP>(acc, sm[q * rb + tr]);
+        out[(size_t)blockIdx.x * nrows + r] = acc;
+    }
+}
+
+// Stage 2 of both reductions: out[i] = op over chunks of part[chunk*n + i], in chunk order.
+template <int OP>
+__global__ __launch_bounds__(BM_BLOCK) void k_reduce_chunks(int n, int nchunks, const float* __restrict__ part,
+                                                            float* __restrict__ out) {
+    const long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    if (i >= n) return;
+    float acc = part[i];
+    for (int q = 1; q < nchunks; ++q) acc = op2<OP>(acc, part[(size_t)q * n + i]);
+    out[i] = acc;
+}
+
+template <int OP>
+hipError_t reduce1_impl(int nrows, int ncols, const float* A, float* B, hipStream_t s) {
+    int lpc = pow2ceil(nrows) < 64 ? pow2ceil(nrows) : 64;
+    // few, very long columns: cut the rows into chunks so the whole chip works
+    int nchunks = 1;
+    if ((long long)ncols * lpc < 64 * 2048 && nrows > 8192) {
+        long long want = (64LL * 4096) / ((long long)ncols * lpc);
+        long long maxc = (nrows + 4095) / 4096;
+        nchunks = (int)(want < maxc ? want : maxc);
+        if (nchunks < 1) nchunks = 1;
+        if (nchunks > 4096) nchunks = 4096;
+    }
+    int rows_per_chunk = (nrows + nchunks - 1) / nchunks;
+    nchunks = (nrows + rows_per_chunk - 1) / rows_per_chunk;
+    long long threads = (long long)ncols * lpc;
+    long long nblk = (threads + BM_BLOCK - 1) / BM_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    float* dst = B;
+    if (nchunks > 1) {
+        hipError_t err;
+        dst = (float*)ws_get(WS_REDUCE, sizeof(float) * (size_t)nchunks * ncols, &err);
+        if (!dst) return err;
+    }
+    hipLaunchKernelGGL(k_reduce_cols<OP>, dim3((unsigned)nblk, (unsigned)nchunks), dim3(BM_BLOCK), 0, s,
+                       nrows, ncols, lpc, rows_per_chunk, A, dst);
+    if (nchunks > 1) {
+        unsigned nb2 = (unsigned)(((long long)ncols + BM_BLOCK - 1) / BM_BLOCK);
+        hipLaunchKernelGGL(k_reduce_chunks<OP>, dim3(nb2), dim3(BM_BLOCK), 0, s, ncols, nchunks, dst, B);
+    }
+    return hipGetLastError();
+}
+
+template <int OP>
+hipError_t reduce2_impl(int nrows, int ncols, const float* A, float* B, hipStream_t s) {
+    int rb = pow2ceil(nrows) < BM_BLOCK ? pow2ceil(nrows) : BM_BLOCK;
+    int cl = BM_BLOCK / rb;
+    long long rowtiles = ((long long)nrows + rb - 1) / rb;
+    // enough column chunks to fill the chip, at least 8 columns per lane
+    long long nchunks = 4096 / rowtiles;
+    long long maxc = ((long long)ncols + (long long)cl * 8 - 1) / ((long long)cl * 8);
+    if (nchunks > maxc) nchunks = maxc;
+    if (nchunks < 1) nchunks = 1;
+    int cols_per_chunk = (int)(((long long)ncols + nchunks - 1) / nchunks);
+    nchunks = ((long long)ncols + cols_per_chunk - 1) / cols_per_chunk;
+    if (rowtiles > 65535) return hipErrorInvalidValue;
+    float* dst = B;
+    if (nchunks > 1) {
+        hipError_t err;
+        dst = (float*)ws_get(WS_REDUCE, sizeof(float) * (size_t)nchunks * nrows, &err);
+        if (!dst) return err;
+    }
+    hipLaunchKernelGGL(k_reduce_rows<OP>, dim3((unsigned)nchunks, (unsigned)rowtiles), dim3(BM_BLOCK), 0, s,
+                       nrows, ncols, rb, cols_per_chunk, A, dst);
+    if (nchunks > 1) {
+        unsigned nb2 = (unsigned)(((long long)nrows + BM_BLOCK - 1) / BM_BLOCK);
+        hipLaunchKernelGGL(k_reduce_chunks<OP>, dim3(nb2), dim3(BM_BLOCK), 0, s, nrows, (int)nchunks, dst, B);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, float* out, int beta, hipStream_t s) {
+    (void)nnz;
+    if (ncols <= 0) return hipSuccess;
+    long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_spsum_ranges<false>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, vals, nullptr, jc, out, beta);
+    return hipGetLastError();
+}
+
+hipError_t spsum_segments(int nseg, const float* vals, const int* perm, const int* segstart,
+                          float* partial, hipStream_t s) {
+    if (nseg <= 0) return hipSuccess;
+    long long nblk = ((long long)nseg * 16 + BM_BLOCK - 1) / BM_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_spsum_ranges<true>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, nseg, vals, perm, segstart, partial, 0);
+    return hipGetLastError();
+}
+
+hipError_t reduce1op(int nrows, int ncols, const float* A, float* B, float initv, int opn, hipStream_t s) {
+    if (ncols <= 0) return hipSuccess;
+    if (nrows <= 0) return fill_f32(B, ncols, initv, s);
+    switch (opn) {
+    case 0: return reduce1_impl<0>(nrows, ncols, A, B, s);
+    case 2: return reduce1_impl<2>(nrows, ncols, A, B, s);
+    case 10: return reduce1_impl<10>(nrows, ncols, A, B, s);
+    case 11: return reduce1_impl<11>(nrows, ncols, A, B, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t reduce2op(int nrows, int ncols, const float* A, float* B, float initv, int opn, hipStream_t s) {
+    if (nrows <= 0) return hipSuccess;
+    if (ncols <= 0) return fill_f32(B, nrows, initv, s);
+    switch (opn) {
+    case 0: return reduce2_impl<0>(nrows, ncols, A, B, s);
+    case 2: return reduce2_impl<2>(nrows, ncols, A, B, s);
+    case 10: return reduce2_impl<10>(nrows, ncols, A, B, s);
+    case 11: return reduce2_impl<11>(nrows, ncols, A, B, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace bm

@@ -1,0 +1,188 @@
+/*
+ * bidmat_hip.h — C ABI of libbidmathip.so, the MI355X (gfx950) native library behind
+ * BIDMat's GMat / GSMat sparse-dense product path.
+ *
+ * Conventions (all entry points):
+ *   - plain C types only; every pointer named d_* / documented "device" is a HIP device
+ *     pointer on the calling thread's current device; nothing is retained after return
+ *     except by plan objects, which say so.
+ *   - dense matrices are column-major fp32 with leading dimension == number of rows
+ *     (GMat.scala:19); sparse matrices are CSC with 0-based int32 indices on the device
+ *     (GSMat.scala:14-15,626-632): ir[nnz] row index, ic[nnz] per-nonzero column index
+ *     (non-decreasing), jc[ncols+1] column pointer, data[nnz] values.  Rows inside a
+ *     column need not be sorted or unique.
+ *   - return value: 0 on success, otherwise a hipError_t value as int
+ *     (1 == hipErrorInvalidValue for rejected arguments).  The reference's launchers
+ *     return cudaGetLastError() the same way (Arith.cu:57-59).
+ *   - entry points WITHOUT a stream argument block until the result is complete, like the
+ *     reference's launchers (cudaStreamSynchronize, MatKernel.hpp:15).  Entry points WITH
+ *     a `stream` argument (a hipStream_t passed as void*, NULL = default stream) only
+ *     enqueue work.
+ *   - results are deterministic: no floating-point atomics anywhere.
+ */
+#ifndef BIDMAT_HIP_H
+#define BIDMAT_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Binary op codes, BinOp in GMat.scala:2245-2261 (device table Operators.cu:86-101). */
+enum {
+    BIDMAT_OP_ADD = 0, BIDMAT_OP_SUB = 1, BIDMAT_OP_MUL = 2, BIDMAT_OP_DIV = 3,
+    BIDMAT_OP_GT = 4, BIDMAT_OP_LT = 5, BIDMAT_OP_EQ = 6, BIDMAT_OP_GE = 7,
+    BIDMAT_OP_LE = 8, BIDMAT_OP_NE = 9, BIDMAT_OP_MAX = 10, BIDMAT_OP_MIN = 11,
+    BIDMAT_OP_ATAN2 = 12, BIDMAT_OP_POW = 13, BIDMAT_OP_IFPOS = 14
+};
+
+/* ------------------------------------------------------------------------------------
+ * 1. Reference-shaped launchers: same argument lists as the reference's native
+ *    launchers, so a JNI wrapper can forward to them unchanged.
+ * ------------------------------------------------------------------------------------ */
+
+/* C += A * S.  Replaces `int dsmult(int nrows,int ncols,int nnz,float*A,float*Bdata,int*Bir,
+ * int*Bic,float*C)` (jni/include/MatKernel.hpp, jni/src/Arith.cu:46-60; Java stub
+ * CUMAT.java:143; caller GMat.scala:1070).  nrows = rows of A and C (k); ncols = columns of
+ * S and C.  C holds the addend (callers clear it first, GMat.scala:1047). */
+int bidmat_dsmult(int nrows, int ncols, int nnz, const float *A, const float *Bdata,
+                  const int *Bir, const int *Bic, float *C);
+
+/* C += A * S^T.  Replaces `int dsmultT(...)` (Arith.cu:234-248; CUMAT.java:152; caller
+ * GMat.scala:1093).  nrows = rows of A and C (k); ncols = columns of S and of A.  C has
+ * one column per row of S; the row count of S is not an argument of the reference launcher,
+ * so rows of C beyond max(Bir) are left untouched, exactly as there. */
+int bidmat_dsmultT(int nrows, int ncols, int nnz, const float *A, const float *Bdata,
+                   const int *Bir, const int *Bic, float *C);
+
+/* P[j] += dot(A[:,Cir[j]], B[:,Cic[j]]).  Replaces `int dds(int nrows,int nnz,float*A,float*B,
+ * int*Cir,int*Cic,float*P)` (Arith.cu:381-389; CUMAT.java:211; caller GSMat.scala:663). */
+int bidmat_dds(int nrows, int nnz, const float *A, const float *B, const int *Cir,
+               const int *Cic, float *P);
+
+/* Sparse sums: n == 1: B[Aic[i]] += P[i] (column sums, B has ncols entries); otherwise
+ * B[Air[i]] += P[i] (row sums, B has nrows entries).  Replaces `int spsum(...)`
+ * (Arith.cu:266-277; CUMAT.java:209; caller GSMat.scala:255). */
+int bidmat_spsum(int nrows, int ncols, int nnz, const int *Air, const int *Aic, const float *P,
+                 float *B, int n);
+
+/* Dense column reduce B[c] = op_r A[r,c] (B has ncols entries).  Replaces
+ * `int reduce1op(int nrows,int ncols,float*A,float*B,float initv,int opn)`
+ * (Operators.cu:735-748; CUMAT.java:111; caller GMat.scala:1186).  Supported opn:
+ * ADD, MUL, MAX, MIN (the ones BIDMat's sum/prod/maxi/mini issue, GFunctions.scala:225-228);
+ * any other code returns hipErrorInvalidValue. */
+int bidmat_reduce1op(int nrows, int ncols, const float *A, float *B, float initv, int opn);
+
+/* Dense row reduce B[r] = op_c A[r,c] (B has nrows entries).  Replaces `int reduce2op(...)`
+ * (Operators.cu:853-866; CUMAT.java:119; caller GMat.scala:1193). Same op set. */
+int bidmat_reduce2op(int nrows, int ncols, const float *A, float *B, float initv, int opn);
+
+/* Elementwise C = op(A, B) with BIDMat's broadcasting (equal shapes, row/column vector on
+ * either side, scalar on either side).  Replaces `int apply_binop(float*A,int Anrows,int Ancols,
+ * float*B,int Bnrows,int Bncols,float*C,int opn)` (Operators.cu:529-553; CUMAT.java:31 applyop;
+ * caller GMat.scala:1125).  All 15 op codes. */
+int bidmat_applyop(const float *A, int Anrows, int Ancols, const float *B, int Bnrows,
+                   int Bncols, float *C, int opn);
+
+/* ------------------------------------------------------------------------------------
+ * 2. Native entry points: take the column pointer jc (GSMat.pjc, which the reference
+ *    keeps on the device but never passes to its kernels), an overwrite/accumulate flag
+ *    and a stream.  beta == 0: the output is overwritten (no clear needed);
+ *    beta == 1: the output holds the addend.  They only enqueue work on `stream`.
+ * ------------------------------------------------------------------------------------ */
+
+/* C = beta*C + A*S.   A k x nrowsS, S nrowsS x ncols (CSC), C k x ncols. */
+int bidmat_dsmult_csc(int k, int ncols, int nnz, const float *A, const float *Sdata,
+                      const int *Sir, const int *Sjc, float *C, int beta, void *stream);
+
+/* P = beta*P + DDS(A,B,pattern).  A k x nrowsS, B k x ncols, P one value per nonzero. */
+int bidmat_dds_csc(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir,
+                   const int *Sjc, float *P, int beta, void *stream);
+
+/* Row-binned execution plan of one sparsity pattern, needed by A*^S and by sparse row sums.
+ * The plan keeps its own device copies of what it needs; the pattern arrays may be freed
+ * afterwards.  The values array is NOT captured: pass the current values to each call.
+ * k_hint: the dense leading dimension the plan will mostly be used with (sizes the column
+ * panels so that one panel of A stays in an XCD's L2); 0 = 256.
+ * Blocking (device synchronisation inside).  Returns 0 and a handle in *plan. */
+typedef struct bidmat_plan bidmat_plan;
+int bidmat_plan_create(int nrows, int ncols, int nnz, const int *Sir, const int *Sjc, int k_hint,
+                       bidmat_plan **plan);
+int bidmat_plan_destroy(bidmat_plan *plan);
+/* Device bytes held by the plan (index arrays + partial-sum workspace). */
+long long bidmat_plan_bytes(const bidmat_plan *plan);
+/* Number of row segments of the plan (each yields one k-vector partial sum). */
+int bidmat_plan_segments(const bidmat_plan *plan);
+
+/* C = beta*C + A*S^T through a plan.  A k x ncols, C k x nrows(S).  Sdata: the nnz values
+ * in the original CSC order.  With beta == 0 every column of C is written (zeros for empty
+ * rows of S). */
+int bidmat_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *Sdata, float *C,
+                        int beta, void *stream);
+
+/* Sparse sums with jc / a plan: out = beta*out + sums.  Column sums need only jc;
+ * row sums need a plan. */
+int bidmat_spsum_cols(int ncols, int nnz, const float *Sdata, const int *Sjc, float *out,
+                      int beta, void *stream);
+int bidmat_spsum_rows_plan(bidmat_plan *plan, const float *Sdata, float *out, int beta,
+                           void *stream);
+
+/* jc[ncols+1] -> ic[nnz] (per-nonzero column index).  Replaces cusparseXcsr2coo at
+ * GSMat.scala:639.  Enqueues on stream. */
+int bidmat_csc_expand_cols(int ncols, int nnz, const int *Sjc, int *Sic, void *stream);
+/* non-decreasing ic[nnz] -> jc[ncols+1].  Replaces cusparseXcoo2csr at GSMat.scala:698,716
+ * and SparseMat.compressInds (SparseMat.scala:857-868). Enqueues on stream. */
+int bidmat_coo_compress_cols(int ncols, int nnz, const int *Sic, int *Sjc, void *stream);
+
+/* Elementwise on flat arrays with a stream (the V./R step on GSMat.contents). */
+int bidmat_applyop_flat(const float *A, const float *B, float *C, long long n, int opn,
+                        void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * 3. Device memory and runtime helpers (what the reference does through JCuda:
+ *    cublasAlloc/cublasFree GSMat.scala:519-522,225-232; cudaMemcpy GSMat.scala:625-633;
+ *    cudaMemset GMat.scala:562-566; cudaMemGetInfo GFunctions.scala:208-213).
+ * ------------------------------------------------------------------------------------ */
+int bidmat_device_count(int *count);
+int bidmat_set_device(int dev);
+int bidmat_get_device(int *dev);
+int bidmat_malloc(void **dptr, long long bytes);
+int bidmat_free(void *dptr);
+int bidmat_memcpy_h2d(void *dst, const void *src, long long bytes);
+int bidmat_memcpy_d2h(void *dst, const void *src, long long bytes);
+int bidmat_memcpy_d2d(void *dst, const void *src, long long bytes);
+int bidmat_memset(void *dptr, int value, long long bytes);
+int bidmat_mem_info(long long *free_bytes, long long *total_bytes);
+int bidmat_synchronize(void);
+/* Pinned host staging buffers (allocated, never registered). */
+int bidmat_host_alloc(void **hptr, long long bytes);
+int bidmat_host_free(void *hptr);
+/* Streams and events for callers that time or overlap work (benchmark harness). */
+int bidmat_stream_create(void **stream);
+int bidmat_stream_destroy(void *stream);
+int bidmat_stream_synchronize(void *stream);
+int bidmat_event_create(void **event);
+int bidmat_event_destroy(void *event);
+int bidmat_event_record(void *event, void *stream);
+int bidmat_event_synchronize(void *event);
+int bidmat_event_elapsed_ms(void *start, void *stop, float *ms);
+/* Text for a return code (cudaGetErrorString in the reference's exceptions, GMat.scala:1071). */
+const char *bidmat_error_string(int err);
+/* Library / device description: "bidmathip <version> gfx950 ..." */
+const char *bidmat_version(void);
+/* Name of the compiled-for architecture of the current device ("gfx950"), CU count. */
+int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *total_mem);
+
+/* Tunables (process-wide, read at call time):
+ *   "seglen"   nonzeros per wavefront segment when a long column / row is split (default 1024)
+ *   "panel_kb" target size in KiB of one column panel of A in a plan (default 2048)
+ * Returns 0, or hipErrorInvalidValue for an unknown name / bad value. */
+int bidmat_set_option(const char *name, long long value);
+long long bidmat_get_option(const char *name);
+
+/* Drops every cached plan and workspace buffer of the current device. */
+int bidmat_release_caches(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BIDMAT_HIP_H */
