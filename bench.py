@@ -43,7 +43,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows/columns of the pattern (testing)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-sample", type=float, default=0.05, help="fraction of columns timed on the CPU")
+    ap.add_argument("--cpu-sample", type=float, default=1.0, help="fraction of the columns timed on the CPU (1.0 = the whole workload)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a plain streaming kernel of known size (C = A + B on 3 x 1 GiB) "
+                         "before the steps: the scale for rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards by "
@@ -109,6 +112,17 @@ def main():
         hip_abi.check(lib.bidmat_dsmultT_plan(plan, k, d_AT.ptr, d_v.ptr, d_G.ptr, 0, stream), "dsmultT")
         if marks:
             hip_abi.check(lib.bidmat_event_record(marks[3], stream))
+
+    if args.calibrate:
+        ncal = 1 << 28                                   # 2^28 floats = 1 GiB per array
+        cal = [DeviceArray(ncal, np.float32) for _ in range(3)]
+        for c in cal:
+            hip_abi.check(lib.bidmat_memset(c.ptr, 0, c.nbytes))
+        for _ in range(3):                               # k_apply_full4: reads 2 GiB, writes 1 GiB
+            hip_abi.check(lib.bidmat_applyop_flat(cal[0].ptr, cal[1].ptr, cal[2].ptr, ncal, 0, stream))
+        hip_abi.check(lib.bidmat_stream_synchronize(stream))
+        for c in cal:
+            c.free()
 
     for _ in range(args.warmup):
         step()

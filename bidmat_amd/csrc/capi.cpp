@@ -18,8 +18,10 @@
 namespace bm {
 namespace {
 std::atomic<int> g_seglen{1024};
-std::atomic<int> g_panel_kb{2048};
+std::atomic<int> g_panel_kb{3072};
+std::atomic<int> g_heavy_min{8};
 }  // namespace
+int opt_heavy_min() { return g_heavy_min.load(std::memory_order_relaxed); }
 int opt_seglen() { return g_seglen.load(std::memory_order_relaxed); }
 int opt_panel_kb() { return g_panel_kb.load(std::memory_order_relaxed); }
 }  // namespace bm
@@ -96,7 +98,7 @@ hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* va
                        hipStream_t s) {
     hipError_t err;
     if ((err = bm::plan_reserve_partial(plan, k)) != hipSuccess) return err;
-    if ((err = bm::gather_segments(k, plan->nseg, A, vals, plan->pc, plan->perm, plan->segstart,
+    if ((err = bm::gather_segments(k, plan->nseg, plan->xcd_start, A, vals, plan->pc, plan->perm, plan->segstart,
                                    plan->partial, s)) != hipSuccess) return err;
     return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, C, beta, s);
 }
@@ -403,6 +405,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_panel_kb.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "heavy_min")) {
+        if (value < 1 || value > (1 << 20)) return kInvalid;
+        bm::g_heavy_min.store((int)value);
+        return 0;
+    }
     return kInvalid;
 }
 
@@ -410,6 +417,7 @@ API long long bidmat_get_option(const char* name) {
     if (!name) return -1;
     if (!strcmp(name, "seglen")) return bm::opt_seglen();
     if (!strcmp(name, "panel_kb")) return bm::opt_panel_kb();
+    if (!strcmp(name, "heavy_min")) return bm::opt_heavy_min();
     return -1;
 }
 

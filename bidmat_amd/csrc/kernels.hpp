@@ -8,6 +8,7 @@ namespace bm {
 // ---- tunables (capi.cpp owns the storage)
 int opt_seglen();      // nonzeros per wave segment for long columns / rows
 int opt_panel_kb();    // KiB of A per column panel in a plan
+int opt_heavy_min();   // a row is cut by panels when it averages at least this many nonzeros per panel
 
 // ---- CSC utilities (csc_util.hip)
 hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);
@@ -36,8 +37,10 @@ hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, co
 
 // ---- plan stage kernels (spmm.hip): segment s gathers columns pc[p] of A scaled by
 // vals[perm[p]] for p in [segstart[s], segstart[s+1]) into partial[s*k ..].
-hipError_t gather_segments(int k, int nseg, const float* A, const float* vals, const int* pc,
-                           const int* perm, const int* segstart, float* partial, hipStream_t s);
+// xcd_start[9]: segment groups per XCD (see plan.hpp); workgroup b is assumed to run on XCD b % 8.
+hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A, const float* vals,
+                           const int* pc, const int* perm, const int* segstart, float* partial,
+                           hipStream_t s);
 // C[:,r] = beta*C[:,r] + sum over q in [rowptr[r], rowptr[r+1]) of partial[rowseg[q]*k ..]
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
                            const float* partial, float* C, int beta, hipStream_t s);

@@ -19,7 +19,6 @@ struct DevBuf {
     template <typename T> T* as() { return static_cast<T*>(p); }
 };
 
-constexpr int MIN_NNZ_PER_PANEL_SEGMENT = 32;   // a heavy row averages at least this per panel
 
 __global__ __launch_bounds__(BM_BLOCK) void k_row_hist(int nnz, int nrows, const int* __restrict__ ir,
                                                        int* __restrict__ cnt, int* __restrict__ bad) {
@@ -49,15 +48,18 @@ __global__ __launch_bounds__(BM_BLOCK) void k_heavy_rows(int nrows, const int* _
 __global__ __launch_bounds__(BM_BLOCK) void k_make_keys(int ncols, int nrows, const int* __restrict__ jc,
                                                         const int* __restrict__ ir, const int* __restrict__ flag,
                                                         const int* __restrict__ hrank, int nheavy, int npanels,
-                                                        int panel_cols, unsigned* __restrict__ keys,
+                                                        int panel_cols, int p8, unsigned* __restrict__ keys,
                                                         int* __restrict__ pos) {
     const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long c = t >> 4;
     const int l = (int)(t & 15);
     if (c >= ncols) return;
     const int s = jc[c], e = jc[c + 1];
-    const unsigned panel = (unsigned)(c / panel_cols);
-    const unsigned light_base = (unsigned)npanels * (unsigned)nheavy;
+    // panels are ordered by the XCD that will own them: panel p -> slot (p % 8) * p8 + p / 8
+    const unsigned praw = (unsigned)(c / panel_cols);
+    const unsigned panel = (praw & 7u) * (unsigned)p8 + (praw >> 3);
+    const unsigned light_base = 8u * (unsigned)p8 * (unsigned)nheavy;
+    (void)npanels;
     for (int j = s + l; j < e; j += 16) {
         int r = ir[j];
         r = r < 0 ? 0 : (r >= nrows ? nrows - 1 : r);
@@ -78,12 +80,14 @@ __global__ __launch_bounds__(BM_BLOCK) void k_boundaries(int nnz, int seglen, co
 __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __restrict__ keys,
                                                    const int* __restrict__ perm, const int* __restrict__ ic,
                                                    const int* __restrict__ flag, const int* __restrict__ segidx,
-                                                   const int* __restrict__ hrow, int nheavy, int npanels,
+                                                   const int* __restrict__ hrow, int nheavy, int p8,
                                                    int* __restrict__ pc, int* __restrict__ segstart,
-                                                   unsigned* __restrict__ segrow, int* __restrict__ segid) {
+                                                   unsigned* __restrict__ segrow, int* __restrict__ segid,
+                                                   int* __restrict__ class_count) {
     long long p = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long stride = (long long)gridDim.x * BM_BLOCK;
-    const unsigned light_base = (unsigned)npanels * (unsigned)nheavy;
+    const unsigned per_xcd = (unsigned)p8 * (unsigned)nheavy;     // keys per XCD group
+    const unsigned light_base = 8u * per_xcd;
     for (; p < nnz; p += stride) {
         pc[p] = ic[perm[p]];
         if (flag[p]) {
@@ -92,6 +96,8 @@ __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __re
             segstart[sidx] = (int)p;
             segrow[sidx] = key >= light_base ? key - light_base : (unsigned)hrow[key % (unsigned)nheavy];
             segid[sidx] = sidx;
+            // segments per XCD group (integer atomics: the counts do not depend on the order)
+            atomicAdd(&class_count[key >= light_base ? 8 : (int)(key / per_xcd)], 1);
         }
     }
 }
@@ -156,6 +162,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     if (pcols > ncols) pcols = ncols > 0 ? ncols : 1;
     plan->panel_cols = (int)pcols;
     plan->npanels = ncols > 0 ? (int)(((long long)ncols + pcols - 1) / pcols) : 1;
+    const int p8 = (plan->npanels + 7) / 8;          // panels per XCD group
 
     PB_CHECK(hipMalloc((void**)&plan->rowptr, sizeof(int) * ((size_t)nrows + 1)));
     plan->index_bytes += sizeof(int) * ((size_t)nrows + 1);
@@ -186,13 +193,13 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     // 2. heavy rows and their ranks
     int nheavy = 0;
     if (plan->npanels >= 2) {
-        long long thresh = (long long)plan->npanels * MIN_NNZ_PER_PANEL_SEGMENT;
+        long long thresh = (long long)plan->npanels * opt_heavy_min();
         if (thresh > 0x7fffffffLL) thresh = 0x7fffffffLL;
         hipLaunchKernelGGL(k_heavy_flag, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, cnt.as<int>(), (int)thresh, hflag.as<int>());
         PB_CHECK(scan_exclusive_i32(hflag.as<int>(), hrank.as<int>(), nrows, scantmp.as<int>(), s));
         PB_CHECK(hipMemcpy(&nheavy, hrank.as<int>() + nrows, sizeof(int), hipMemcpyDeviceToHost));
         // keys must fit 32 bits
-        if ((unsigned long long)plan->npanels * (unsigned long long)nheavy + (unsigned long long)nrows > 0xffffffffULL) nheavy = 0;
+        if (8ULL * (unsigned long long)p8 * (unsigned long long)nheavy + (unsigned long long)nrows > 0xffffffffULL) nheavy = 0;
     }
     if (nheavy == 0) {
         PB_CHECK(fill_i32(hflag.as<int>(), nrows, 0, s));
@@ -212,10 +219,10 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     {
         long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
         hipLaunchKernelGGL(k_make_keys, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nrows, jc, ir,
-                           hflag.as<int>(), hrank.as<int>(), nheavy, plan->npanels, plan->panel_cols,
+                           hflag.as<int>(), hrank.as<int>(), nheavy, plan->npanels, plan->panel_cols, p8,
                            keys_in.as<unsigned>(), pos_in.as<int>());
     }
-    const unsigned long long maxkey = (unsigned long long)plan->npanels * nheavy + (unsigned long long)nrows;
+    const unsigned long long maxkey = 8ULL * (unsigned long long)p8 * nheavy + (unsigned long long)nrows;
     const int end_bit = bits_for(maxkey);
     {
         size_t tmp_bytes = 0;
@@ -239,7 +246,9 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     PB_CHECK(hipMemcpy(&nseg, segidx.as<int>() + nnz, sizeof(int), hipMemcpyDeviceToHost));
     plan->nseg = nseg;
 
-    DevBuf segrow, segid, segrow_sorted;
+    DevBuf segrow, segid, segrow_sorted, class_count;
+    PB_CHECK(class_count.alloc(sizeof(int) * 9));
+    PB_CHECK(fill_i32(class_count.as<int>(), 9, 0, s));
     PB_CHECK(segrow.alloc(sizeof(unsigned) * (size_t)nseg));
     PB_CHECK(segid.alloc(sizeof(int) * (size_t)nseg));
     PB_CHECK(segrow_sorted.alloc(sizeof(unsigned) * (size_t)nseg));
@@ -248,8 +257,15 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     plan->index_bytes += sizeof(int) * (2 * (size_t)nseg + 1);
     hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out.as<unsigned>(), plan->perm,
                        ic.as<int>(), flag.as<int>(), segidx.as<int>(), hrow.as<int>(), nheavy > 0 ? nheavy : 1,
-                       nheavy > 0 ? plan->npanels : 0, plan->pc, plan->segstart, segrow.as<unsigned>(), segid.as<int>());
+                       nheavy > 0 ? p8 : 0, plan->pc, plan->segstart, segrow.as<unsigned>(), segid.as<int>(),
+                       class_count.as<int>());
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
+    {
+        int h_count[9];
+        PB_CHECK(hipMemcpy(h_count, class_count.p, sizeof(h_count), hipMemcpyDeviceToHost));
+        plan->xcd_start[0] = 0;
+        for (int x = 0; x < 8; ++x) plan->xcd_start[x + 1] = plan->xcd_start[x] + h_count[x];
+    }
 
     // 5. a row's segments, in ascending segment order (stable sort by row)
     {

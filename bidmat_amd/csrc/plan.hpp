@@ -19,6 +19,10 @@ struct bidmat_plan {
     int npanels = 0;
     int panel_cols = 0;
     int seglen = 0;
+    // Segments are stored heavy first, grouped by the XCD that is to process them: group x
+    // (panels x, x+8, x+16, ... in ascending order) is [xcd_start[x], xcd_start[x+1]); the
+    // light-row segments follow from xcd_start[8] and are dealt round-robin to the XCDs.
+    int xcd_start[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
     int* pc = nullptr;       // [nnz]    column of the p-th nonzero in plan order
     int* perm = nullptr;     // [nnz]    its position in the original CSC order
     int* segstart = nullptr; // [nseg+1] segment boundaries in plan order

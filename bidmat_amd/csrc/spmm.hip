@@ -15,6 +15,7 @@
 #include "kernels.hpp"
 #include "scan.hpp"
 #include "workspace.hpp"
+#include <algorithm>
 
 namespace bm {
 namespace {
@@ -32,6 +33,7 @@ struct GatherArgs {
     const int* ovf;      // CSC mode: overflow table (nullable)
     float* out;          // C (CSC mode) / partial (plan mode)
     float* partial;      // CSC mode: partial sums of overflow segments
+    int xcd_start[9];    // plan mode: segment groups per XCD, light segments from xcd_start[8]
 };
 
 template <int V, int LPN>
@@ -115,10 +117,21 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
     float* outp;
     bool accumulate;
     if (PLAN) {
-        if (w >= a.nfirst) return;
-        jstart = a.ptr[w];
-        jend = a.ptr[w + 1];
-        outp = a.out + (size_t)w * (size_t)a.k;
+        // Workgroups are dealt to the 8 XCDs round-robin, so workgroup b runs on XCD b % 8.
+        // Each XCD first walks its own group of heavy segments (whole column panels, one after
+        // the other, so that the panel of A it is gathering stays in its L2), then its share of
+        // the light segments (every 8th one). Interleaving the two kinds, with or without
+        // non-temporal loads for the light gathers, was measured slower: the light gathers miss
+        // L2 and evict the panel the heavy segments are reusing.
+        const int xcd = blockIdx.x & 7;
+        const long long wi = (long long)(blockIdx.x >> 3) * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+        const int hstart = a.xcd_start[xcd];
+        const int hcount = a.xcd_start[xcd + 1] - hstart;
+        const long long seg = wi < hcount ? hstart + wi : a.xcd_start[8] + (wi - hcount) * 8 + xcd;
+        if (seg >= a.nfirst) return;
+        jstart = a.ptr[seg];
+        jend = a.ptr[seg + 1];
+        outp = a.out + (size_t)seg * (size_t)a.k;
         accumulate = false;
     } else if (w < a.nfirst) {
         const int s = a.ptr[w], e = a.ptr[w + 1];
@@ -290,6 +303,7 @@ hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* va
     a.k = k; a.nfirst = ncols; a.seglen = seglen; a.beta = beta;
     a.A = A; a.vals = vals; a.idx = ir; a.perm = nullptr; a.ptr = jc; a.ovf = ovf;
     a.out = C; a.partial = partial;
+    for (int x = 0; x < 9; ++x) a.xcd_start[x] = 0;
     err = launch_gather<false>(sh, a, (long long)ncols + novf_max, s);
     if (err != hipSuccess) return err;
     if (ovf) {
@@ -300,15 +314,23 @@ hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* va
     return err;
 }
 
-hipError_t gather_segments(int k, int nseg, const float* A, const float* vals, const int* pc,
-                           const int* perm, const int* segstart, float* partial, hipStream_t s) {
+hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A, const float* vals,
+                           const int* pc, const int* perm, const int* segstart, float* partial,
+                           hipStream_t s) {
     if (k <= 0 || nseg <= 0) return hipSuccess;
     Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(partial)));
     GatherArgs a;
     a.k = k; a.nfirst = nseg; a.seglen = 0; a.beta = 0;
     a.A = A; a.vals = vals; a.idx = pc; a.perm = perm; a.ptr = segstart; a.ovf = nullptr;
     a.out = partial; a.partial = nullptr;
-    return launch_gather<true>(sh, a, nseg, s);
+    int maxheavy = 0;
+    for (int x = 0; x < 9; ++x) a.xcd_start[x] = xcd_start[x];
+    for (int x = 0; x < 8; ++x) maxheavy = std::max(maxheavy, xcd_start[x + 1] - xcd_start[x]);
+    const long long nlight = (long long)nseg - xcd_start[8];
+    // waves per XCD, rounded up to whole workgroups, times 8 XCDs
+    const long long per_xcd = (long long)maxheavy + (nlight + 7) / 8;
+    const long long blocks_per_xcd = (per_xcd + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
+    return launch_gather<true>(sh, a, blocks_per_xcd * 8 * BM_WAVES_PER_BLOCK, s);
 }
 
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,

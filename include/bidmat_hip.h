@@ -174,7 +174,9 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
 
 /* Tunables (process-wide, read at call time):
  *   "seglen"   nonzeros per wavefront segment when a long column / row is split (default 1024)
- *   "panel_kb" target size in KiB of one column panel of A in a plan (default 2048)
+ *   "panel_kb" target size in KiB of one column panel of A in a plan (default 3072)
+ *   "heavy_min" a row is cut by column panels when it averages at least this many nonzeros
+ *              per panel (default 8)
  * Returns 0, or hipErrorInvalidValue for an unknown name / bad value. */
 int bidmat_set_option(const char *name, long long value);
 long long bidmat_get_option(const char *name);
