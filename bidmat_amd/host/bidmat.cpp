@@ -1,0 +1,428 @@
+#include "bidmat.hpp"
+#include "../../include/bidmat_hip.h"
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <mutex>
+
+namespace BIDMat {
+
+// ------------------------------------------------------------------ globals
+int Mat::ioneBased = 1;
+bool Mat::useGPUcache = false;
+double Mat::recycleGrow = 1.2;
+bool Mat::debugMem = false;
+int Mat::numThreads = 8;
+std::atomic<long long> Mat::nflops{0};
+
+namespace {
+std::atomic<long long> g_guid{1000};
+std::mutex g_cache_mu;
+using Key = std::tuple<long long, long long, long long, long long, int>;
+std::map<Key, GMatP> g_gcache;
+std::map<Key, GSMatP> g_scache;
+
+std::string fmt(const char* f, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, f);
+    vsnprintf(buf, sizeof buf, f, ap);
+    va_end(ap);
+    return buf;
+}
+
+[[noreturn]] void fail(const std::string& msg) { throw std::runtime_error(msg); }
+
+void hipcheck(int err, const char* what) {
+    if (err != 0) fail(std::string(what) + " " + bidmat_error_string(err));
+}
+
+long long opHash(const char* name) { return (long long)std::hash<std::string>()(name); }
+
+void checkThread(int myGPU, const char* where, long long guid) {
+    int cur = getGPU();
+    if (myGPU != cur) fail(fmt("%s wrong thread %d %d for mat %lld", where, myGPU, cur, guid));
+}
+}  // namespace
+
+long long Mat::newGUID() { return g_guid.fetch_add(1); }
+
+void Mat::clearCaches() {
+    std::lock_guard<std::mutex> lock(g_cache_mu);
+    g_gcache.clear();
+    g_scache.clear();
+}
+
+int getGPU() {
+    int d = 0;
+    hipcheck(bidmat_get_device(&d), "getGPU");
+    return d;
+}
+void setGPU(int dev) { hipcheck(bidmat_set_device(dev), "setGPU"); }
+std::pair<float, long long> GPUmem() {
+    long long f = 0, t = 0;
+    hipcheck(bidmat_mem_info(&f, &t), "GPUmem");
+    return {t ? (float)((double)f / (double)t) : 0.f, f};
+}
+
+// ------------------------------------------------------------------ timers
+namespace {
+std::chrono::steady_clock::time_point g_tic = std::chrono::steady_clock::now();
+long long g_lastFlops = 0;
+float toc() { return std::chrono::duration<float>(std::chrono::steady_clock::now() - g_tic).count(); }
+}  // namespace
+void flip() { g_lastFlops = Mat::nflops.load(); g_tic = std::chrono::steady_clock::now(); }
+std::pair<float, float> flop() { float t = toc(); return {(float)(Mat::nflops.load() - g_lastFlops) / t, t}; }
+std::pair<float, float> gflop() { float t = toc(); return {(float)(Mat::nflops.load() - g_lastFlops) / t / 1e9f, t}; }
+
+// ------------------------------------------------------------------ FMat / SMat
+FMat::FMat(int nr, int nc) : nrows(nr), ncols(nc), data((size_t)nr * nc, 0.f), GUID(Mat::newGUID()) {}
+FMat::FMat(int nr, int nc, const float* src) : nrows(nr), ncols(nc), data(src, src + (size_t)nr * nc), GUID(Mat::newGUID()) {}
+
+SMat::SMat(int nr, int nc, int nnz) : nrows(nr), ncols(nc), ir((size_t)nnz), jc((size_t)nc + 1, Mat::ioneBased),
+                                      data((size_t)nnz), GUID(Mat::newGUID()) {}
+
+void SMat::check() const {
+    const int ioff = Mat::ioneBased;
+    if (jc[0] != ioff) fail(fmt("jc(0) should be %d", ioff));
+    for (int i = 0; i < ncols; ++i) {
+        int j = jc[i] - ioff;
+        if (jc[i] > jc[i + 1]) fail(fmt("jc(i) out of order %d %d %d", i, jc[i], jc[i + 1]));
+        while (j < jc[i + 1] - ioff - 1 && j + 1 < nnz()) {    // never read past the arrays
+            if (ir[j + 1] <= ir[j]) fail(fmt("ir(j) out of order %d %d %d", j, ir[j], ir[j + 1]));
+            if (ir[j] < ioff) fail(fmt("ir(%d)=%d too small", j, ir[j]));
+            if (ir[j + 1] >= nrows + ioff) fail(fmt("ir(%d)=%d out of range %d", j + 1, ir[j + 1], nrows + ioff));
+            ++j;
+        }
+    }
+    if (jc[ncols] != nnz() + ioff) fail(fmt("jc(ncols) should be %d", nnz()));
+}
+
+FMat SMat::full() const {
+    FMat out(nrows, ncols);
+    const int ioff = Mat::ioneBased;
+    for (int i = 0; i < ncols; ++i)
+        for (int j = jc[i] - ioff; j < jc[i + 1] - ioff; ++j)
+            out.data[(size_t)(ir[j] - ioff) + (size_t)i * nrows] += data[j];
+    return out;
+}
+
+// ------------------------------------------------------------------ GMat
+GMat::GMat(int nr, int nc, float* p, long long rs, bool o)
+    : nrows(nr), ncols(nc), pdata(p), realsize(rs), GUID(Mat::newGUID()), myGPU(getGPU()), owns(o) {}
+
+GMat::~GMat() { free(); }
+
+void GMat::free() {
+    if (owns && pdata) bidmat_free(pdata);
+    pdata = nullptr;
+}
+
+GMatP GMat::make(int nr, int nc) {
+    long long n = (long long)nr * nc;
+    if (Mat::debugMem) fprintf(stderr, "GMat %d %d, %d %f\n", nr, nc, getGPU(), GPUmem().first);
+    void* p = nullptr;
+    hipcheck(bidmat_malloc(&p, n * (long long)sizeof(float)), "GPU alloc failed");
+    return std::make_shared<GMat>(nr, nc, (float*)p, n, true);
+}
+
+GMatP GMat::zeros(int nr, int nc) {
+    GMatP m = make(nr, nc);
+    m->clear();
+    return m;
+}
+
+GMat& GMat::clear() {
+    hipcheck(bidmat_memset(pdata, 0, (long long)sizeof(float) * length()), "GMat.clear");
+    return *this;
+}
+
+GMatP GMat::fromFMat(const FMat& a, GMatP out) {
+    GMatP m = newOrCheckGMat(a.nrows, a.ncols, out);
+    hipcheck(bidmat_memcpy_h2d(m->pdata, a.data.data(), (long long)sizeof(float) * a.length()), "GMat() copy");
+    return m;
+}
+
+FMat GMat::toFMat() const {
+    FMat out(nrows, ncols);
+    hipcheck(bidmat_memcpy_d2h(out.data.data(), pdata, (long long)sizeof(float) * length()), "toFMat copy");
+    return out;
+}
+
+GMatP GMat::newOrCheckGMat(int nr, int nc, GMatP outmat) {
+    if (!outmat || (outmat->nrows == 0 && outmat->ncols == 0)) return make(nr, nc);
+    if (outmat->nrows != nr || outmat->ncols != nc) {
+        // recycle: reuse the buffer when it is large enough (GMat.scala:1315-1331)
+        if (outmat->realsize >= (long long)nr * nc) {
+            auto m = std::make_shared<GMat>(nr, nc, outmat->pdata, outmat->realsize, false);
+            m->keepalive = outmat;
+            return m;
+        }
+        return make(nr, nc);
+    }
+    return outmat;
+}
+
+GMatP GMat::newOrCheckGMat(int nr, int nc, GMatP outmat, long long g1, long long g2, long long oph) {
+    GMatP m;
+    if (outmat || !Mat::useGPUcache) {
+        m = newOrCheckGMat(nr, nc, outmat);
+    } else {
+        Key key(g1, g2, 0, oph, getGPU());
+        std::lock_guard<std::mutex> lock(g_cache_mu);
+        auto it = g_gcache.find(key);
+        GMatP res = it == g_gcache.end() ? nullptr : it->second;
+        m = newOrCheckGMat(nr, nc, res);
+        if (m != res) g_gcache[key] = m;
+    }
+    checkThread(m->myGPU, "newOrCheckGMat", m->GUID);
+    return m;
+}
+
+GMatP GMat::GSMult(const GSMatP& a, GMatP oldmat) {
+    if (ncols != a->nrows) fail(fmt("GSMult dimensions mismatch (%d %d) (%d %d)", nrows, ncols, a->nrows, a->ncols));
+    GMatP out = newOrCheckGMat(nrows, a->ncols, oldmat, GUID, a->GUID, opHash("GSMult"));
+    // the reference clears `out` and accumulates (GMat.scala:1047-1048); beta = 0 overwrites instead
+    Mat::nflops += 2LL * nrows * a->nnz();
+    int err = bidmat_dsmult_csc(nrows, a->ncols, a->nnz(), pdata, a->pdata, a->pir, a->pjc, out->pdata, 0, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("GMult: HIP kernel error in dsmult ") + bidmat_error_string(err));
+    return out;
+}
+
+GMatP GMat::madd(const GSMatP& a, GMatP out) {
+    if (ncols != a->nrows || nrows != out->nrows || a->ncols != out->ncols)
+        fail(fmt("GSMadd dimensions mismatch (%d %d) (%d %d) (%d %d)", nrows, ncols, a->nrows, a->ncols, out->nrows, out->ncols));
+    Mat::nflops += 2LL * nrows * a->nnz();
+    int err = bidmat_dsmult_csc(nrows, a->ncols, a->nnz(), pdata, a->pdata, a->pir, a->pjc, out->pdata, 1, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("GMult: HIP kernel error in dsmult ") + bidmat_error_string(err));
+    return out;
+}
+
+GMatP GMat::GSMultT(const GSMatP& a, GMatP oldmat) {
+    if (ncols != a->ncols) fail(fmt("GSMult dimensions mismatch (%d %d) (%d %d)", nrows, ncols, a->ncols, a->nrows));
+    GMatP out = newOrCheckGMat(nrows, a->nrows, oldmat, GUID, a->GUID, opHash("GSMultT"));
+    Mat::nflops += 2LL * nrows * a->nnz();
+    int err = bidmat_dsmultT_plan(a->plan(nrows), nrows, pdata, a->pdata, out->pdata, 0, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("GMult: HIP kernel error in dsmultT ") + bidmat_error_string(err));
+    return out;
+}
+
+GMatP GMat::maddT(const GSMatP& a, GMatP out) {
+    if (ncols != a->ncols || nrows != out->nrows || a->nrows != out->ncols)
+        fail(fmt("GSMadd dimensions mismatch (%d %d) (%d %d) (%d %d)", nrows, ncols, a->ncols, a->nrows, out->nrows, out->ncols));
+    Mat::nflops += 2LL * nrows * a->nnz();
+    int err = bidmat_dsmultT_plan(a->plan(nrows), nrows, pdata, a->pdata, out->pdata, 1, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("GMult: HIP kernel error in dsmultT ") + bidmat_error_string(err));
+    return out;
+}
+
+GMatP GMat::gOp(const GMatP& a, GMatP oldmat, int op) {
+    // compatible shapes (ND.compatibleGDims for the 2-D case): equal, or a row/column/scalar on either side
+    const int nr = std::max(nrows, a->nrows), nc = std::max(ncols, a->ncols);
+    const bool ok = (nrows == a->nrows || nrows == 1 || a->nrows == 1) && (ncols == a->ncols || ncols == 1 || a->ncols == 1) &&
+                    ((nrows == a->nrows && ncols == a->ncols) || (a->nrows == 1 && a->ncols == 1) || (nrows == 1 && ncols == 1) ||
+                     (nrows == a->nrows && (a->ncols == 1 || ncols == 1)) || (ncols == a->ncols && (a->nrows == 1 || nrows == 1)));
+    if (!ok) fail(fmt("DenseMat Op: dimensions mismatch (%d %d) (%d %d)", nrows, ncols, a->nrows, a->ncols));
+    GMatP out = newOrCheckGMat(nr, nc, oldmat, GUID, a->GUID, op);
+    Mat::nflops += std::max(length(), a->length());
+    int err = bidmat_applyop(pdata, nrows, ncols, a->pdata, a->nrows, a->ncols, out->pdata, op);
+    if (err != 0) fail(fmt("HIP kernel error %d in applyop", err));
+    return out;
+}
+
+GMatP GMat::reduceOp(GMatP oldmat, int dir, float initval, int op) {
+    if (dir == 1 || (dir == 0 && nrows > 1)) {
+        GMatP out = newOrCheckGMat(1, ncols, oldmat, GUID, 1, op);
+        int err = bidmat_reduce1op(nrows, ncols, pdata, out->pdata, initval, op);
+        if (err != 0) fail(std::string("HIP kernel error in reduce1op ") + bidmat_error_string(err));
+        Mat::nflops += length();
+        return out;
+    } else if (dir == 2 || dir == 0) {
+        GMatP out = newOrCheckGMat(nrows, 1, oldmat, GUID, 2, op);
+        int err = bidmat_reduce2op(nrows, ncols, pdata, out->pdata, initval, op);
+        if (err != 0) fail(std::string("HIP kernel error in reduce2op ") + bidmat_error_string(err));
+        Mat::nflops += length();
+        return out;
+    }
+    fail("dimension must be 1 or 2");
+}
+
+// ------------------------------------------------------------------ GSMat
+PlanHolder::~PlanHolder() {
+    if (plan) bidmat_plan_destroy(plan);
+}
+
+GSMat::GSMat(int nr, int nc, int nnz, int rn)
+    : nrows(nr), ncols(nc), nnz0(nnz), pir(nullptr), pic(nullptr), pjc(nullptr), pdata(nullptr),
+      realnnz(std::max(1, rn)), GUID(Mat::newGUID()), myGPU(getGPU()), planHolder(std::make_shared<PlanHolder>()) {
+    if (Mat::debugMem) fprintf(stderr, "GSMat %d %d %d, %d %f\n", nr, nc, nnz, getGPU(), GPUmem().first);
+    void* p = nullptr;
+    int err = bidmat_malloc(&p, (long long)sizeof(int) * realnnz); pir = (int*)p;
+    if (err == 0) { err = bidmat_malloc(&p, (long long)sizeof(int) * realnnz); pic = (int*)p; }
+    if (err == 0) { err = bidmat_malloc(&p, (long long)sizeof(int) * ((long long)ncols + 1)); pjc = (int*)p; }
+    if (err == 0) { err = bidmat_malloc(&p, (long long)sizeof(float) * realnnz); pdata = (float*)p; }
+    if (err != 0) { free(); fail(std::string("HIP error in GSMat() ") + bidmat_error_string(err)); }
+}
+
+GSMat::~GSMat() { free(); }
+
+void GSMat::free() {
+    if (pdata) bidmat_free(pdata);
+    if (pic) bidmat_free(pic);
+    if (pir) bidmat_free(pir);
+    if (pjc) bidmat_free(pjc);
+    pdata = nullptr; pic = pir = pjc = nullptr;
+}
+
+GSMatP GSMat::make(int nr, int nc, int nnz, int realnnz) { return std::make_shared<GSMat>(nr, nc, nnz, realnnz); }
+
+GSMat& GSMat::clear() {
+    hipcheck(bidmat_memset(pdata, 0, (long long)sizeof(float) * nnz0), "GSMat.clear");
+    return *this;
+}
+
+GSMatP GSMat::newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP oldmat) {
+    if (!oldmat || (oldmat->nrows == 0 && oldmat->ncols == 0)) {
+        if (Mat::useGPUcache) return make(nr, nc, nnz, std::max((int)(Mat::recycleGrow * nnz), realnnz));
+        return make(nr, nc, nnz, realnnz);
+    }
+    if (oldmat->nrows == nr && oldmat->ncols == nc && nnz <= oldmat->realnnz) {
+        oldmat->nnz0 = nnz;
+        return oldmat;
+    }
+    // recycle (GSMat.scala:234-248): the column pointer depends on ncols, so a new shape gets new buffers
+    GSMatP m = Mat::useGPUcache ? make(nr, nc, nnz, (int)(Mat::recycleGrow * nnz)) : make(nr, nc, nnz, nnz);
+    if (oldmat->nrows == nr && oldmat->ncols == nc) m->GUID = oldmat->GUID;
+    return m;
+}
+
+GSMatP GSMat::newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP outmat, long long g1, long long g2,
+                              long long g3, long long oph) {
+    GSMatP m;
+    if (outmat || !Mat::useGPUcache) {
+        m = newOrCheckGSMat(nr, nc, nnz, realnnz, outmat);
+    } else {
+        Key key(g1, g2, g3, oph, getGPU());
+        std::lock_guard<std::mutex> lock(g_cache_mu);
+        auto it = g_scache.find(key);
+        GSMatP res = it == g_scache.end() ? nullptr : it->second;
+        m = newOrCheckGSMat(nr, nc, nnz, realnnz, res);
+        if (m != res) g_scache[key] = m;
+    }
+    checkThread(m->myGPU, "newOrCheckGSMat3", m->GUID);
+    return m;
+}
+
+GSMatP GSMat::fromSMat(const SMat& a, GSMatP b) {
+    GSMatP out = newOrCheckGSMat(a.nrows, a.ncols, a.nnz(), a.nnz(), b, a.GUID, 0, 0, opHash("fromSMat"));
+    out->nnz0 = a.nnz();
+    out->planHolder = std::make_shared<PlanHolder>();      // new pattern: any older plan is stale
+    const int n = a.nnz();
+    hipcheck(bidmat_memcpy_h2d(out->pdata, a.data.data(), (long long)sizeof(float) * n), "copy error in GSMat.fromSMat");
+    if (Mat::ioneBased == 1) {   // device indices are always 0-based (GSMat.scala:626-632)
+        std::vector<int> ir0(a.ir), jc0(a.jc);
+        for (auto& v : ir0) v -= 1;
+        for (auto& v : jc0) v -= 1;
+        hipcheck(bidmat_memcpy_h2d(out->pir, ir0.data(), (long long)sizeof(int) * n), "copy error in GSMat.fromSMat");
+        hipcheck(bidmat_memcpy_h2d(out->pjc, jc0.data(), (long long)sizeof(int) * (a.ncols + 1)), "copy error in GSMat.fromSMat");
+    } else {
+        hipcheck(bidmat_memcpy_h2d(out->pir, a.ir.data(), (long long)sizeof(int) * n), "copy error in GSMat.fromSMat");
+        hipcheck(bidmat_memcpy_h2d(out->pjc, a.jc.data(), (long long)sizeof(int) * (a.ncols + 1)), "copy error in GSMat.fromSMat");
+    }
+    // per-nonzero column indices (the reference calls cusparseXcsr2coo here, GSMat.scala:639)
+    int err = bidmat_csc_expand_cols(out->ncols, n, out->pjc, out->pic, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("HIP error in GSMat.fromSMat ") + bidmat_error_string(err));
+    return out;
+}
+
+SMat GSMat::toSMat() const {
+    SMat out(nrows, ncols, nnz0);
+    std::vector<int> tmpcols((size_t)nnz0);
+    hipcheck(bidmat_memcpy_d2h(out.ir.data(), pir, (long long)sizeof(int) * nnz0), "HIP error in GSMat.toSMat");
+    hipcheck(bidmat_memcpy_d2h(out.data.data(), pdata, (long long)sizeof(float) * nnz0), "HIP error in GSMat.toSMat");
+    hipcheck(bidmat_memcpy_d2h(tmpcols.data(), pic, (long long)sizeof(int) * nnz0), "HIP error in GSMat.toSMat");
+    // SparseMat.compressInds (SparseMat.scala:857-868)
+    const int ioff = Mat::ioneBased;
+    out.jc[0] = ioff;
+    int j = 0;
+    for (int i = 0; i < ncols; ++i) {
+        while (j < nnz0 && tmpcols[j] <= i) ++j;
+        out.jc[i + 1] = j + ioff;
+    }
+    if (ioff == 1) for (auto& v : out.ir) v += 1;
+    return out;
+}
+
+GMatP GSMat::contents() {
+    auto out = std::make_shared<GMat>(nnz0, 1, pdata, realnnz, false);
+    return out;
+}
+
+bidmat_plan* GSMat::plan(int k_hint) {
+    if (!planHolder->plan) {
+        int err = bidmat_plan_create(nrows, ncols, nnz0, pir, pjc, k_hint, &planHolder->plan);
+        if (err != 0) fail(std::string("HIP error building the row plan ") + bidmat_error_string(err));
+        planHolder->k_hint = k_hint;
+    }
+    return planHolder->plan;
+}
+
+GMatP GSMat::sum(int n, GMatP oldmat) {
+    const int nn = n > 0 ? n : (nrows == 1 ? 2 : 1);
+    GMatP out = GMat::newOrCheckGMat(nn == 1 ? 1 : nrows, nn == 1 ? ncols : 1, oldmat, GUID, n, opHash("sum"));
+    Mat::nflops += nnz0;
+    int err;
+    if (nn == 1) err = bidmat_spsum_cols(ncols, nnz0, pdata, pjc, out->pdata, 0, nullptr);
+    else if (nn == 2) err = bidmat_spsum_rows_plan(plan(0), pdata, out->pdata, 0, nullptr);
+    else fail("index must 1 or 2");
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("HIP error in GSMat.sum ") + bidmat_error_string(err));
+    return out;
+}
+
+GSMatP GSMat::DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat) {
+    if (A->nrows != B->nrows || C->nrows != A->ncols || C->ncols != B->ncols)
+        fail(fmt("dimensions mismatch %d,%d  %d,%d  %d,%d", A->nrows, A->ncols, B->nrows, B->ncols, C->nrows, C->ncols));
+    GSMatP out = newOrCheckGSMat(C->nrows, C->ncols, C->nnz(), C->realnnz, oldmat, A->GUID, B->GUID, C->GUID, opHash("DDS"));
+    if (out != C) {
+        // the result carries C's pattern: row indices, column indices AND the column pointer
+        // (the reference copies pir and pic only and leaves out.pjc stale, GSMat.scala:656-661)
+        hipcheck(bidmat_memcpy_d2d(out->pir, C->pir, (long long)sizeof(int) * C->nnz()), "DDS row copy error");
+        hipcheck(bidmat_memcpy_d2d(out->pic, C->pic, (long long)sizeof(int) * C->nnz()), "DDS column copy error");
+        hipcheck(bidmat_memcpy_d2d(out->pjc, C->pjc, (long long)sizeof(int) * ((long long)C->ncols + 1)), "DDS column pointer copy error");
+        out->planHolder = C->planHolder;       // same pattern, same plan
+    }
+    int err = bidmat_dds_csc(A->nrows, C->ncols, C->nnz(), A->pdata, B->pdata, C->pir, C->pjc, out->pdata, 0, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(fmt("GPU %d DDS kernel error %s", getGPU(), bidmat_error_string(err)));
+    Mat::nflops += 2LL * C->nnz() * A->nrows;
+    return out;
+}
+
+GSMatP GSMat::withValues(const GMatP& vals) const {
+    if (vals->length() != nnz0) fail(fmt("withValues: %lld values for %d nonzeros", vals->length(), nnz0));
+    GSMatP out = make(nrows, ncols, nnz0, realnnz);
+    hipcheck(bidmat_memcpy_d2d(out->pir, pir, (long long)sizeof(int) * nnz0), "pattern copy error");
+    hipcheck(bidmat_memcpy_d2d(out->pic, pic, (long long)sizeof(int) * nnz0), "pattern copy error");
+    hipcheck(bidmat_memcpy_d2d(out->pjc, pjc, (long long)sizeof(int) * ((long long)ncols + 1)), "pattern copy error");
+    hipcheck(bidmat_memcpy_d2d(out->pdata, vals->pdata, (long long)sizeof(float) * nnz0), "value copy error");
+    out->planHolder = planHolder;
+    return out;
+}
+
+// ------------------------------------------------------------------ operators / free functions
+GMatP operator*(const GMatP& a, const GSMatP& s) { return a->GSMult(s, nullptr); }
+GMatP xT(const GMatP& a, const GSMatP& s) { return a->GSMultT(s, nullptr); }
+GMatP operator/(const GMatP& a, const GMatP& b) { return a->gOp(b, nullptr, op_div); }
+GSMatP DDS(const GMatP& a, const GMatP& b, const GSMatP& c, GSMatP omat) { return GSMat::DDS(a, b, c, omat); }
+GMatP sum(const GSMatP& s, int n, GMatP omat) { return s->sum(n, omat); }
+GMatP sum(const GMatP& a, int n, GMatP omat) { return a->reduceOp(omat, n, 0.f, op_add); }
+
+}  // namespace BIDMat

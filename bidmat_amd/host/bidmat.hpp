@@ -1,0 +1,169 @@
+// Host-side mirror of BIDMat's operator interface for the sparse-dense product path
+// (C++ stand-in for the Scala layer: no JVM/Scala toolchain exists on the build or GPU boxes).
+// Same class and method names, argument meaning, flop accounting and exception texts as
+//   GMat   src/main/scala/BIDMat/GMat.scala   (GSMult :1041, madd :1051, GSMultT :1076, maddT :1086,
+//                                              gOp :1119, reduceOp :1182, clear :562, operators :1684-1688)
+//   GSMat  src/main/scala/BIDMat/GSMat.scala  (fromSMat :620, toSMat :108, DDS :649, sum :250,
+//                                              contents :21, free :225, newOrCheckGSMat :722-806)
+//   SMat / FMat host containers, Mat globals (Mat.scala:646-724), flip/flop/gflop
+//   (MatFunctions.scala:19-51), sum dispatch (SFunctions.scala:10-15, GFunctions.scala:227).
+// Everything device-side goes through the C ABI of libbidmathip.so (include/bidmat_hip.h);
+// this layer never touches HIP directly.
+#pragma once
+#include <atomic>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <vector>
+
+struct bidmat_plan;
+
+namespace BIDMat {
+
+// ---- global flags and counters (object Mat, Mat.scala:670-724)
+struct Mat {
+    static int ioneBased;          // index base of host sparse matrices (1 like the reference)
+    static bool useGPUcache;       // cache operator outputs under (operand GUIDs, op, GPU)
+    static double recycleGrow;     // growth factor for recycled buffers
+    static bool debugMem;          // print every device allocation
+    static int numThreads;
+    static std::atomic<long long> nflops;
+    static long long newGUID();
+    static void clearCaches();
+};
+
+enum BinOp { op_add = 0, op_sub, op_mul, op_div, op_gt, op_lt, op_eq, op_ge, op_le, op_ne,
+             op_max, op_min, op_atan2, op_pow, op_ifpos };
+
+// ---- host dense, column-major (FMat)
+class FMat {
+public:
+    int nrows = 0, ncols = 0;
+    std::vector<float> data;
+    long long GUID;
+    FMat(int nr, int nc);
+    FMat(int nr, int nc, const float* src);
+    long long length() const { return (long long)nrows * ncols; }
+    std::string mytype() const { return "FMat"; }
+};
+
+// ---- host sparse CSC (SMat); ir / jc carry Mat::ioneBased
+class SMat {
+public:
+    int nrows = 0, ncols = 0;
+    std::vector<int> ir, jc;
+    std::vector<float> data;
+    long long GUID;
+    SMat(int nr, int nc, int nnz);
+    int nnz() const { return (int)data.size(); }
+    // SparseMat.check (SparseMat.scala:710-740): throws with the reference's messages
+    void check() const;
+    FMat full() const;
+    std::string mytype() const { return "SMat"; }
+};
+
+class GSMat;
+class GMat;
+using GMatP = std::shared_ptr<GMat>;
+using GSMatP = std::shared_ptr<GSMat>;
+
+// ---- device dense (GMat)
+class GMat {
+public:
+    int nrows, ncols;
+    float* pdata;              // device, column-major, leading dimension nrows
+    long long realsize;        // capacity in floats
+    long long GUID;
+    int myGPU;
+    bool owns;
+    std::shared_ptr<void> keepalive;   // a view (GSMat.contents) keeps its parent's buffer alive
+
+    GMat(int nr, int nc, float* p, long long realsize, bool owns);
+    ~GMat();
+    static GMatP make(int nr, int nc);                       // GMat(nr, nc)  (GMat.scala:2338-2353)
+    static GMatP zeros(int nr, int nc);
+    static GMatP fromFMat(const FMat& a, GMatP out = nullptr);
+    FMat toFMat() const;
+    long long length() const { return (long long)nrows * ncols; }
+    std::string mytype() const { return "GMat"; }
+    GMat& clear();                                           // GMat.scala:562-566
+    void free();
+
+    // C = this * S and C += this * S
+    GMatP GSMult(const GSMatP& a, GMatP oldmat);
+    GMatP madd(const GSMatP& a, GMatP out);
+    // C = this *^ S and C += this *^ S
+    GMatP GSMultT(const GSMatP& a, GMatP oldmat);
+    GMatP maddT(const GSMatP& a, GMatP out);
+    // elementwise binary op with broadcasting, reductions
+    GMatP gOp(const GMatP& a, GMatP oldmat, int op);
+    GMatP reduceOp(GMatP oldmat, int dir, float initval, int op);
+
+    static GMatP newOrCheckGMat(int nr, int nc, GMatP outmat);
+    static GMatP newOrCheckGMat(int nr, int nc, GMatP outmat, long long g1, long long g2, long long opHash);
+};
+
+// shared by all GSMats that carry the same pattern buffers' content (a DDS result, V./R ...)
+struct PlanHolder {
+    bidmat_plan* plan = nullptr;
+    int k_hint = 0;
+    ~PlanHolder();
+};
+
+// ---- device sparse (GSMat): pir/pic/pjc/pdata, all 0-based on the device
+class GSMat {
+public:
+    int nrows, ncols;
+    int nnz0;
+    int* pir;
+    int* pic;
+    int* pjc;
+    float* pdata;
+    int realnnz;
+    long long GUID;
+    int myGPU;
+    std::shared_ptr<PlanHolder> planHolder;
+
+    GSMat(int nr, int nc, int nnz, int realnnz);
+    ~GSMat();
+    int nnz() const { return nnz0; }
+    std::string mytype() const { return "GSMat"; }
+    static GSMatP make(int nr, int nc, int nnz, int realnnz);
+    static GSMatP fromSMat(const SMat& a, GSMatP b = nullptr);   // GSMat.scala:620-647
+    SMat toSMat() const;                                         // GSMat.scala:108-127
+    GMatP contents();                                            // GSMat.scala:21-25
+    GSMat& clear();
+    void free();
+    GMatP sum(int n, GMatP oldmat);                              // GSMat.scala:250-261
+    static GSMatP DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat);   // GSMat.scala:649-667
+    // a sparse matrix with this pattern and other values (the V./R step keeps V's pattern)
+    GSMatP withValues(const GMatP& vals) const;
+    bidmat_plan* plan(int k_hint);
+
+    static GSMatP newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP oldmat);
+    static GSMatP newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP outmat, long long g1,
+                                  long long g2, long long g3, long long opHash);
+};
+
+// ---- operators (GMat.scala:1684-1688, 1972-1976) and free functions
+GMatP operator*(const GMatP& a, const GSMatP& s);                 // a * s
+GMatP xT(const GMatP& a, const GSMatP& s);                        // a *^ s  (alias xT in the reference)
+GMatP operator/(const GMatP& a, const GMatP& b);                  // elementwise
+GSMatP DDS(const GMatP& a, const GMatP& b, const GSMatP& c, GSMatP omat = nullptr);
+GMatP sum(const GSMatP& s, int n = 0, GMatP omat = nullptr);      // SFunctions.scala:10-15
+GMatP sum(const GMatP& a, int n = 0, GMatP omat = nullptr);       // GFunctions.scala:227
+// host reference path: FMat * SMat, FMat *^ SMat, DDS on host are NOT provided here (the CPU
+// restatement of those loops lives with the tests); these mirror only the GPU dispatch.
+
+// timers (MatFunctions.scala:19-51)
+void flip();
+std::pair<float, float> flop();
+std::pair<float, float> gflop();
+
+int getGPU();
+void setGPU(int dev);
+std::pair<float, long long> GPUmem();     // (free fraction, free bytes)  GFunctions.scala:208-213
+
+}  // namespace BIDMat

@@ -1,0 +1,243 @@
+"""Python face of the host-side mirror (libbidmathost.so): GMat / GSMat objects with BIDMat's
+operator names, for scripts and tests. All arithmetic happens in the HIP library; this module
+only moves handles around.
+
+    a * s            GMat * GSMat            (GMat.scala:1684)
+    a.xT(s)          a *^ s                  (GMat.scala:1686, alias xT :1688)
+    DDS(a, b, s)     a ^* (b @@ s)           (MatFunctions.scala:1656-1674)
+    sum(s, n), sum(a, n)                     (SFunctions.scala:10-15, GFunctions.scala:227)
+    a / b            elementwise             (GMat.scala:1681)
+    c.madd / c.maddT via out=...             (the `c ~ a * b` output-reuse form)
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import hip_abi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libbidmathost.so")
+_lib = None
+vp = C.c_void_p
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        hip_abi.load()          # raises if the HIP library is missing; RTLD_GLOBAL for the host layer
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("libbidmathost.so is not built; run `make -C bidmat_amd/host`")
+        L = C.CDLL(LIB_PATH)
+        for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
+                     "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
+                     "bmh_gop", "bmh_contents", "bmh_with_values"):
+            getattr(L, name).restype = vp
+        L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
+        L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
+        L.bmh_gsmat_from_host.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp, vp]
+        for name in ("bmh_mult", "bmh_madd", "bmh_multT", "bmh_maddT"):
+            getattr(L, name).argtypes = [vp, vp, vp]
+        L.bmh_dds.argtypes = [vp, vp, vp, vp]
+        L.bmh_sum_sparse.argtypes = [vp, C.c_int, vp]
+        L.bmh_sum_dense.argtypes = [vp, C.c_int, vp]
+        L.bmh_reduce.argtypes = [vp, vp, C.c_int, C.c_float, C.c_int]
+        L.bmh_gop.argtypes = [vp, vp, vp, C.c_int]
+        L.bmh_contents.argtypes = [vp]
+        L.bmh_with_values.argtypes = [vp, vp]
+        L.bmh_release.argtypes = [vp]
+        L.bmh_release.restype = None
+        L.bmh_last_error.restype = C.c_char_p
+        L.bmh_type.restype = C.c_char_p
+        L.bmh_type.argtypes = [vp]
+        L.bmh_guid.restype = C.c_longlong
+        L.bmh_guid.argtypes = [vp]
+        L.bmh_same_object.argtypes = [vp, vp]
+        L.bmh_gmat_dims.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.bmh_gmat_to_host.argtypes = [vp, vp]
+        L.bmh_gsmat_dims.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.bmh_gsmat_to_host.argtypes = [vp, vp, vp, vp]
+        L.bmh_gsmat_device_jc.argtypes = [vp, vp]
+        L.bmh_nflops.restype = C.c_longlong
+        L.bmh_gflop.restype = C.c_double
+        L.bmh_gflop.argtypes = [C.POINTER(C.c_float)]
+        L.bmh_set_flag.argtypes = [C.c_char_p, C.c_double]
+        L.bmh_get_flag.argtypes = [C.c_char_p]
+        L.bmh_get_flag.restype = C.c_double
+        L.bmh_smat_check.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp]
+        _lib = L
+    return _lib
+
+
+def _ok(h):
+    if not h:
+        raise RuntimeError(_load().bmh_last_error().decode())
+    return h
+
+
+class Mat:
+    """Global flags (object Mat in the reference)."""
+
+    @staticmethod
+    def set(name, value):
+        if _load().bmh_set_flag(name.encode(), float(value)) != 0:
+            raise KeyError(name)
+
+    @staticmethod
+    def get(name):
+        return _load().bmh_get_flag(name.encode())
+
+    @staticmethod
+    def nflops():
+        return _load().bmh_nflops()
+
+    @staticmethod
+    def clear_caches():
+        _load().bmh_clear_caches()
+
+
+def flip():
+    _load().bmh_flip()
+
+
+def gflop():
+    secs = C.c_float(0)
+    g = _load().bmh_gflop(C.byref(secs))
+    return g, secs.value
+
+
+class _Handle:
+    def __init__(self, h):
+        self._h = _ok(h)
+
+    def __del__(self):
+        try:
+            if self._h:
+                _load().bmh_release(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    @property
+    def mytype(self):
+        return _load().bmh_type(self._h).decode()
+
+    @property
+    def GUID(self):
+        return _load().bmh_guid(self._h)
+
+    def same(self, other):
+        return bool(_load().bmh_same_object(self._h, other._h))
+
+
+class GMat(_Handle):
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.asfortranarray(a, dtype=np.float32)
+        if a.ndim == 1:
+            a = a.reshape(-1, 1, order="F")
+        flat = np.ascontiguousarray(a.ravel(order="F"))
+        return cls(_load().bmh_gmat_from_host(a.shape[0], a.shape[1], flat.ctypes.data))
+
+    @classmethod
+    def zeros(cls, nr, nc):
+        return cls(_load().bmh_gmat_zeros(nr, nc))
+
+    @property
+    def shape(self):
+        nr, nc = C.c_int(), C.c_int()
+        _load().bmh_gmat_dims(self._h, C.byref(nr), C.byref(nc))
+        return nr.value, nc.value
+
+    def numpy(self):
+        nr, nc = self.shape
+        out = np.empty(nr * nc, dtype=np.float32)
+        if _load().bmh_gmat_to_host(self._h, out.ctypes.data) != 0:
+            raise RuntimeError(_load().bmh_last_error().decode())
+        return out.reshape(nc, nr).T
+
+    def __mul__(self, s):                 # a * s
+        return GMat(_load().bmh_mult(self._h, s._h, None))
+
+    def GSMult(self, s, out=None):
+        return GMat(_load().bmh_mult(self._h, s._h, out._h if out else None))
+
+    def madd(self, s, out):
+        return GMat(_load().bmh_madd(self._h, s._h, out._h))
+
+    def xT(self, s):                      # a *^ s
+        return GMat(_load().bmh_multT(self._h, s._h, None))
+
+    def GSMultT(self, s, out=None):
+        return GMat(_load().bmh_multT(self._h, s._h, out._h if out else None))
+
+    def maddT(self, s, out):
+        return GMat(_load().bmh_maddT(self._h, s._h, out._h))
+
+    def gOp(self, b, op, out=None):
+        return GMat(_load().bmh_gop(self._h, b._h, out._h if out else None, op))
+
+    def __truediv__(self, b):
+        return self.gOp(b, 3)
+
+    def reduceOp(self, dir, initv, op, out=None):
+        return GMat(_load().bmh_reduce(self._h, out._h if out else None, dir, initv, op))
+
+
+class GSMat(_Handle):
+    @classmethod
+    def from_csc(cls, nrows, ncols, data, ir, jc):
+        """Host SMat arrays; ir / jc carry the base Mat.get('ioneBased')."""
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        ir = np.ascontiguousarray(ir, dtype=np.int32)
+        jc = np.ascontiguousarray(jc, dtype=np.int32)
+        return cls(_load().bmh_gsmat_from_host(nrows, ncols, data.size, data.ctypes.data, ir.ctypes.data, jc.ctypes.data))
+
+    @property
+    def dims(self):
+        nr, nc, nnz = C.c_int(), C.c_int(), C.c_int()
+        _load().bmh_gsmat_dims(self._h, C.byref(nr), C.byref(nc), C.byref(nnz))
+        return nr.value, nc.value, nnz.value
+
+    def to_csc(self):
+        """Back to host SMat arrays (with SparseMat.check applied): (data, ir, jc)."""
+        nr, nc, nnz = self.dims
+        data = np.empty(nnz, np.float32)
+        ir = np.empty(nnz, np.int32)
+        jc = np.empty(nc + 1, np.int32)
+        if _load().bmh_gsmat_to_host(self._h, data.ctypes.data, ir.ctypes.data, jc.ctypes.data) != 0:
+            raise RuntimeError(_load().bmh_last_error().decode())
+        return data, ir, jc
+
+    def device_jc(self):
+        nr, nc, nnz = self.dims
+        jc = np.empty(nc + 1, np.int32)
+        hip_abi.check(_load().bmh_gsmat_device_jc(self._h, jc.ctypes.data))
+        return jc
+
+    def contents(self):
+        return GMat(_load().bmh_contents(self._h))
+
+    def with_values(self, vals):
+        return GSMat(_load().bmh_with_values(self._h, vals._h))
+
+    def sum(self, n=0, out=None):
+        return GMat(_load().bmh_sum_sparse(self._h, n, out._h if out else None))
+
+
+def DDS(a, b, c, out=None):
+    return GSMat(_load().bmh_dds(a._h, b._h, c._h, out._h if out else None))
+
+
+def sum(a, n=0, out=None):      # noqa: A001  (the reference's name)
+    if isinstance(a, GSMat):
+        return a.sum(n, out)
+    return GMat(_load().bmh_sum_dense(a._h, n, out._h if out else None))
+
+
+def smat_check(nrows, ncols, ir, jc):
+    """SparseMat.check on host arrays; raises RuntimeError with the reference's message."""
+    ir = np.ascontiguousarray(ir, dtype=np.int32)
+    jc = np.ascontiguousarray(jc, dtype=np.int32)
+    if _load().bmh_smat_check(nrows, ncols, ir.size, ir.ctypes.data, jc.ctypes.data) != 0:
+        raise RuntimeError(_load().bmh_last_error().decode())

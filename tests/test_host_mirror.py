@@ -1,0 +1,251 @@
+"""The host-side mirror of BIDMat's GMat / GSMat operator interface, exercised the way the
+reference's own tests do (src/test/scala/BIDMat/GSMatTest.scala, GMatTest.scala): random
+inputs at nr=10, nc=20, nk=30, results compared with a dense computation at eps 1e-4,
+result types checked, SparseMat.check on sparse results. Host arrays are 1-based
+(Mat.ioneBased = 1, the reference's default).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from bidmat_amd import mats
+from bidmat_amd.mats import DDS, GMat, GSMat, Mat
+from util import dense_full, random_csc
+
+nr, nc, nk = 10, 20, 30
+EPS = 1e-4
+
+
+def sprand(rng, m, n, density):
+    """Host SMat arrays with the reference's default 1-based indices."""
+    data, ir, jc = random_csc(rng, m, n, density)
+    return data, ir + 1, jc + 1
+
+
+def full(m, n, data, ir, jc):
+    return dense_full(m, n, data, ir - 1, jc - 1)
+
+
+# ----------------------------------------------------------------------- no GPU needed
+def test_sparse_check_messages():
+    mats.smat_check(4, 3, np.array([1, 3, 2, 4]), np.array([1, 3, 3, 5]))
+    for ir, jc, msg in [
+        ([1, 3, 2, 4], [0, 3, 3, 5], "jc(0) should be 1"),
+        ([1, 2, 3, 4], [1, 4, 3, 5], "jc(i) out of order"),
+        ([3, 1, 2, 4], [1, 3, 3, 5], "ir(j) out of order"),
+        ([1, 9, 2, 4], [1, 3, 3, 5], "out of range"),
+        ([1, 3, 2, 4], [1, 3, 3, 4], "jc(ncols) should be"),
+    ]:
+        with pytest.raises(RuntimeError, match=msg.replace("(", r"\(").replace(")", r"\)")):
+            mats.smat_check(4, 3, np.array(ir), np.array(jc))
+
+
+def test_flags_default_to_the_reference_values():
+    assert Mat.get("ioneBased") == 1 and Mat.get("recycleGrow") == pytest.approx(1.2)
+    assert Mat.get("useGPUcache") == 0
+    with pytest.raises(KeyError):
+        Mat.set("noSuchFlag", 1)
+
+
+# ----------------------------------------------------------------------- GPU
+gpu = pytest.mark.gpu
+
+
+@gpu
+def test_matrix_multiplication(hip):
+    """'A GSMat should support matrix multiplication' (GSMatTest.scala:55-71), GMat * GSMat half."""
+    rng = np.random.default_rng(1)
+    b = rng.random((nk, nc)).astype(np.float32)
+    bt = np.ascontiguousarray(b.T)                                   # nc x nk
+    at = sprand(rng, nk, nr, 0.2)
+    aat, bbt = GSMat.from_csc(nk, nr, *at), GMat.from_numpy(bt)
+    before = Mat.nflops()
+    cct = bbt * aat
+    assert cct.mytype == "GMat" and cct.shape == (nc, nr)
+    assert Mat.nflops() - before == 2 * nc * at[0].size              # Mat.nflops += 2L * nrows * a.nnz
+    dt = bt.astype(np.float64) @ full(nk, nr, *at)
+    np.testing.assert_allclose(cct.numpy(), dt, rtol=0, atol=EPS)
+
+
+@gpu
+def test_matrix_times_transpose(hip):
+    """'support matrix *^' (GSMatTest.scala:74-83)."""
+    rng = np.random.default_rng(2)
+    a = rng.random((nr, nk)).astype(np.float32)
+    b = sprand(rng, nc, nk, 0.2)
+    aa, bb = GMat.from_numpy(a), GSMat.from_csc(nc, nk, *b)
+    cc = aa.xT(bb)
+    assert cc.mytype == "GMat" and cc.shape == (nr, nc)
+    np.testing.assert_allclose(cc.numpy(), a.astype(np.float64) @ full(nc, nk, *b).T, rtol=0, atol=EPS)
+
+
+@gpu
+@pytest.mark.parametrize("axis", [1, 2, 0])
+def test_sparse_sums(hip, axis):
+    """'support 2D column sum' / 'row sum' (GSMatTest.scala:283-316), loops as written there."""
+    rng = np.random.default_rng(3 + axis)
+    data, ir, jc = sprand(rng, nr, nc, 0.2)
+    aa = GSMat.from_csc(nr, nc, data, ir, jc)
+    ax = axis if axis else 1
+    b = np.zeros(nc if ax == 1 else nr, dtype=np.float32)
+    for i in range(nc):
+        j0, j1 = jc[i] - 1, jc[i + 1] - 1
+        if ax == 1:
+            if j1 > j0:
+                b[i] = data[j0]
+            for j in range(j0 + 1, j1):
+                b[i] = b[i] + data[j]
+        else:
+            for j in range(j0, j1):
+                b[ir[j] - 1] = b[ir[j] - 1] + data[j]
+    cc = mats.sum(aa, axis)
+    assert cc.mytype == "GMat" and cc.shape == ((1, nc) if ax == 1 else (nr, 1))
+    np.testing.assert_allclose(cc.numpy().ravel(), b, rtol=0, atol=EPS)
+
+
+@gpu
+@pytest.mark.parametrize("axis", [1, 2])
+def test_dense_sums(hip, axis):
+    """GMat sum (GMatTest.scala:938-979)."""
+    rng = np.random.default_rng(5)
+    a = rng.random((nr, nc)).astype(np.float32)
+    cc = mats.sum(GMat.from_numpy(a), axis)
+    want = a.astype(np.float64).sum(axis=axis - 1)
+    assert cc.shape == ((1, nc) if axis == 1 else (nr, 1))
+    np.testing.assert_allclose(cc.numpy().ravel(), want, rtol=0, atol=EPS)
+
+
+@gpu
+def test_dds_keeps_the_pattern(hip):
+    """DDS has no test in the reference; pinned by its closed form and by the pattern rule:
+    the result's ir / jc equal the input's bit for bit (DDShelper copies them)."""
+    rng = np.random.default_rng(6)
+    a = rng.random((nk, nr)).astype(np.float32)       # k x nrows(S)
+    b = rng.random((nk, nc)).astype(np.float32)       # k x ncols(S)
+    data, ir, jc = sprand(rng, nr, nc, 0.3)
+    cs = GSMat.from_csc(nr, nc, data, ir, jc)
+    before = Mat.nflops()
+    p = DDS(GMat.from_numpy(a), GMat.from_numpy(b), cs)
+    assert p.mytype == "GSMat" and p.dims == (nr, nc, data.size)
+    assert Mat.nflops() - before == 2 * data.size * nk
+    vals, pir, pjc = p.to_csc()                        # runs SparseMat.check as well
+    assert np.array_equal(pir, ir) and np.array_equal(pjc, jc)
+    assert np.array_equal(p.device_jc(), jc - 1)       # the device column pointer travels too
+    cols = np.repeat(np.arange(nc), np.diff(jc))
+    want = np.einsum("kn,kn->n", a.astype(np.float64)[:, ir - 1], b.astype(np.float64)[:, cols])
+    np.testing.assert_allclose(vals, want, rtol=0, atol=EPS)
+    ref, _, _ = oracle.dds(a.ravel(order="F"), b.ravel(order="F"), nk, ir, jc, ioff=1)
+    np.testing.assert_allclose(vals, ref, rtol=1e-5, atol=1e-6)
+
+
+@gpu
+def test_output_reuse_and_accumulate(hip):
+    """`c ~ a * b` reuses c; madd / maddT accumulate into it (GMat.scala:1051-1096)."""
+    rng = np.random.default_rng(7)
+    a = rng.random((nr, nk)).astype(np.float32)
+    s = sprand(rng, nk, nc, 0.2)
+    aa, ss = GMat.from_numpy(a), GSMat.from_csc(nk, nc, *s)
+    c = GMat.zeros(nr, nc)
+    c2 = aa.GSMult(ss, c)
+    assert c2.same(c)
+    once = c.numpy().copy()
+    aa.madd(ss, c)
+    np.testing.assert_allclose(c.numpy(), 2 * once, rtol=1e-6)
+    bb = GMat.from_numpy(rng.random((nr, nc)).astype(np.float32))
+    g = GMat.zeros(nr, nk)
+    assert bb.GSMultT(ss, g).same(g)
+    once = g.numpy().copy()
+    bb.maddT(ss, g)
+    np.testing.assert_allclose(g.numpy(), 2 * once, rtol=1e-6)
+
+
+@gpu
+def test_gpu_cache_returns_the_same_output_for_the_same_operands(hip):
+    rng = np.random.default_rng(8)
+    aa = GMat.from_numpy(rng.random((nr, nk)).astype(np.float32))
+    ss = GSMat.from_csc(nk, nc, *sprand(rng, nk, nc, 0.2))
+    Mat.set("useGPUcache", 1)
+    try:
+        c1 = aa * ss
+        c2 = aa * ss
+        assert c1.same(c2)
+        Mat.set("useGPUcache", 0)
+        assert not (aa * ss).same(c1)
+    finally:
+        Mat.set("useGPUcache", 0)
+        Mat.clear_caches()
+
+
+@gpu
+def test_dimension_mismatch_messages(hip):
+    rng = np.random.default_rng(9)
+    aa = GMat.from_numpy(rng.random((nr, nk)).astype(np.float32))
+    bad = GSMat.from_csc(nk + 1, nc, *sprand(rng, nk + 1, nc, 0.2))
+    with pytest.raises(RuntimeError, match=r"GSMult dimensions mismatch \(10 30\) \(31 20\)"):
+        aa * bad
+    with pytest.raises(RuntimeError, match=r"GSMult dimensions mismatch"):
+        aa.xT(bad)
+    with pytest.raises(RuntimeError, match=r"GSMadd dimensions mismatch"):
+        aa.madd(GSMat.from_csc(nk, nc, *sprand(rng, nk, nc, 0.2)), GMat.zeros(nr, nc + 1))
+    with pytest.raises(RuntimeError, match=r"dimensions mismatch 10,30  10,20  31,20"):
+        DDS(aa, GMat.from_numpy(rng.random((nr, nc)).astype(np.float32)), bad)
+    with pytest.raises(RuntimeError, match="dimension must be 1 or 2"):
+        aa.reduceOp(3, 0.0, 0)
+
+
+@gpu
+def test_index_base_zero_host_matrices(hip):
+    rng = np.random.default_rng(10)
+    data, ir, jc = random_csc(rng, nk, nc, 0.2)      # 0-based
+    Mat.set("ioneBased", 0)
+    try:
+        ss = GSMat.from_csc(nk, nc, data, ir, jc)
+        d2, ir2, jc2 = ss.to_csc()
+        assert np.array_equal(ir2, ir) and np.array_equal(jc2, jc) and np.array_equal(d2, data)
+    finally:
+        Mat.set("ioneBased", 1)
+    ss1 = GSMat.from_csc(nk, nc, data, ir + 1, jc + 1)
+    d3, ir3, jc3 = ss1.to_csc()
+    assert np.array_equal(ir3, ir + 1) and np.array_equal(jc3, jc + 1)
+
+
+@gpu
+def test_nmf_multiplicative_update_chain(hip):
+    """The chain of BASELINE configs[4] at a small size: R = DDS(W,H,V); Q = V ./ R on the
+    nonzeros; G = W *^ Q; rs = sum(H, 2)."""
+    rng = np.random.default_rng(11)
+    k, m, n = 16, 40, 60
+    W = (rng.random((k, m)) * 0.99 + 0.01).astype(np.float32)
+    H = (rng.random((k, n)) * 0.99 + 0.01).astype(np.float32)
+    data, ir, jc = sprand(rng, m, n, 0.15)
+    data = rng.exponential(size=data.size).astype(np.float32)
+    V = GSMat.from_csc(m, n, data, ir, jc)
+    gW, gH = GMat.from_numpy(W), GMat.from_numpy(H)
+    R = DDS(gW, gH, V)
+    # `R.contents ~ V.contents / R.contents`: the quotient overwrites R's values in place
+    V.contents().gOp(R.contents(), 3, out=R.contents())
+    Q = R
+    Q2 = V.with_values(V.contents() / DDS(gW, gH, V).contents())       # the copying form
+    assert np.array_equal(Q2.to_csc()[0], Q.to_csc()[0])
+    G = gH.xT(Q)                                   # k x m : sum_c H[:,c] * Q[r,c]
+    rs = mats.sum(gH, 2)
+    cols = np.repeat(np.arange(n), np.diff(jc))
+    r64 = np.einsum("kn,kn->n", W.astype(np.float64)[:, ir - 1], H.astype(np.float64)[:, cols])
+    q64 = data.astype(np.float64) / r64
+    g64 = np.zeros((k, m))
+    np.add.at(g64.T, ir - 1, (H.astype(np.float64)[:, cols] * q64).T)
+    np.testing.assert_allclose(Q.to_csc()[0], q64, rtol=1e-4)
+    np.testing.assert_allclose(G.numpy(), g64, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(rs.numpy().ravel(), H.astype(np.float64).sum(axis=1), rtol=1e-5)
+
+
+@gpu
+def test_flip_gflop_accounting(hip):
+    rng = np.random.default_rng(12)
+    aa = GMat.from_numpy(rng.random((64, 200)).astype(np.float32))
+    s = sprand(rng, 200, 300, 0.1)
+    ss = GSMat.from_csc(200, 300, *s)
+    mats.flip()
+    aa * ss
+    g, secs = mats.gflop()
+    assert secs > 0 and g == pytest.approx(2 * 64 * s[0].size / secs / 1e9, rel=0.2)
