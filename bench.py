@@ -1,15 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-dense product path on one MI355X.
 
-One step = one pass of the path over the headline pattern: P = DDS(A,B,S), C = A*S and
-G = A_T *^ S at k=256 on the Zipf(1.1) 100000 x 500000 pattern with ~100 M nonzeros
-(BASELINE.json configs[1] and configs[2] plus A*S on the same pattern, which the metric names).
-Inputs are synthetic, seeded, and resident in HBM before the timed region.
+Default workload ("headline"): one step = one pass of the path over the headline pattern:
+P = DDS(A,B,S), C = A*S and G = A_T *^ S at k=256 on the Zipf(1.1) 100000 x 500000 pattern with
+~100 M nonzeros (BASELINE.json configs[1] and configs[2] plus A*S on the same pattern, which
+the metric names). Inputs are synthetic, seeded, and resident in HBM before the timed region.
 
-Prints ONE JSON line. `value` is the algorithmic GB/s of the whole step (all three ops);
-per-op figures, the roofline object of the DDS kernel and the CPU baseline ride along.
+Prints ONE JSON line. `value` is the algorithmic GB/s of the whole step; per-op figures, the
+roofline object of the DDS kernel and the CPU baseline ride along.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--scale S] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload headline|C1|C4|C5]
+                  [--scale S] [--no-cpu] [--calibrate]
+
+The other workloads (C1: A*S k=32; C4: A*S k=1024 with Pareto columns; C5: the NMF update
+chain at k=128, ~400 M nonzeros) are the remaining BASELINE.json configurations; they are
+parity-test cases and are timed only on request.
 """
 import argparse
 import ctypes as C
@@ -33,7 +38,21 @@ def alg_bytes(op, k, nnz, nrows, ncols):
         return nnz * (4 * k + 8) + ncols * (4 * k + 4) + 4
     if op == "dsmultT":
         return nnz * (4 * k + 8) + nrows * (4 * k + 4) + 4
+    if op == "ewise":              # elementwise on the nonzero values: two reads, one write
+        return 12 * nnz
+    if op == "rowsum":             # dense row sums of a k x ncols matrix
+        return 4 * k * ncols + 4 * k
     raise ValueError(op)
+
+
+def flops(op, k, nnz, ncols):
+    """The reference's own accounting (GMat.scala:1057,1092; GSMat.scala:665; length for the
+    elementwise op and the reduction)."""
+    if op in ("dds", "dsmult", "dsmultT"):
+        return 2.0 * k * nnz
+    if op == "ewise":
+        return float(nnz)
+    return float(k) * ncols
 
 
 def main():
@@ -41,22 +60,24 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="headline", choices=["headline", "C1", "C4", "C5"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows/columns of the pattern (testing)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-sample", type=float, default=1.0, help="fraction of the columns timed on the CPU (1.0 = the whole workload)")
+    ap.add_argument("--cpu-sample", type=float, default=1.0,
+                    help="fraction of the columns timed on the CPU (1.0 = the whole workload)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain streaming kernel of known size (C = A + B on 3 x 1 GiB) "
                          "before the steps: the scale for rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards by "
-              "columns of S, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "columns of S; a multi-GPU figure is not part of this build)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     from bidmat_amd import gen, hip_abi
     from bidmat_amd.device import DeviceArray
 
-    lib = hip_abi.load()     # raises if the HIP library is not built: no fallback
+    lib = hip_abi.load()     # raises if the HIP library is not built: there is no fallback
     ndev = C.c_int(0)
     hip_abi.check(lib.bidmat_device_count(C.byref(ndev)), "device_count")
     if ndev.value < 1:
@@ -68,32 +89,73 @@ def main():
     hip_abi.check(lib.bidmat_device_info(arch, 64, C.byref(cus), C.byref(mem)))
 
     t0 = time.time()
-    cfg = gen.config("HEAD", args.scale)
+    cfg = gen.config("HEAD" if args.workload == "headline" else args.workload, args.scale)
     k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
     ir, jc = cfg["ir"], cfg["jc"]
     nnz = int(ir.size)
     t_gen = time.time() - t0
 
-    d_A = DeviceArray.from_numpy(cfg["A"])          # k x nrows  U(0,1)    (DDS, A*S)
-    d_B = DeviceArray.from_numpy(cfg["B"])          # k x ncols  U(0,1)    (DDS)
-    d_AT = DeviceArray.from_numpy(cfg["A_T"])       # k x ncols  N(0,1)    (A*^S)
-    d_v = DeviceArray.from_numpy(cfg["vals"])       # nnz        U(0,1]
-    d_ir = DeviceArray.from_numpy(ir)
-    d_jc = DeviceArray.from_numpy(jc)
-    d_P = DeviceArray(nnz, np.float32)
-    d_C = DeviceArray(k * ncols, np.float32)
-    d_G = DeviceArray(k * nrows, np.float32)
-
-    # plan for A*^S: built once per pattern, timed separately
-    plan = C.c_void_p()
-    hip_abi.check(lib.bidmat_synchronize())
-    t0 = time.time()
-    hip_abi.check(lib.bidmat_plan_create(nrows, ncols, nnz, d_ir.ptr, d_jc.ptr, k, C.byref(plan)), "plan_create")
-    hip_abi.check(lib.bidmat_synchronize())
-    t_plan = time.time() - t0
-
     stream = C.c_void_p()
     hip_abi.check(lib.bidmat_stream_create(C.byref(stream)))
+    h2d = {"bytes": 0, "s": 0.0}
+
+    def up(a):       # host -> device copy of an input, timed (pageable host memory)
+        t = time.perf_counter()
+        d = DeviceArray.from_numpy(a)
+        h2d["s"] += time.perf_counter() - t
+        h2d["bytes"] += a.nbytes
+        return d
+
+    d_ir, d_jc = up(ir), up(jc)
+    d_v = up(cfg["vals"])
+    keep = [d_ir, d_jc, d_v]
+    plan = C.c_void_p()
+    t_plan = [None]
+
+    def build_plan():
+        hip_abi.check(lib.bidmat_synchronize())
+        t = time.time()
+        hip_abi.check(lib.bidmat_plan_create(nrows, ncols, nnz, d_ir.ptr, d_jc.ptr, k, C.byref(plan)), "plan_create")
+        hip_abi.check(lib.bidmat_synchronize())
+        t_plan[0] = time.time() - t
+
+    # ---- the ops of one step: (name, kind, launcher)
+    if args.workload == "headline":
+        d_A, d_B, d_AT = (up(cfg[x]) for x in ("A", "B", "A_T"))
+        d_P, d_C, d_G = DeviceArray(nnz, np.float32), DeviceArray(k * ncols, np.float32), DeviceArray(k * nrows, np.float32)
+        keep += [d_A, d_B, d_AT, d_P, d_C, d_G]
+        build_plan()
+        ops = [
+            ("dds", "dds", lambda: lib.bidmat_dds_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_P.ptr, 0, stream)),
+            ("dsmult", "dsmult", lambda: lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream)),
+            ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_AT.ptr, d_v.ptr, d_G.ptr, 0, stream)),
+        ]
+        workload = "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), step = DDS, A*S, A*^S"
+        metric = "achieved HBM GB/s (algorithmic bytes) for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
+        roof_op, roof_kernel = "dds", "k_dds<W=4,V=1,LPN=64> (one launch = DDS over the whole pattern)"
+    elif args.workload in ("C1", "C4"):
+        d_A = up(cfg["A"])
+        d_C = DeviceArray(k * ncols, np.float32)
+        keep += [d_A, d_C]
+        ops = [("dsmult", "dsmult", lambda: lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream))]
+        workload = "configs[0]: A*S, k=32, 50 nnz per column" if args.workload == "C1" else \
+            "configs[3]: A*S, k=1024, Pareto(1.5) column lengths in [1,50000]"
+        metric = "achieved HBM GB/s (algorithmic bytes) for A*S (%s)" % args.workload
+        roof_op = "dsmult"
+        roof_kernel = "k_gather_axpy<W=4,V=1,LPN=8>" if args.workload == "C1" else "k_gather_axpy<W=4,V=4,LPN=64>"
+    else:  # C5: R = DDS(W,H,V); Q = V./R; G = H *^ Q; rs = sum(H,2)
+        d_W, d_H = up(cfg["W"]), up(cfg["H"])
+        d_R, d_G, d_rs = DeviceArray(nnz, np.float32), DeviceArray(k * nrows, np.float32), DeviceArray(k, np.float32)
+        keep += [d_W, d_H, d_R, d_G, d_rs]
+        build_plan()
+        ops = [
+            ("dds", "dds", lambda: lib.bidmat_dds_csc(k, ncols, nnz, d_W.ptr, d_H.ptr, d_ir.ptr, d_jc.ptr, d_R.ptr, 0, stream)),
+            ("ewise", "ewise", lambda: lib.bidmat_applyop_flat(d_v.ptr, d_R.ptr, d_R.ptr, nnz, 3, stream)),
+            ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_H.ptr, d_R.ptr, d_G.ptr, 0, stream)),
+        ]
+        workload = "configs[4]: NMF update chain R=DDS(W,H,V), Q=V./R, G=H*^Q (dense row sums timed apart)"
+        metric = "achieved HBM GB/s (algorithmic bytes) for the NMF update chain at k=128, ~400M nnz"
+        roof_op, roof_kernel = "dsmultT", "k_gather_axpy<W=4,V=1,LPN=32,plan>"
 
     def ev():
         e = C.c_void_p()
@@ -101,17 +163,12 @@ def main():
         return e
 
     def step(marks=None):
+        for i, (name, _, fn) in enumerate(ops):
+            if marks:
+                hip_abi.check(lib.bidmat_event_record(marks[i], stream))
+            hip_abi.check(fn(), name)
         if marks:
-            hip_abi.check(lib.bidmat_event_record(marks[0], stream))
-        hip_abi.check(lib.bidmat_dds_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_P.ptr, 0, stream), "dds")
-        if marks:
-            hip_abi.check(lib.bidmat_event_record(marks[1], stream))
-        hip_abi.check(lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream), "dsmult")
-        if marks:
-            hip_abi.check(lib.bidmat_event_record(marks[2], stream))
-        hip_abi.check(lib.bidmat_dsmultT_plan(plan, k, d_AT.ptr, d_v.ptr, d_G.ptr, 0, stream), "dsmultT")
-        if marks:
-            hip_abi.check(lib.bidmat_event_record(marks[3], stream))
+            hip_abi.check(lib.bidmat_event_record(marks[len(ops)], stream))
 
     if args.calibrate:
         ncal = 1 << 28                                   # 2^28 floats = 1 GiB per array
@@ -128,7 +185,7 @@ def main():
         step()
     hip_abi.check(lib.bidmat_stream_synchronize(stream))
 
-    marks = [[ev() for _ in range(4)] for _ in range(args.steps)]
+    marks = [[ev() for _ in range(len(ops) + 1)] for _ in range(args.steps)]
     hip_abi.check(lib.bidmat_synchronize())
     t0 = time.perf_counter()
     for s in range(args.steps):
@@ -136,74 +193,76 @@ def main():
     hip_abi.check(lib.bidmat_stream_synchronize(stream))
     hip_abi.check(lib.bidmat_synchronize())
     wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
 
     def elapsed(a, b):
         ms = C.c_float(0)
         hip_abi.check(lib.bidmat_event_elapsed_ms(a, b, C.byref(ms)))
         return float(ms.value)
 
-    op_ms = {"dds": [], "dsmult": [], "dsmultT": []}
-    for m in marks:
-        op_ms["dds"].append(elapsed(m[0], m[1]))
-        op_ms["dsmult"].append(elapsed(m[1], m[2]))
-        op_ms["dsmultT"].append(elapsed(m[2], m[3]))
-    ms_per_step = wall * 1e3 / args.steps
-
-    ops = {}
-    total_bytes = 0
-    for op in ("dds", "dsmult", "dsmultT"):
-        b = alg_bytes(op, k, nnz, nrows, ncols)
+    per_op, total_bytes, total_flops = {}, 0, 0.0
+    for i, (name, kind, _) in enumerate(ops):
+        t = [elapsed(m[i], m[i + 1]) for m in marks]
+        b = alg_bytes(kind, k, nnz, nrows, ncols)
         total_bytes += b
-        avg = float(np.mean(op_ms[op]))
-        ops[op] = {
-            "ms_avg": round(avg, 4), "ms_min": round(float(np.min(op_ms[op])), 4),
-            "alg_GB": round(b / 1e9, 3),
-            "GBps": round(b / avg / 1e6, 1),
-            "nnz_per_s": round(nnz / avg * 1e3, 1),
-            "GFLOPs": round(2.0 * k * nnz / avg / 1e6, 1),
+        total_flops += flops(kind, k, nnz, ncols)
+        avg = float(np.mean(t))
+        per_op[name] = {
+            "ms_avg": round(avg, 4), "ms_min": round(float(np.min(t)), 4), "alg_GB": round(b / 1e9, 3),
+            "GBps": round(b / avg / 1e6, 1), "nnz_per_s": round(nnz / avg * 1e3, 1),
+            "GFLOPs": round(flops(kind, k, nnz, ncols) / avg / 1e6, 1),
             "frac_of_hbm_peak": round(b / avg / 1e6 / HBM_PEAK_GBS, 4),
         }
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # roofline object: the DDS kernel (the configuration the metric is quoted on)
-    dds_avg = float(np.mean(op_ms["dds"]))
-    dds_bytes = alg_bytes("dds", k, nnz, nrows, ncols)
+    r_avg, r_bytes = per_op[roof_op]["ms_avg"], alg_bytes(roof_op, k, nnz, nrows, ncols)
     roofline = {
-        "kernel": "k_dds<W=4,V=1,LPN=64> (one launch = DDS over the whole pattern)",
-        "bound": "hbm", "achieved": round(dds_bytes / dds_avg / 1e6, 1), "peak": HBM_PEAK_GBS,
-        "unit": "GB/s", "frac": round(dds_bytes / dds_avg / 1e6 / HBM_PEAK_GBS, 4),
-        "traffic": None,
-        "bytes_per_launch": dds_bytes, "avg_launch_ms": round(dds_avg, 4),
+        "kernel": roof_kernel, "bound": "hbm", "achieved": round(r_bytes / r_avg / 1e6, 1), "peak": HBM_PEAK_GBS,
+        "unit": "GB/s", "frac": round(r_bytes / r_avg / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
+        "bytes_per_launch": r_bytes, "avg_launch_ms": round(r_avg, 4),
     }
 
     out = {
-        "metric": "achieved HBM GB/s (algorithmic bytes) for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), "
-                               "step = DDS, A*S, A*^S", "k": k, "nrows": nrows, "ncols": ncols, "nnz": nnz,
-                   "scale": args.scale},
-        "nnz_per_s": round(3 * nnz / (ms_per_step * 1e-3), 1),
-        "GFLOPs": round(3 * 2.0 * k * nnz / (ms_per_step * 1e-3) / 1e9, 1),
+        "metric": metric, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": workload, "k": k, "nrows": nrows, "ncols": ncols, "nnz": nnz, "scale": args.scale},
+        "nnz_per_s": round(len([o for o in ops if o[1] != "ewise"]) * nnz / (ms_per_step * 1e-3), 1),
+        "GFLOPs": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "ops": ops,
-        "roofline": roofline,
-        "plan": {"build_ms": round(t_plan * 1e3, 2), "segments": lib.bidmat_plan_segments(plan),
-                 "bytes": lib.bidmat_plan_bytes(plan)},
+        "ops": per_op, "roofline": roofline,
         "device": {"arch": arch.value.decode(), "compute_units": cus.value, "mem_GiB": round(mem.value / 2**30, 1)},
         "gen_s": round(t_gen, 2),
+        # informational: what one step would cost if every input crossed PCIe first (never `value`)
+        "h2d": {"GB": round(h2d["bytes"] / 1e9, 3), "s": round(h2d["s"], 3),
+                "GBps": round(h2d["bytes"] / h2d["s"] / 1e9, 2),
+                "step_GBps_incl_h2d": round(total_bytes / (ms_per_step * 1e-3 + h2d["s"]) / 1e9, 1)},
     }
+    if t_plan[0] is not None:
+        out["plan"] = {"build_ms": round(t_plan[0] * 1e3, 2), "segments": lib.bidmat_plan_segments(plan),
+                       "bytes": lib.bidmat_plan_bytes(plan)}
+    if args.workload == "C5":      # the dense row sums of H, timed apart from the chain
+        e0, e1 = ev(), ev()
+        hip_abi.check(lib.bidmat_reduce2op(k, ncols, d_H.ptr, d_rs.ptr, 0.0, 0))
+        hip_abi.check(lib.bidmat_event_record(e0, None))
+        for _ in range(5):
+            hip_abi.check(lib.bidmat_reduce2op(k, ncols, d_H.ptr, d_rs.ptr, 0.0, 0))
+        hip_abi.check(lib.bidmat_event_record(e1, None))
+        hip_abi.check(lib.bidmat_synchronize())
+        t = elapsed(e0, e1) / 5
+        b = alg_bytes("rowsum", k, nnz, nrows, ncols)
+        out["rowsum"] = {"ms_avg": round(t, 4), "GBps": round(b / t / 1e6, 1),
+                         "frac_of_hbm_peak": round(b / t / 1e6 / HBM_PEAK_GBS, 4)}
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample)
+        out["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_sample)
 
     print(json.dumps(out))
 
 
-def cpu_baseline(cfg, frac):
-    """The CPU restatement of the reference's loops (oracle/, threads as the reference splits
-    them) on the first `frac` of the columns of the same workload."""
+def cpu_baseline(workload, cfg, frac):
+    """The CPU restatement of the reference's loops (oracle/, threads split as the reference
+    splits them) on the first `frac` of the columns of the same workload, best of two runs."""
     import oracle
     k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
     nc = max(1, int(ncols * frac))
@@ -212,19 +271,43 @@ def cpu_baseline(cfg, frac):
     ir = cfg["ir"][:nnz]
     vals = cfg["vals"][:nnz]
     threads = oracle.max_threads()
-    A, B, AT = cfg["A"], cfg["B"][: k * nc], cfg["A_T"][: k * nc]
+
+    def best(fn, reps=2):
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return min(ts)
+
     t = {}
-    t0 = time.perf_counter(); oracle.dds(A, B, k, ir, jc, nthreads=threads); t["dds"] = time.perf_counter() - t0
-    t0 = time.perf_counter(); oracle.fsmult(A, k, vals, ir, jc, nthreads=threads); t["dsmult"] = time.perf_counter() - t0
-    t0 = time.perf_counter(); oracle.fsmultT(AT, k, nrows, vals, ir, jc, nthreads=threads); t["dsmultT"] = time.perf_counter() - t0
+    if workload == "headline":
+        A, B, AT = cfg["A"], cfg["B"][: k * nc], cfg["A_T"][: k * nc]
+        t["dds"] = best(lambda: oracle.dds(A, B, k, ir, jc, nthreads=threads))
+        t["dsmult"] = best(lambda: oracle.fsmult(A, k, vals, ir, jc, nthreads=threads))
+        t["dsmultT"] = best(lambda: oracle.fsmultT(AT, k, nrows, vals, ir, jc, nthreads=threads))
+    elif workload in ("C1", "C4"):
+        t["dsmult"] = best(lambda: oracle.fsmult(cfg["A"], k, vals, ir, jc, nthreads=threads))
+    else:
+        W, H = cfg["W"], cfg["H"][: k * nc]
+        r, q = [None], [None]
+
+        def dds():
+            r[0] = oracle.dds(W, H, k, ir, jc, nthreads=threads)[0]
+
+        def ew():
+            q[0] = oracle.applyop(vals, r[0], 3)
+        t["dds"] = best(dds, 1)
+        t["ewise"] = best(ew, 1)
+        t["dsmultT"] = best(lambda: oracle.fsmultT(H, k, nrows, q[0], ir, jc, nthreads=threads), 1)
     total_b = sum(alg_bytes(op, k, nnz, nrows, nc) for op in t)
     total_s = sum(t.values())
     return {
         "value": round(total_b / total_s / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-        "sample": "first %d of %d columns (%d nnz) of the same workload; DDS, A*S, A*^S each once; A*^S "
-                  "uses min(cores, k/32) threads as the reference does" % (nc, ncols, nnz),
+        "sample": "first %d of %d columns (%d nnz) of the same workload, every op of the step, best of two "
+                  "runs; A*^S uses min(cores, k/32) threads as the reference does" % (nc, ncols, nnz),
         "seconds": {op: round(s, 3) for op, s in t.items()},
-        "nnz_per_s": round(3 * nnz / total_s, 1),
+        "nnz_per_s": round(len([o for o in t if o != "ewise"]) * nnz / total_s, 1),
     }
 
 

@@ -1,0 +1,177 @@
+"""Parity at the full sizes of BASELINE.json's configurations, where the oracle cannot run the
+whole problem in seconds: size-independent properties (the Frobenius identity that ties the
+three products together, linearity, sum-of-sums) plus oracle checks on random samples of
+columns / rows / nonzeros of the full-size result.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from bidmat_amd import gen, hip_abi
+from bidmat_amd.device import DeviceArray
+from util import make_plan
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-4
+
+
+def close(x, ref64, sa, what):
+    ok, worst = oracle.within_tolerance(x, ref64, sa, RTOL)
+    assert ok, "%s: worst error measure %.3e" % (what, worst)
+
+
+def sub_csc(ir, jc, vals, cols):
+    """CSC restricted to the given columns (kept in the given order)."""
+    lens = jc[cols + 1] - jc[cols]
+    sjc = np.zeros(cols.size + 1, dtype=np.int32)
+    sjc[1:] = np.cumsum(lens)
+    idx = np.concatenate([np.arange(jc[c], jc[c + 1]) for c in cols]) if cols.size else np.zeros(0, np.int64)
+    return (vals[idx] if vals is not None else None), ir[idx], sjc, idx
+
+
+def rows_sub_csc(ir, jc, vals, rows):
+    """All nonzeros of the given rows, as a CSC over all columns with rows renumbered 0..len-1."""
+    pos = np.full(int(ir.max()) + 1, -1, dtype=np.int64)
+    pos[rows] = np.arange(rows.size)
+    keep = np.flatnonzero(pos[ir] >= 0)
+    ic = np.searchsorted(jc, keep, side="right") - 1
+    sjc = np.zeros(jc.size, dtype=np.int32)
+    sjc[1:] = np.cumsum(np.bincount(ic, minlength=jc.size - 1))
+    return vals[keep], pos[ir[keep]].astype(np.int32), sjc
+
+
+@pytest.mark.timeout(600)
+def test_headline_pattern_dds_dsmult_dsmultT(hip):
+    """configs[1] (DDS) and configs[2] (A*^S) at full size, plus A*S on the same pattern."""
+    cfg = gen.config("HEAD", 1.0)
+    k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
+    ir, jc, vals = cfg["ir"], cfg["jc"], cfg["vals"]
+    nnz = int(ir.size)
+    assert 0.9e8 < nnz < 1.1e8
+    assert oracle.check(nrows, ncols, nnz, ir, jc, 0)[0] == 0
+    A, B, AT = cfg["A"], cfg["B"], cfg["A_T"]
+    dA, dB, dAT = DeviceArray.from_numpy(A), DeviceArray.from_numpy(B), DeviceArray.from_numpy(AT)
+    dv, dir_, djc = DeviceArray.from_numpy(vals), DeviceArray.from_numpy(ir), DeviceArray.from_numpy(jc)
+    dP, dC, dG = DeviceArray(nnz, np.float32), DeviceArray(k * ncols, np.float32), DeviceArray(k * nrows, np.float32)
+    plan = make_plan(hip, nrows, ncols, nnz, dir_, djc, k)
+    hip_abi.check(hip.bidmat_dds_csc(k, ncols, nnz, dA.ptr, dB.ptr, dir_.ptr, djc.ptr, dP.ptr, 0, None))
+    hip_abi.check(hip.bidmat_dsmult_csc(k, ncols, nnz, dA.ptr, dv.ptr, dir_.ptr, djc.ptr, dC.ptr, 0, None))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, dAT.ptr, dv.ptr, dG.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    P, Cm, G = dP.numpy(), dC.numpy(), dG.numpy()
+    # pattern arrays untouched, bit for bit
+    assert np.array_equal(dir_.numpy(), ir) and np.array_equal(djc.numpy(), jc)
+
+    rng = np.random.default_rng(0)
+    # --- sampled columns against the oracle: DDS and A*S
+    cols = np.unique(np.concatenate([rng.integers(0, ncols, 300), [0, ncols - 1]]))
+    sv, sir, sjc, idx = sub_csc(ir, jc, vals, cols)
+    Bs = B.reshape(ncols, k)[cols].ravel()
+    ref64, sa = oracle.dds_f64(A, Bs, k, sir, sjc, nthreads=8)
+    close(P[idx], ref64, sa, "DDS sampled columns")
+    ref64, sa = oracle.fsmult_f64(A, k, sv, sir, sjc, nthreads=8)
+    close(Cm.reshape(ncols, k)[cols].ravel(), ref64, sa, "A*S sampled columns")
+    # --- sampled rows against the oracle: A*^S (head rows have ~500k terms each, tail rows a few)
+    rows = np.unique(np.concatenate([rng.integers(0, nrows, 200), [0, 1, 2, nrows - 1]]))
+    rv, rir, rjc = rows_sub_csc(ir, jc, vals, rows)
+    ref64, sa = oracle.fsmultT_f64(AT, k, rows.size, rv, rir, rjc, nthreads=8)
+    close(G.reshape(nrows, k)[rows].ravel(), ref64, sa, "A*^S sampled rows")
+
+    # --- the three products agree: <A*S, B> == sum_j v_j * DDS_j ; <B*^S, A> checked with A_T's own DDS
+    f1 = np.dot(Cm.astype(np.float64), B.astype(np.float64))
+    f2 = np.dot(P.astype(np.float64), vals.astype(np.float64))
+    assert abs(f1 - f2) <= 1e-6 * abs(f2)
+    hip_abi.check(hip.bidmat_dds_csc(k, ncols, nnz, dA.ptr, dAT.ptr, dir_.ptr, djc.ptr, dP.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    f3 = np.dot(G.astype(np.float64), A.astype(np.float64))
+    f4 = np.dot(dP.numpy().astype(np.float64), vals.astype(np.float64))
+    scale = np.dot(np.abs(G).astype(np.float64), np.abs(A).astype(np.float64))
+    assert abs(f3 - f4) <= 1e-6 * scale
+
+    # --- sparse sums on the same pattern: sum of column sums == sum of row sums == sum of values
+    dcs, drs = DeviceArray(ncols, np.float32), DeviceArray(nrows, np.float32)
+    hip_abi.check(hip.bidmat_spsum_cols(ncols, nnz, dv.ptr, djc.ptr, dcs.ptr, 0, None))
+    hip_abi.check(hip.bidmat_spsum_rows_plan(plan, dv.ptr, drs.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    total = vals.sum(dtype=np.float64)
+    assert abs(dcs.numpy().sum(dtype=np.float64) - total) <= 1e-6 * total
+    assert abs(drs.numpy().sum(dtype=np.float64) - total) <= 1e-6 * total
+    ref64, sa = oracle.spsum_f64(nrows, vals, ir, jc, 2)
+    close(drs.numpy(), ref64, sa, "row sums")
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+
+
+@pytest.mark.timeout(600)
+def test_config4_wide_k_power_law_columns(hip):
+    """configs[3]: k=1024, Pareto column lengths clipped to [1,50000] (split-column path),
+    output 1024 x 1 000 000 (4.1 GB)."""
+    cfg = gen.config("C4", 1.0)
+    k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
+    ir, jc, vals, A = cfg["ir"], cfg["jc"], cfg["vals"], cfg["A"]
+    nnz = int(ir.size)
+    lens = np.diff(jc)
+    assert lens.max() > 10000 and 25e6 < nnz < 60e6
+    dA, dv = DeviceArray.from_numpy(A), DeviceArray.from_numpy(vals)
+    dir_, djc = DeviceArray.from_numpy(ir), DeviceArray.from_numpy(jc)
+    dC = DeviceArray(k * ncols, np.float32)
+    hip_abi.check(hip.bidmat_dsmult_csc(k, ncols, nnz, dA.ptr, dv.ptr, dir_.ptr, djc.ptr, dC.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    rng = np.random.default_rng(4)
+    longest = np.argsort(lens)[-5:]
+    cols = np.unique(np.concatenate([rng.integers(0, ncols, 100), longest, [0, ncols - 1]]))
+    got = np.concatenate([dC_slice(dC, c, k) for c in cols])
+    sv, sir, sjc, _ = sub_csc(ir, jc, vals, cols)
+    ref64, sa = oracle.fsmult_f64(A, k, sv, sir, sjc, nthreads=8)
+    close(got, ref64, sa, "C4 sampled + longest columns")
+    # linearity in the values: A*(2S) == 2*(A*S) exactly (scaling by 2 is exact in fp32)
+    dv2 = DeviceArray.from_numpy(vals * np.float32(2))
+    dC2 = DeviceArray(k * 4096, np.float32)
+    hip_abi.check(hip.bidmat_dsmult_csc(k, 4096, int(jc[4096]), dA.ptr, dv2.ptr, dir_.ptr, djc.ptr, dC2.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert np.array_equal(dC2.numpy(), 2 * dC.numpy(k * 4096))
+
+
+def dC_slice(d, c, k):
+    out = np.empty(k, dtype=np.float32)
+    hip_abi.check(d.lib.bidmat_memcpy_d2h(out.ctypes.data, d.ptr + 4 * k * int(c), 4 * k))
+    return out
+
+
+@pytest.mark.timeout(900)
+def test_config5_nmf_step(hip):
+    """configs[4]: R = DDS(W,H,V); Q = V./R on the nonzeros; G = H *^ Q; rs = sum(H,2), k=128,
+    V 1M x 1M with ~400M nonzeros."""
+    cfg = gen.config("C5", 1.0)
+    k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
+    ir, jc, vals, W, H = cfg["ir"], cfg["jc"], cfg["vals"], cfg["W"], cfg["H"]
+    nnz = int(ir.size)
+    assert 3.5e8 < nnz < 4.5e8
+    dW, dH, dv = DeviceArray.from_numpy(W), DeviceArray.from_numpy(H), DeviceArray.from_numpy(vals)
+    dir_, djc = DeviceArray.from_numpy(ir), DeviceArray.from_numpy(jc)
+    dR, dG, drs = DeviceArray(nnz, np.float32), DeviceArray(k * nrows, np.float32), DeviceArray(k, np.float32)
+    plan = make_plan(hip, nrows, ncols, nnz, dir_, djc, k)
+    hip_abi.check(hip.bidmat_dds_csc(k, ncols, nnz, dW.ptr, dH.ptr, dir_.ptr, djc.ptr, dR.ptr, 0, None))
+    hip_abi.check(hip.bidmat_applyop_flat(dv.ptr, dR.ptr, dR.ptr, nnz, 3, None))          # Q = V ./ R in place
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, dH.ptr, dR.ptr, dG.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    hip_abi.check(hip.bidmat_reduce2op(k, ncols, dH.ptr, drs.ptr, 0.0, 0))
+    Q, G = dR.numpy(), dG.numpy()
+    rng = np.random.default_rng(5)
+    # sampled columns: Q against the oracle (DDS then an IEEE division)
+    cols = np.unique(rng.integers(0, ncols, 200))
+    sv, sir, sjc, idx = sub_csc(ir, jc, vals, cols)
+    r32, _, _ = oracle.dds(W, H.reshape(ncols, k)[cols].ravel(), k, sir, sjc, nthreads=8)
+    r64, sa = oracle.dds_f64(W, H.reshape(ncols, k)[cols].ravel(), k, sir, sjc, nthreads=8)
+    np.testing.assert_allclose(Q[idx], sv.astype(np.float64) / r64, rtol=2e-4)
+    np.testing.assert_allclose(Q[idx], sv / r32, rtol=2e-5)
+    # sampled rows: G against the oracle fed with the device's own Q
+    rows = np.unique(np.concatenate([rng.integers(0, nrows, 100), [0, 1, nrows - 1]]))
+    rv, rir, rjc = rows_sub_csc(ir, jc, Q, rows)
+    ref64, sa = oracle.fsmultT_f64(H, k, rows.size, rv, rir, rjc, nthreads=8)
+    close(G.reshape(nrows, k)[rows].ravel(), ref64, sa, "NMF G sampled rows")
+    # dense row sums of H
+    ref = H.reshape(ncols, k).astype(np.float64).sum(axis=0)
+    np.testing.assert_allclose(drs.numpy(), ref, rtol=1e-5)
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
