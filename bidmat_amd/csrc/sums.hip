@@ -39,9 +39,9 @@ template <> __device__ __forceinline__ float op_identity<2>() { return 1.f; }
 template <> __device__ __forceinline__ float op_identity<10>() { return -INFINITY; }
 template <> __device__ __forceinline__ float op_identity<11>() { return INFINITY; }
 
-// Column reduce. lpc lanes (power of two <= 64) per column; rows [r0, r1) of chunk blockIdx.y.
-// out[chunk*ncols + c].
-template <int OP>
+// Column reduce. lpc lanes (power of two <= 64) per column, W consecutive rows per lane and step
+// (W = 4: 128-bit loads); rows [r0, r1) of chunk blockIdx.y. out[chunk*ncols + c].
+template <int OP, int W>
 __global__ __launch_bounds__(BM_BLOCK) void k_reduce_cols(int nrows, int ncols, int lpc, int rows_per_chunk,
                                                           const float* __restrict__ A,
                                                           float* __restrict__ out) {
@@ -54,35 +54,68 @@ __global__ __launch_bounds__(BM_BLOCK) void k_reduce_cols(int nrows, int ncols, 
     float acc = op_identity<OP>();
     if (c < ncols) {
         const float* col = A + (size_t)c * nrows;
-        for (long long r = r0 + l; r < r1; r += lpc) acc = op2<OP>(acc, col[r]);
+        for (long long r = r0 + (long long)l * W; r < r1; r += (long long)lpc * W) {
+            const Vec<W> v = Vec<W>::load(col + r);
+            const float* f = reinterpret_cast<const float*>(&v);
+#pragma unroll
+            for (int i = 0; i < W; ++i) acc = op2<OP>(acc, f[i]);
+        }
     }
     for (int d = 1; d < lpc; d <<= 1) acc = op2<OP>(acc, __shfl_xor(acc, d, 64));
     if (c < ncols && l == 0) out[(size_t)blockIdx.y * ncols + c] = acc;
 }
 
-// Row reduce, stage 1. Block = rb rows x cl column lanes (rb*cl == 256); blockIdx.y = row tile,
-// blockIdx.x = column chunk. out[chunk*nrows + r].
-template <int OP>
+// Row reduce, stage 1. A block is rb row-lanes x cl column-lanes (rb*cl == 256); every lane owns W
+// consecutive rows (W = 4: 128-bit loads); blockIdx.x = row tile, blockIdx.y = column chunk.
+// Four independent accumulators per lane keep four loads in flight. out[chunk*nrows + r].
+template <int OP, int W>
 __global__ __launch_bounds__(BM_BLOCK) void k_reduce_rows(int nrows, int ncols, int rb, int cols_per_chunk,
                                                           const float* __restrict__ A,
                                                           float* __restrict__ out) {
-    __shared__ float sm[BM_BLOCK];
+    __shared__ float sm[BM_BLOCK * W];
     const int cl = BM_BLOCK / rb;
     const int tr = threadIdx.x % rb;
     const int tc = threadIdx.x / rb;
-    const long long r = (long long)blockIdx.y * rb + tr;
-    const long long c0 = (long long)blockIdx.x * cols_per_chunk;
+    const long long r = ((long long)blockIdx.x * rb + tr) * W;
+    const long long c0 = (long long)blockIdx.y * cols_per_chunk;
     long long c1 = c0 + cols_per_chunk;
     if (c1 > ncols) c1 = ncols;
-    float acc = op_identity<OP>();
+    float acc[4][W];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < W; ++i) acc[u][i] = op_identity<OP>();
     if (r < nrows) {
-        for (long long c = c0 + tc; c < c1; c += cl) acc = op2<OP>(acc, A[(size_t)c * nrows + r]);
+        long long c = c0 + tc;
+        for (; c + 3LL * cl < c1; c += 4LL * cl) {
+            Vec<W> v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = Vec<W>::load(A + (size_t)(c + (long long)u * cl) * nrows + r);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const float* f = reinterpret_cast<const float*>(&v[u]);
+#pragma unroll
+                for (int i = 0; i < W; ++i) acc[u][i] = op2<OP>(acc[u][i], f[i]);
+            }
+        }
+        for (; c < c1; c += cl) {
+            Vec<W> v = Vec<W>::load(A + (size_t)c * nrows + r);
+            const float* f = reinterpret_cast<const float*>(&v);
+#pragma unroll
+            for (int i = 0; i < W; ++i) acc[0][i] = op2<OP>(acc[0][i], f[i]);
+        }
     }
-    sm[threadIdx.x] = acc;
+#pragma unroll
+    for (int i = 0; i < W; ++i)
+        sm[threadIdx.x * W + i] = op2<OP>(op2<OP>(acc[0][i], acc[1][i]), op2<OP>(acc[2][i], acc[3][i]));
     __syncthreads();
     if (tc == 0 && r < nrows) {
-        for (int q = 1; q < cl; ++q) acc = op2<OP>(acc, sm[q * rb + tr]);
-        out[(size_t)blockIdx.x * nrows + r] = acc;
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+            float a = sm[threadIdx.x * W + i];
+            for (int q = 1; q < cl; ++q) a = op2<OP>(a, sm[(q * rb + tr) * W + i]);
+            out[(size_t)blockIdx.y * nrows + r + i] = a;
+        }
     }
 }
 
@@ -99,7 +132,10 @@ __global__ __launch_bounds__(BM_BLOCK) void k_reduce_chunks(int n, int nchunks, 
 
 template <int OP>
 hipError_t reduce1_impl(int nrows, int ncols, const float* A, float* B, hipStream_t s) {
-    int lpc = pow2ceil(nrows) < 64 ? pow2ceil(nrows) : 64;
+    const bool vec = (nrows % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
+    const int W = vec ? 4 : 1;
+    const int nv = (nrows + W - 1) / W;
+    int lpc = pow2ceil(nv) < 64 ? pow2ceil(nv) : 64;
     // few, very long columns: cut the rows into chunks so the whole chip works
     int nchunks = 1;
     if ((long long)ncols * lpc < 64 * 2048 && nrows > 8192) {
@@ -110,6 +146,7 @@ hipError_t reduce1_impl(int nrows, int ncols, const float* A, float* B, hipStrea
         if (nchunks > 4096) nchunks = 4096;
     }
     int rows_per_chunk = (nrows + nchunks - 1) / nchunks;
+    rows_per_chunk = (rows_per_chunk + 3) & ~3;            // chunk starts stay 16-byte aligned
     nchunks = (nrows + rows_per_chunk - 1) / rows_per_chunk;
     long long threads = (long long)ncols * lpc;
     long long nblk = (threads + BM_BLOCK - 1) / BM_BLOCK;
@@ -120,8 +157,10 @@ hipError_t reduce1_impl(int nrows, int ncols, const float* A, float* B, hipStrea
         dst = (float*)ws_get(WS_REDUCE, sizeof(float) * (size_t)nchunks * ncols, &err);
         if (!dst) return err;
     }
-    hipLaunchKernelGGL(k_reduce_cols<OP>, dim3((unsigned)nblk, (unsigned)nchunks), dim3(BM_BLOCK), 0, s,
-                       nrows, ncols, lpc, rows_per_chunk, A, dst);
+    if (vec) hipLaunchKernelGGL((k_reduce_cols<OP, 4>), dim3((unsigned)nblk, (unsigned)nchunks), dim3(BM_BLOCK), 0, s,
+                                nrows, ncols, lpc, rows_per_chunk, A, dst);
+    else hipLaunchKernelGGL((k_reduce_cols<OP, 1>), dim3((unsigned)nblk, (unsigned)nchunks), dim3(BM_BLOCK), 0, s,
+                            nrows, ncols, lpc, rows_per_chunk, A, dst);
     if (nchunks > 1) {
         unsigned nb2 = (unsigned)(((long long)ncols + BM_BLOCK - 1) / BM_BLOCK);
         hipLaunchKernelGGL(k_reduce_chunks<OP>, dim3(nb2), dim3(BM_BLOCK), 0, s, ncols, nchunks, dst, B);
@@ -129,27 +168,48 @@ hipError_t reduce1_impl(int nrows, int ncols, const float* A, float* B, hipStrea
     return hipGetLastError();
 }
 
+// Row reduce of a column-major nrows x ncols matrix with leading dimension nrows. Stage 1 cuts the
+// columns into chunks (one workgroup each); the chunk partials form an nrows x nchunks matrix that
+// is reduced the same way again until few enough chunks remain for k_reduce_chunks. `scratch`
+// is a workspace of `scratch_floats` floats for the partials (nullptr: take it from the slot).
 template <int OP>
-hipError_t reduce2_impl(int nrows, int ncols, const float* A, float* B, hipStream_t s) {
-    int rb = pow2ceil(nrows) < BM_BLOCK ? pow2ceil(nrows) : BM_BLOCK;
+hipError_t reduce2_impl(int nrows, int ncols, const float* A, float* B, hipStream_t s,
+                        float* scratch = nullptr, size_t scratch_floats = 0) {
+    const bool vec = (nrows % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
+    const int W = vec ? 4 : 1;
+    const int lanes = (nrows + W - 1) / W;                 // row-lanes needed
+    int rb = pow2ceil(lanes) < BM_BLOCK ? pow2ceil(lanes) : BM_BLOCK;
     int cl = BM_BLOCK / rb;
-    long long rowtiles = ((long long)nrows + rb - 1) / rb;
-    // enough column chunks to fill the chip, at least 8 columns per lane
+    long long rowtiles = ((long long)lanes + rb - 1) / rb;
+    // enough column chunks to fill the chip, at least 16 columns per column-lane
     long long nchunks = 4096 / rowtiles;
-    long long maxc = ((long long)ncols + (long long)cl * 8 - 1) / ((long long)cl * 8);
+    long long maxc = ((long long)ncols + (long long)cl * 16 - 1) / ((long long)cl * 16);
     if (nchunks > maxc) nchunks = maxc;
     if (nchunks < 1) nchunks = 1;
     int cols_per_chunk = (int)(((long long)ncols + nchunks - 1) / nchunks);
     nchunks = ((long long)ncols + cols_per_chunk - 1) / cols_per_chunk;
-    if (rowtiles > 65535) return hipErrorInvalidValue;
+    if (rowtiles > 0x7fffffffLL || nchunks > 65535) return hipErrorInvalidValue;
     float* dst = B;
     if (nchunks > 1) {
-        hipError_t err;
-        dst = (float*)ws_get(WS_REDUCE, sizeof(float) * (size_t)nchunks * nrows, &err);
-        if (!dst) return err;
+        const size_t need = (size_t)nchunks * nrows;
+        if (!scratch) {
+            // room for this level's partials and, behind them, every deeper level's (each at most
+            // 1/16 of the one before)
+            hipError_t err;
+            scratch_floats = need + need / 8 + 4096;
+            scratch = (float*)ws_get(WS_REDUCE, sizeof(float) * scratch_floats, &err);
+            if (!scratch) return err;
+        }
+        if (need > scratch_floats) return hipErrorInvalidValue;
+        dst = scratch;
     }
-    hipLaunchKernelGGL(k_reduce_rows<OP>, dim3((unsigned)nchunks, (unsigned)rowtiles), dim3(BM_BLOCK), 0, s,
-                       nrows, ncols, rb, cols_per_chunk, A, dst);
+    dim3 grid((unsigned)rowtiles, (unsigned)nchunks), block(BM_BLOCK);
+    if (vec) hipLaunchKernelGGL((k_reduce_rows<OP, 4>), grid, block, 0, s, nrows, ncols, rb, cols_per_chunk, A, dst);
+    else hipLaunchKernelGGL((k_reduce_rows<OP, 1>), grid, block, 0, s, nrows, ncols, rb, cols_per_chunk, A, dst);
+    if (nchunks > 32) {
+        const size_t used = ((size_t)nchunks * nrows + 3) & ~size_t(3);     // keep 16-byte alignment
+        return reduce2_impl<OP>(nrows, (int)nchunks, dst, B, s, scratch + used, scratch_floats - used);
+    }
     if (nchunks > 1) {
         unsigned nb2 = (unsigned)(((long long)nrows + BM_BLOCK - 1) / BM_BLOCK);
         hipLaunchKernelGGL(k_reduce_chunks<OP>, dim3(nb2), dim3(BM_BLOCK), 0, s, nrows, (int)nchunks, dst, B);
