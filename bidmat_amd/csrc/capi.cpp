@@ -144,6 +144,51 @@ API int bidmat_dsmultT(int nrows, int ncols, int nnz, const float* A, const floa
     return finish_blocking(err);
 }
 
+API int bidmat_dsmultTile(int nr, int nc, int kk, int nnz, const float* A, int lda, const float* Bdata,
+                          const int* Bir, const int* Bic, int broff, int bcoff, float* C, int ldc) {
+    if (nr < 0 || nc < 0 || kk < 0 || nnz < 0 || broff < 0 || bcoff < 0 || lda < nr || ldc < nr) return kInvalid;
+    if (nr == 0 || nc == 0 || kk == 0 || nnz == 0) return 0;
+    if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
+    // the launcher does not receive S's column count: it is max(Bic)+1, and Bic is non-decreasing
+    int last = 0;
+    hipError_t err = hipMemcpy(&last, Bic + (nnz - 1), sizeof(int), hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return (int)err;
+    if (last < 0 || last == 0x7fffffff) return kInvalid;
+    const int ncolsS = last + 1;
+    if (bcoff >= ncolsS) return 0;                       // the tile holds no stored column
+    const int nc_eff = nc < ncolsS - bcoff ? nc : ncolsS - bcoff;
+    int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncolsS + 1), &err);
+    if (!jc) return (int)err;
+    err = bm::coo_compress_cols(ncolsS, nnz, Bic, jc, nullptr);
+    if (err == hipSuccess)
+        err = bm::dsmult_csc_ex(nr, lda, ldc, nc_eff, nnz, A, Bdata, Bir, jc + bcoff, C, 1, bm::Window{1, broff, kk}, nullptr);
+    return finish_blocking(err);
+}
+
+API int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float* A, int lda, const float* Bdata,
+                           const int* Bir, const int* Bic, int broff, int bcoff, float* C, int ldc) {
+    if (nr < 0 || nc < 0 || kk < 0 || nnz < 0 || broff < 0 || bcoff < 0 || lda < nr || ldc < nr) return kInvalid;
+    if (nr == 0 || nc == 0 || kk == 0 || nnz == 0) return 0;
+    if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
+    int last = 0;
+    hipError_t err = hipMemcpy(&last, Bic + (nnz - 1), sizeof(int), hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return (int)err;
+    if (last < 0 || last == 0x7fffffff) return kInvalid;
+    bidmat_plan* plan = nullptr;
+    err = cached_plan(last + 1, nnz, Bir, Bic, nr, &plan);
+    if (err != hipSuccess) return finish_blocking(err);
+    if (broff >= plan->nrows) return 0;                  // the tile holds no stored row
+    const int nrows_eff = nc < plan->nrows - broff ? nc : plan->nrows - broff;
+    err = bm::plan_reserve_partial(plan, nr);
+    if (err == hipSuccess)
+        err = bm::gather_segments_ex(nr, lda, plan->nseg, plan->xcd_start, A, Bdata, plan->pc, plan->perm,
+                                     plan->segstart, plan->partial, bm::Window{1, bcoff, kk}, plan->segrow,
+                                     bm::Window{1, broff, nrows_eff}, nullptr);
+    if (err == hipSuccess)
+        err = bm::reduce_segments_ex(nr, ldc, broff, nrows_eff, plan->rowptr, plan->rowseg, plan->partial, C, 1, nullptr);
+    return finish_blocking(err);
+}
+
 API int bidmat_dds(int nrows, int nnz, const float* A, const float* B, const int* Cir,
                    const int* Cic, float* P) {
     if (nrows < 0 || nnz < 0) return kInvalid;

@@ -26,6 +26,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_compress_cols(int ncols, int nnz, 
     int prev = (j == 0) ? -1 : ic[j - 1];
     int cur = (j == nnz) ? ncols : ic[j];
     if (prev >= ncols) prev = ncols - 1;      // malformed input: stay inside jc
+    if (prev < -1) prev = -1;
     if (cur > ncols) cur = ncols;
     for (int c = prev + 1; c <= cur; ++c) jc[c] = (int)j;
 }

@@ -24,6 +24,13 @@ JFN(jint, dsmult)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong A, jlong Bd
 JFN(jint, dsmultT)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong A, jlong Bdata, jlong Bir, jlong Bic, jlong C) {
     return bidmat_dsmultT(nr, nc, nnz, P(const float, A), P(const float, Bdata), P(const int, Bir), P(const int, Bic), P(float, C));
 }
+// replaces Java_edu_berkeley_bid_CUMAT_dsmultTile (BIDMat_CUMAT.cpp:1456-1471), transpose flag included
+JFN(jint, dsmultTile)(JNIEnv*, jclass, jint nr, jint nc, jint kk, jint nnz, jlong A, jint lda, jlong Bdata, jlong Bir, jlong Bic,
+                      jint broff, jint bcoff, jlong C, jint ldc, jint transpose) {
+    if (transpose)
+        return bidmat_dsmultTileT(nr, nc, kk, nnz, P(const float, A), lda, P(const float, Bdata), P(const int, Bir), P(const int, Bic), broff, bcoff, P(float, C), ldc);
+    return bidmat_dsmultTile(nr, nc, kk, nnz, P(const float, A), lda, P(const float, Bdata), P(const int, Bir), P(const int, Bic), broff, bcoff, P(float, C), ldc);
+}
 // replaces Java_edu_berkeley_bid_CUMAT_dds (BIDMat_CUMAT.cpp:774-785)
 JFN(jint, dds)(JNIEnv*, jclass, jint nr, jint nnz, jlong A, jlong B, jlong Cir, jlong Cic, jlong Pv) {
     return bidmat_dds(nr, nnz, P(const float, A), P(const float, B), P(const int, Cir), P(const int, Cic), P(float, Pv));

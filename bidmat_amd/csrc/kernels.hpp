@@ -28,9 +28,16 @@ hipError_t fingerprint(const int* a, long long na, const int* b, long long nb,
 hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, int** d_ovf,
                                 hipStream_t s);
 
+// A window [off, off+len) on the gather index of the nonzeros (tile variants); on == 0: no filter.
+struct Window { int on, off, len; };
+
 // ---- A*S (spmm.hip)
 hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* vals, const int* ir,
                       const int* jc, float* C, int beta, hipStream_t s);
+// tile form: A and C with their own column strides; only nonzeros with a row inside `rows`
+// take part, rebased to rows.off (jc already points at the first column of the tile).
+hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const float* A, const float* vals,
+                         const int* ir, const int* jc, float* C, int beta, Window rows, hipStream_t s);
 // ---- DDS (dds.hip)
 hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
                    const int* jc, float* P, int beta, hipStream_t s);
@@ -41,9 +48,17 @@ hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, co
 hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A, const float* vals,
                            const int* pc, const int* perm, const int* segstart, float* partial,
                            hipStream_t s);
+// tile form: column stride lda of A; only nonzeros whose column lies in `cols` (rebased), only
+// segments whose row (segrow) lies in `rowsel`.
+hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, const float* A,
+                              const float* vals, const int* pc, const int* perm, const int* segstart,
+                              float* partial, Window cols, const int* segrow, Window rowsel, hipStream_t s);
 // C[:,r] = beta*C[:,r] + sum over q in [rowptr[r], rowptr[r+1]) of partial[rowseg[q]*k ..]
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
                            const float* partial, float* C, int beta, hipStream_t s);
+// tile form: rows [row0, row0+nrows) of the plan go to columns 0.. of C (stride ldc)
+hipError_t reduce_segments_ex(int k, int ldc, int row0, int nrows, const int* rowptr, const int* rowseg,
+                              const float* partial, float* C, int beta, hipStream_t s);
 
 // ---- sums (sums.hip)
 hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, float* out, int beta,

@@ -120,7 +120,7 @@ inline int bits_for(unsigned long long maxval) {
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
     hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->pc, p->perm, p->segstart, p->rowptr, p->rowseg, p->partial};
+    void* bufs[] = {p->pc, p->perm, p->segstart, p->segrow, p->rowptr, p->rowseg, p->partial};
     for (void* b : bufs)
         if (b && (f = hipFree(b)) != hipSuccess) e = f;
     delete p;
@@ -246,18 +246,19 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     PB_CHECK(hipMemcpy(&nseg, segidx.as<int>() + nnz, sizeof(int), hipMemcpyDeviceToHost));
     plan->nseg = nseg;
 
-    DevBuf segrow, segid, segrow_sorted, class_count;
+    DevBuf segid, segrow_sorted, class_count;
     PB_CHECK(class_count.alloc(sizeof(int) * 9));
     PB_CHECK(fill_i32(class_count.as<int>(), 9, 0, s));
-    PB_CHECK(segrow.alloc(sizeof(unsigned) * (size_t)nseg));
+    PB_CHECK(hipMalloc((void**)&plan->segrow, sizeof(int) * (size_t)(nseg > 0 ? nseg : 1)));
+    unsigned* const segrow_u = reinterpret_cast<unsigned*>(plan->segrow);
     PB_CHECK(segid.alloc(sizeof(int) * (size_t)nseg));
     PB_CHECK(segrow_sorted.alloc(sizeof(unsigned) * (size_t)nseg));
     PB_CHECK(hipMalloc((void**)&plan->segstart, sizeof(int) * ((size_t)nseg + 1)));
     PB_CHECK(hipMalloc((void**)&plan->rowseg, sizeof(int) * (size_t)nseg));
-    plan->index_bytes += sizeof(int) * (2 * (size_t)nseg + 1);
+    plan->index_bytes += sizeof(int) * (3 * (size_t)nseg + 1);
     hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out.as<unsigned>(), plan->perm,
                        ic.as<int>(), flag.as<int>(), segidx.as<int>(), hrow.as<int>(), nheavy > 0 ? nheavy : 1,
-                       nheavy > 0 ? p8 : 0, plan->pc, plan->segstart, segrow.as<unsigned>(), segid.as<int>(),
+                       nheavy > 0 ? p8 : 0, plan->pc, plan->segstart, segrow_u, segid.as<int>(),
                        class_count.as<int>());
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
     {
@@ -271,11 +272,11 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     {
         const int rbits = bits_for((unsigned long long)nrows);
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, segrow.as<unsigned>(), segrow_sorted.as<unsigned>(),
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, segrow_u, segrow_sorted.as<unsigned>(),
                                            segid.as<int>(), plan->rowseg, (size_t)nseg, 0, rbits, s));
         DevBuf sorttmp;
         PB_CHECK(sorttmp.alloc(tmp_bytes));
-        PB_CHECK(rocprim::radix_sort_pairs(sorttmp.p, tmp_bytes, segrow.as<unsigned>(), segrow_sorted.as<unsigned>(),
+        PB_CHECK(rocprim::radix_sort_pairs(sorttmp.p, tmp_bytes, segrow_u, segrow_sorted.as<unsigned>(),
                                            segid.as<int>(), plan->rowseg, (size_t)nseg, 0, rbits, s));
         PB_CHECK(coo_compress_cols(nrows, nseg, reinterpret_cast<const int*>(segrow_sorted.as<unsigned>()), plan->rowptr, s));
         PB_CHECK(hipStreamSynchronize(s));

@@ -26,6 +26,7 @@ struct bidmat_plan {
     int* pc = nullptr;       // [nnz]    column of the p-th nonzero in plan order
     int* perm = nullptr;     // [nnz]    its position in the original CSC order
     int* segstart = nullptr; // [nseg+1] segment boundaries in plan order
+    int* segrow = nullptr;   // [nseg]   row of each segment
     int* rowptr = nullptr;   // [nrows+1] range of a row's segments in rowseg
     int* rowseg = nullptr;   // [nseg]   segment ids grouped by row, ascending within a row
     float* partial = nullptr;

@@ -21,7 +21,15 @@ namespace bm {
 namespace {
 
 struct GatherArgs {
-    int k;
+    int k;               // rows of A / of the output that are computed
+    int lda;             // column stride of A
+    int ldo;             // column stride of the output C (partials always use k)
+    int win_on;          // tile mode: only nonzeros whose gather index lies in [win_off, win_off+win_len)
+    int win_off;         //   take part, and the index is rebased to win_off
+    int win_len;
+    const int* segrow;   // tile mode on a plan: row of each segment; segments outside
+    int row_off;         //   [row_off, row_off+row_len) are skipped
+    int row_len;
     int nfirst;          // columns (CSC mode) or segments (plan mode)
     int seglen;
     int beta;
@@ -39,7 +47,7 @@ struct GatherArgs {
 template <int V, int LPN>
 struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw < 1 ? 1 : (raw > LPN ? LPN : raw); };
 
-template <int W, int V, int LPN, bool PLAN, bool FULL>
+template <int W, int V, int LPN, bool PLAN, bool FULL, bool TILE>
 __device__ __forceinline__ void gather_chunk(const GatherArgs& a, int j0, int rem, int g, int l,
                                              const int (&eld)[V], Vec<W> (&acc)[V]) {
     constexpr int NG = 64 / LPN;
@@ -53,6 +61,15 @@ __device__ __forceinline__ void gather_chunk(const GatherArgs& a, int j0, int re
         const int p = j0 + q;
         myrow = a.idx[p];
         myval = PLAN ? a.vals[a.perm[p]] : a.vals[p];
+    }
+    unsigned long long inmask = ~0ULL;
+    if (TILE) {
+        // window filter: nonzeros outside the tile contribute nothing (their lane keeps index 0)
+        const int rr = myrow - a.win_off;
+        const bool inside = (FULL || q < rem) && (unsigned)rr < (unsigned)a.win_len;
+        myrow = inside ? rr : 0;
+        myval = inside ? myval : 0.f;
+        inmask = __ballot(inside);
     }
     const int niter = FULL ? LPN : (rem + NG - 1) / NG;
     for (int it0 = 0; it0 < niter; it0 += U) {
@@ -70,13 +87,14 @@ __device__ __forceinline__ void gather_chunk(const GatherArgs& a, int j0, int re
                 r = lane_read(myrow, src);
                 vv[u] = lane_read(myval, src);
             }
-            const float* ap = a.A + (size_t)r * (size_t)a.k;
+            const float* ap = a.A + (size_t)r * (size_t)a.lda;
 #pragma unroll
             for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
-            if (!FULL) {
-                // past the end of the segment: lane data is (row 0, value 0); drop the load so
-                // that a non-finite entry of A's column 0 cannot leak in as 0*inf.
-                const bool ok = (it * NG + g) < rem;
+            if (!FULL || TILE) {
+                // past the end of the segment (or outside the tile): lane data is (row 0, value 0);
+                // drop the load so that a non-finite entry of A's column 0 cannot leak in as 0*inf.
+                bool ok = FULL || (it * NG + g) < rem;
+                if (TILE) ok = ok && ((inmask >> (LPN == 64 ? it : g * LPN + it)) & 1ULL);
 #pragma unroll
                 for (int i = 0; i < V; ++i) av[u][i] = ok ? av[u][i] : Vec<W>::zero();
             }
@@ -129,6 +147,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
         const int hcount = a.xcd_start[xcd + 1] - hstart;
         const long long seg = wi < hcount ? hstart + wi : a.xcd_start[8] + (wi - hcount) * 8 + xcd;
         if (seg >= a.nfirst) return;
+        if (a.segrow != nullptr && (unsigned)(a.segrow[seg] - a.row_off) >= (unsigned)a.row_len) return;
         jstart = a.ptr[seg];
         jend = a.ptr[seg + 1];
         outp = a.out + (size_t)seg * (size_t)a.k;
@@ -137,7 +156,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
         const int s = a.ptr[w], e = a.ptr[w + 1];
         jstart = s;
         jend = (e - s > a.seglen) ? s + a.seglen : e;
-        outp = a.out + (size_t)w * (size_t)a.k;
+        outp = a.out + (size_t)w * (size_t)a.ldo;
         accumulate = a.beta != 0;
     } else {
         if (a.ovf == nullptr) return;
@@ -169,8 +188,13 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
             acc[i] = Vec<W>::zero();
         }
         int j0 = jstart;
-        for (; j0 + 64 <= jend; j0 += 64) gather_chunk<W, V, LPN, PLAN, true>(a, j0, 64, g, l, eld, acc);
-        if (j0 < jend) gather_chunk<W, V, LPN, PLAN, false>(a, j0, jend - j0, g, l, eld, acc);
+        if (a.win_on) {
+            for (; j0 + 64 <= jend; j0 += 64) gather_chunk<W, V, LPN, PLAN, true, true>(a, j0, 64, g, l, eld, acc);
+            if (j0 < jend) gather_chunk<W, V, LPN, PLAN, false, true>(a, j0, jend - j0, g, l, eld, acc);
+        } else {
+            for (; j0 + 64 <= jend; j0 += 64) gather_chunk<W, V, LPN, PLAN, true, false>(a, j0, 64, g, l, eld, acc);
+            if (j0 < jend) gather_chunk<W, V, LPN, PLAN, false, false>(a, j0, jend - j0, g, l, eld, acc);
+        }
 
 #pragma unroll
         for (int m = LPN; m < 64; m <<= 1) {
@@ -192,7 +216,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
 }
 
 // C[:,c] += sum of the overflow partials of column c, in segment order.
-__global__ __launch_bounds__(BM_BLOCK) void k_overflow_reduce(int k, int ncols, const int* __restrict__ ovf,
+__global__ __launch_bounds__(BM_BLOCK) void k_overflow_reduce(int k, int ldc, int ncols, const int* __restrict__ ovf,
                                                               const float* __restrict__ partial,
                                                               float* __restrict__ C) {
     const int lane = threadIdx.x & 63;
@@ -201,9 +225,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_overflow_reduce(int k, int ncols, 
     const int s = ovf[w], e = ovf[w + 1];
     if (s == e) return;
     for (int el = lane; el < k; el += 64) {
-        float acc = C[(size_t)w * k + el];
+        float acc = C[(size_t)w * ldc + el];
         for (int q = s; q < e; ++q) acc += partial[(size_t)q * k + el];
-        C[(size_t)w * k + el] = acc;
+        C[(size_t)w * ldc + el] = acc;
     }
 }
 
@@ -216,8 +240,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_extra_segments(int ncols, const in
 }
 
 // Plan stage 2: rows handled by groups of LPR lanes.
+// Rows [row0, row0+nrows) of the plan; output column (row - row0) of C with stride ldc.
 template <int W>
-__global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int nrows, int lpr,
+__global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int ldc, int row0, int nrows, int lpr,
                                                               const int* __restrict__ rowptr,
                                                               const int* __restrict__ rowseg,
                                                               const float* __restrict__ partial,
@@ -226,9 +251,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int nrows, 
     const long long row = t / lpr;
     const int l = (int)(t % lpr);
     if (row >= nrows) return;
-    const int s = rowptr[row], e = rowptr[row + 1];
+    const int s = rowptr[row0 + row], e = rowptr[row0 + row + 1];
     for (int el = l * W; el < k; el += lpr * W) {
-        float* o = C + (size_t)row * k + el;
+        float* o = C + (size_t)row * ldc + el;
         Vec<W> acc = beta ? Vec<W>::load(o) : Vec<W>::zero();
         for (int q = s; q < e; ++q) acc.add(Vec<W>::load(partial + (size_t)rowseg[q] * k + el));
         acc.store(o);
@@ -284,8 +309,21 @@ hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, i
     return hipGetLastError();
 }
 
+namespace {
+void init_args(GatherArgs& a) {
+    a.win_on = 0; a.win_off = 0; a.win_len = 0;
+    a.segrow = nullptr; a.row_off = 0; a.row_len = 0;
+    for (int x = 0; x < 9; ++x) a.xcd_start[x] = 0;
+}
+}  // namespace
+
 hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* vals, const int* ir,
                       const int* jc, float* C, int beta, hipStream_t s) {
+    return dsmult_csc_ex(k, k, k, ncols, nnz, A, vals, ir, jc, C, beta, Window{0, 0, 0}, s);
+}
+
+hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const float* A, const float* vals,
+                         const int* ir, const int* jc, float* C, int beta, Window rows, hipStream_t s) {
     if (k <= 0 || ncols <= 0) return hipSuccess;
     const int seglen = opt_seglen();
     int* ovf = nullptr;
@@ -298,17 +336,19 @@ hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* va
         partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err);
         if (!partial) return err;
     }
-    Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(C) && aligned16(partial)));
+    const bool al = aligned16(A) && aligned16(C) && aligned16(partial) && lda % 4 == 0 && ldc % 4 == 0;
+    Shape sh = clamp_shape(pick_shape(k, al));
     GatherArgs a;
-    a.k = k; a.nfirst = ncols; a.seglen = seglen; a.beta = beta;
+    init_args(a);
+    a.k = k; a.lda = lda; a.ldo = ldc; a.nfirst = ncols; a.seglen = seglen; a.beta = beta;
     a.A = A; a.vals = vals; a.idx = ir; a.perm = nullptr; a.ptr = jc; a.ovf = ovf;
     a.out = C; a.partial = partial;
-    for (int x = 0; x < 9; ++x) a.xcd_start[x] = 0;
+    a.win_on = rows.on; a.win_off = rows.off; a.win_len = rows.len;
     err = launch_gather<false>(sh, a, (long long)ncols + novf_max, s);
     if (err != hipSuccess) return err;
     if (ovf) {
         unsigned nblk = (unsigned)(((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK);
-        hipLaunchKernelGGL(k_overflow_reduce, dim3(nblk), dim3(BM_BLOCK), 0, s, k, ncols, ovf, partial, C);
+        hipLaunchKernelGGL(k_overflow_reduce, dim3(nblk), dim3(BM_BLOCK), 0, s, k, ldc, ncols, ovf, partial, C);
         err = hipGetLastError();
     }
     return err;
@@ -317,12 +357,22 @@ hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* va
 hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A, const float* vals,
                            const int* pc, const int* perm, const int* segstart, float* partial,
                            hipStream_t s) {
+    return gather_segments_ex(k, k, nseg, xcd_start, A, vals, pc, perm, segstart, partial,
+                              Window{0, 0, 0}, nullptr, Window{0, 0, 0}, s);
+}
+
+hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, const float* A,
+                              const float* vals, const int* pc, const int* perm, const int* segstart,
+                              float* partial, Window cols, const int* segrow, Window rowsel, hipStream_t s) {
     if (k <= 0 || nseg <= 0) return hipSuccess;
-    Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(partial)));
+    Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(partial) && lda % 4 == 0));
     GatherArgs a;
-    a.k = k; a.nfirst = nseg; a.seglen = 0; a.beta = 0;
+    init_args(a);
+    a.k = k; a.lda = lda; a.ldo = k; a.nfirst = nseg; a.seglen = 0; a.beta = 0;
     a.A = A; a.vals = vals; a.idx = pc; a.perm = perm; a.ptr = segstart; a.ovf = nullptr;
     a.out = partial; a.partial = nullptr;
+    a.win_on = cols.on; a.win_off = cols.off; a.win_len = cols.len;
+    if (rowsel.on) { a.segrow = segrow; a.row_off = rowsel.off; a.row_len = rowsel.len; }
     int maxheavy = 0;
     for (int x = 0; x < 9; ++x) a.xcd_start[x] = xcd_start[x];
     for (int x = 0; x < 8; ++x) maxheavy = std::max(maxheavy, xcd_start[x + 1] - xcd_start[x]);
@@ -335,16 +385,21 @@ hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A
 
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
                            const float* partial, float* C, int beta, hipStream_t s) {
+    return reduce_segments_ex(k, k, 0, nrows, rowptr, rowseg, partial, C, beta, s);
+}
+
+hipError_t reduce_segments_ex(int k, int ldc, int row0, int nrows, const int* rowptr, const int* rowseg,
+                              const float* partial, float* C, int beta, hipStream_t s) {
     if (k <= 0 || nrows <= 0) return hipSuccess;
-    const bool al = aligned16(C) && aligned16(partial) && (k % 4 == 0);
+    const bool al = aligned16(C) && aligned16(partial) && (k % 4 == 0) && (ldc % 4 == 0);
     const int W = al ? 4 : 1;
     int nv = (k + W - 1) / W;
     int lpr = pow2ceil(nv) < 64 ? pow2ceil(nv) : 64;
     long long threads = (long long)nrows * lpr;
     long long nblk = (threads + BM_BLOCK - 1) / BM_BLOCK;
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (al) hipLaunchKernelGGL(k_reduce_segments<4>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, nrows, lpr, rowptr, rowseg, partial, C, beta);
-    else hipLaunchKernelGGL(k_reduce_segments<1>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, nrows, lpr, rowptr, rowseg, partial, C, beta);
+    if (al) hipLaunchKernelGGL(k_reduce_segments<4>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, ldc, row0, nrows, lpr, rowptr, rowseg, partial, C, beta);
+    else hipLaunchKernelGGL(k_reduce_segments<1>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, ldc, row0, nrows, lpr, rowptr, rowseg, partial, C, beta);
     return hipGetLastError();
 }
 

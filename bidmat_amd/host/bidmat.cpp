@@ -222,6 +222,34 @@ GMatP GMat::maddT(const GSMatP& a, GMatP out) {
     return out;
 }
 
+GMatP GMat::tileMult(int nr, int nc, int kk, int aroff, int acoff, const GSMatP& b, int broff, int bcoff,
+                     GMatP c, int croff, int ccoff) {
+    if (aroff < 0 || acoff < 0 || broff < 0 || bcoff < 0 || croff < 0 || ccoff < 0 || nr < 0 || nc < 0 || kk < 0)
+        fail("tileMult: cant have negative offsets or dimensions");
+    if (aroff + nr > nrows || acoff + kk > ncols || broff + kk > b->nrows || bcoff + nc > b->ncols ||
+        croff + nr > c->nrows || ccoff + nc > c->ncols)
+        fail("tileMult: tile strays outside matrix dimensions");
+    Mat::nflops += 2LL * nr * b->nnz();
+    int err = bidmat_dsmultTile(nr, nc, kk, b->nnz(), pdata + (aroff + (long long)acoff * nrows), nrows, b->pdata,
+                                b->pir, b->pic, broff, bcoff, c->pdata + (croff + (long long)ccoff * c->nrows), c->nrows);
+    if (err != 0) fail(std::string("tileMult error ") + bidmat_error_string(err));
+    return c;
+}
+
+GMatP GMat::tileMultNT(int nr, int nc, int kk, int aroff, int acoff, const GSMatP& b, int broff, int bcoff,
+                       GMatP c, int croff, int ccoff) {
+    if (aroff < 0 || acoff < 0 || broff < 0 || bcoff < 0 || croff < 0 || ccoff < 0 || nr < 0 || nc < 0 || kk < 0)
+        fail("tileMultNT: cant have negative offsets or dimensions");
+    if (aroff + nr > nrows || acoff + kk > ncols || broff + nc > b->nrows || bcoff + kk > b->ncols ||
+        croff + nr > c->nrows || ccoff + nc > c->ncols)
+        fail("tileMultNT: tile strays outside matrix dimensions");
+    Mat::nflops += 2LL * nr * b->nnz() * kk / std::max(1, b->ncols);
+    int err = bidmat_dsmultTileT(nr, nc, kk, b->nnz(), pdata + (aroff + (long long)acoff * nrows), nrows, b->pdata,
+                                 b->pir, b->pic, broff, bcoff, c->pdata + (croff + (long long)ccoff * c->nrows), c->nrows);
+    if (err != 0) fail(std::string("tileMultT error ") + bidmat_error_string(err));
+    return c;
+}
+
 GMatP GMat::gOp(const GMatP& a, GMatP oldmat, int op) {
     // compatible shapes (ND.compatibleGDims for the 2-D case): equal, or a row/column/scalar on either side
     const int nr = std::max(nrows, a->nrows), nc = std::max(ncols, a->ncols);

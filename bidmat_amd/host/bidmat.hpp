@@ -97,6 +97,11 @@ public:
     // C = this *^ S and C += this *^ S
     GMatP GSMultT(const GSMatP& a, GMatP oldmat);
     GMatP maddT(const GSMatP& a, GMatP out);
+    // windowed products for tiled matrices (GMat.scala:961-997): c[croff.., ccoff..] += this[aroff.., acoff..] * b[broff.., bcoff..]
+    GMatP tileMult(int nr, int nc, int kk, int aroff, int acoff, const GSMatP& b, int broff, int bcoff,
+                   GMatP c, int croff, int ccoff);
+    GMatP tileMultNT(int nr, int nc, int kk, int aroff, int acoff, const GSMatP& b, int broff, int bcoff,
+                     GMatP c, int croff, int ccoff);
     // elementwise binary op with broadcasting, reductions
     GMatP gOp(const GMatP& a, GMatP oldmat, int op);
     GMatP reduceOp(GMatP oldmat, int dir, float initval, int op);

@@ -81,6 +81,13 @@ API void* bmh_mult(void* a, void* s, void* out) { return guard_ptr([&] { return 
 API void* bmh_madd(void* a, void* s, void* out) { return guard_ptr([&] { return wrap(G(a)->madd(S(s), G(out))); }); }
 API void* bmh_multT(void* a, void* s, void* out) { return guard_ptr([&] { return wrap(G(a)->GSMultT(S(s), G(out))); }); }
 API void* bmh_maddT(void* a, void* s, void* out) { return guard_ptr([&] { return wrap(G(a)->maddT(S(s), G(out))); }); }
+API void* bmh_tile_mult(void* a, int nr, int nc, int kk, int aroff, int acoff, void* b, int broff, int bcoff,
+                        void* c, int croff, int ccoff, int transposed) {
+    return guard_ptr([&] {
+        return wrap(transposed ? G(a)->tileMultNT(nr, nc, kk, aroff, acoff, S(b), broff, bcoff, G(c), croff, ccoff)
+                               : G(a)->tileMult(nr, nc, kk, aroff, acoff, S(b), broff, bcoff, G(c), croff, ccoff));
+    });
+}
 API void* bmh_dds(void* a, void* b, void* c, void* out) {
     return guard_ptr([&] { return wrap(GSMat::DDS(G(a), G(b), S(c), S(out))); });
 }

@@ -31,7 +31,7 @@ def _load():
         L = C.CDLL(LIB_PATH)
         for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
                      "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
-                     "bmh_gop", "bmh_contents", "bmh_with_values"):
+                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult"):
             getattr(L, name).restype = vp
         L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
         L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
@@ -39,6 +39,7 @@ def _load():
         for name in ("bmh_mult", "bmh_madd", "bmh_multT", "bmh_maddT"):
             getattr(L, name).argtypes = [vp, vp, vp]
         L.bmh_dds.argtypes = [vp, vp, vp, vp]
+        L.bmh_tile_mult.argtypes = [vp] + [C.c_int] * 5 + [vp, C.c_int, C.c_int, vp, C.c_int, C.c_int, C.c_int]
         L.bmh_sum_sparse.argtypes = [vp, C.c_int, vp]
         L.bmh_sum_dense.argtypes = [vp, C.c_int, vp]
         L.bmh_reduce.argtypes = [vp, vp, C.c_int, C.c_float, C.c_int]
@@ -173,6 +174,12 @@ class GMat(_Handle):
 
     def maddT(self, s, out):
         return GMat(_load().bmh_maddT(self._h, s._h, out._h))
+
+    def tileMult(self, nr, nc, kk, aroff, acoff, b, broff, bcoff, c, croff, ccoff):
+        return GMat(_load().bmh_tile_mult(self._h, nr, nc, kk, aroff, acoff, b._h, broff, bcoff, c._h, croff, ccoff, 0))
+
+    def tileMultNT(self, nr, nc, kk, aroff, acoff, b, broff, bcoff, c, croff, ccoff):
+        return GMat(_load().bmh_tile_mult(self._h, nr, nc, kk, aroff, acoff, b._h, broff, bcoff, c._h, croff, ccoff, 1))
 
     def gOp(self, b, op, out=None):
         return GMat(_load().bmh_gop(self._h, b._h, out._h if out else None, op))

@@ -54,6 +54,18 @@ int bidmat_dsmult(int nrows, int ncols, int nnz, const float *A, const float *Bd
 int bidmat_dsmultT(int nrows, int ncols, int nnz, const float *A, const float *Bdata,
                    const int *Bir, const int *Bic, float *C);
 
+/* Windowed products used by tiled matrices (TMat).
+ * bidmat_dsmultTile:  C[0:nr,0:nc] += A[0:nr,0:kk] * S[broff:broff+kk, bcoff:bcoff+nc]
+ * bidmat_dsmultTileT: C[0:nr,0:nc] += A[0:nr,0:kk] * S[broff:broff+nc, bcoff:bcoff+kk]^T
+ * A and C are windows of larger matrices: lda / ldc are their column strides.  Replace
+ * `int dsmultTile(int nr,int nc,int kk,int nnz,float*A,int lda,float*Bdata,int*Bir,int*Bic,int broff,
+ * int bcoff,float*C,int ldc)` and `dsmultTileT` (Arith.cu:63-189, MatKernel.hpp:142-144; Java stub
+ * CUMAT.java:145 with its transpose flag; callers GMat.tileMult / tileMultNT, GMat.scala:961-997). */
+int bidmat_dsmultTile(int nr, int nc, int kk, int nnz, const float *A, int lda, const float *Bdata,
+                      const int *Bir, const int *Bic, int broff, int bcoff, float *C, int ldc);
+int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float *A, int lda, const float *Bdata,
+                       const int *Bir, const int *Bic, int broff, int bcoff, float *C, int ldc);
+
 /* P[j] += dot(A[:,Cir[j]], B[:,Cic[j]]).  Replaces `int dds(int nrows,int nnz,float*A,float*B,
  * int*Cir,int*Cic,float*P)` (Arith.cu:381-389; CUMAT.java:211; caller GSMat.scala:663). */
 int bidmat_dds(int nrows, int nnz, const float *A, const float *B, const int *Cir,

@@ -35,6 +35,10 @@ def lib():
         L.oracle_smcsrm.argtypes = [i, i, vp, i, vp, vp, vp, vp, i]
         L.oracle_fsmultT.argtypes = [i, i, vp, vp, vp, vp, i, vp, i]
         L.oracle_fsmultT_f64.argtypes = [i, i, vp, vp, vp, vp, i, vp, vp, i]
+        L.oracle_fsmult_tile.argtypes = [i, i, i, vp, i, vp, vp, vp, i, i, i, vp, i, vp, vp, i]
+        L.oracle_fsmult_tileT.argtypes = [i, i, i, vp, i, vp, vp, vp, i, i, i, vp, i, vp, vp]
+        L.oracle_fsmult_tile.restype = None
+        L.oracle_fsmult_tileT.restype = None
         L.oracle_dds.argtypes = [i, i, vp, vp, vp, vp, i, vp, vp, vp, i]
         L.oracle_dds_f64.argtypes = [i, i, vp, vp, vp, vp, i, vp, vp, i]
         L.oracle_spsum.argtypes = [i, i, vp, vp, vp, i, i, vp]
@@ -116,6 +120,25 @@ def fsmultT_f64(A, k, nrowsS, data, ir, jc, ioff=0, nthreads=1):
     sa = np.zeros(k * nrowsS, dtype=np.float64)
     lib().oracle_fsmultT_f64(k, ncols, A.ctypes.data, data.ctypes.data, ir.ctypes.data, jc.ctypes.data, ioff,
                              ref.ctypes.data, sa.ctypes.data, nthreads)
+    return ref, sa
+
+
+def fsmult_tile(Aparent, anrows, aroff, acoff, nr, nc, kk, data, ir, jc, broff, bcoff, Cparent, cnrows, croff,
+                ccoff, ioff=0, transposed=False, nthreads=1):
+    """tileMult / tileMultNT on flattened column-major parents. Adds into Cparent (float32, in
+    place) and returns (ref64, sumabs) of the product alone as nr x nc column-major arrays."""
+    Aparent, data, ir, jc = _f32(Aparent), _f32(data), _i32(ir), _i32(jc)
+    assert Cparent.dtype == np.float32 and Cparent.flags.c_contiguous
+    ref = np.zeros(nr * nc, dtype=np.float64)
+    sa = np.zeros(nr * nc, dtype=np.float64)
+    ap = Aparent.ctypes.data + 4 * (aroff + acoff * anrows)
+    cp = Cparent.ctypes.data + 4 * (croff + ccoff * cnrows)
+    if transposed:
+        lib().oracle_fsmult_tileT(nr, nc, kk, ap, anrows, data.ctypes.data, ir.ctypes.data, jc.ctypes.data, ioff,
+                                  broff, bcoff, cp, cnrows, ref.ctypes.data, sa.ctypes.data)
+    else:
+        lib().oracle_fsmult_tile(nr, nc, kk, ap, anrows, data.ctypes.data, ir.ctypes.data, jc.ctypes.data, ioff,
+                                 broff, bcoff, cp, cnrows, ref.ctypes.data, sa.ctypes.data, nthreads)
     return ref, sa
 
 

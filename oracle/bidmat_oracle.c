@@ -20,6 +20,7 @@
  *   oracle_smcscm / oracle_fsmult     dense GEMM A*full(S) in numpy fp64, scipy csc product,
  *                                     one-hot gather (bit-exact), identity, golden fixtures
  *   oracle_smcsrm / oracle_fsmultT    A*full(S)^T in fp64, np.add.at, transpose identity, fixtures
+ *   oracle_fsmult_tile / _tileT       dense products of numpy windows A[a:b,c:d] @ full(S)[e:f,g:h](^T)
  *   oracle_dds                        closed form dot(A[:,r],B[:,c]); dense pattern == A^T B; fixtures
  *   oracle_spsum                      np.bincount / np.add.reduceat; sum of col sums == sum of row sums
  *   oracle_dsum                       numpy sum along axis
@@ -186,6 +187,70 @@ EXPORT void oracle_fsmultT_f64(int nrows, int ncols, const float *A, const float
                     double t = (double)A[k + (size_t)i * nrows] * dval;
                     if (ref) ref[k + ival * nrows] += t;
                     if (sumabs) sumabs[k + ival * nrows] += fabs(t);
+                }
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------ tile variants */
+
+/* C[0:nr,0:nc] += A[0:nr,0:kk] * S[broff:broff+kk, bcoff:bcoff+nc] on windows of larger
+ * matrices.  Follows FMat.scala:1200-1223 (fSMultHelperTile): columns bcoff..bcoff+nc of S,
+ * nonzeros in stored order, rows outside [broff, broff+kk) skipped, row rebased to broff.
+ * A / C point at the first element of their windows; lda / ldc are the parents' row counts.
+ * Threads over column ranges as FMat.scala:1260-1270.  ref/sumabs (double, nr x nc with
+ * leading dimension nr) are optional fp64 arbiters of the product alone. */
+EXPORT void oracle_fsmult_tile(int nr, int nc, int kk, const float *A, int lda, const float *data,
+                               const int *ir, const int *jc, int ioff, int broff, int bcoff,
+                               float *C, int ldc, double *ref, double *sumabs, int nthreads)
+{
+    int i;
+    if (nthreads < 1) nthreads = 1;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (i = 0; i < nc; i++) {
+        int j, k;
+        for (j = jc[i + bcoff] - ioff; j < jc[i + bcoff + 1] - ioff; j++) {
+            int irow0 = ir[j] - ioff;
+            if (irow0 >= broff && irow0 < broff + kk) {
+                size_t irow = (size_t)(irow0 - broff);
+                float dval = data[j];
+                for (k = 0; k < nr; k++) {
+                    if (C) C[k + (size_t)i * ldc] += A[k + irow * lda] * dval;
+                    if (ref) {
+                        double t = (double)A[k + irow * lda] * (double)dval;
+                        ref[k + (size_t)i * nr] += t;
+                        if (sumabs) sumabs[k + (size_t)i * nr] += fabs(t);
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* C[0:nr,0:nc] += A[0:nr,0:kk] * S[broff:broff+nc, bcoff:bcoff+kk]^T.  Follows
+ * FMat.scala:1225-1248 (fSMultHelperTileT): columns bcoff..bcoff+kk of S, rows outside
+ * [broff, broff+nc) skipped, C[:,row-broff] += A[:,i]*v.  Single thread here: the
+ * reference's own column-range threading of this scatter (FMat.scala:1286-1296) lets two
+ * threads add into the same output column at once. */
+EXPORT void oracle_fsmult_tileT(int nr, int nc, int kk, const float *A, int lda, const float *data,
+                                const int *ir, const int *jc, int ioff, int broff, int bcoff,
+                                float *C, int ldc, double *ref, double *sumabs)
+{
+    int i, j, k;
+    for (i = 0; i < kk; i++) {
+        for (j = jc[i + bcoff] - ioff; j < jc[i + bcoff + 1] - ioff; j++) {
+            int irow0 = ir[j] - ioff;
+            if (irow0 >= broff && irow0 < broff + nc) {
+                size_t irow = (size_t)(irow0 - broff);
+                float dval = data[j];
+                for (k = 0; k < nr; k++) {
+                    if (C) C[k + irow * ldc] += A[k + (size_t)i * lda] * dval;
+                    if (ref) {
+                        double t = (double)A[k + (size_t)i * lda] * (double)dval;
+                        ref[k + irow * nr] += t;
+                        if (sumabs) sumabs[k + irow * nr] += fabs(t);
+                    }
                 }
             }
         }

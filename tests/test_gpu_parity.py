@@ -491,3 +491,69 @@ def test_argument_validation(hip):
     p = C.c_void_p()
     assert hip.bidmat_plan_create(10, 2, 3, e.ir.ptr, e.jc.ptr, 0, C.byref(p)) == 1
     e.free(), d.free()
+
+
+# ------------------------------------------------------------------------------ tile variants
+@pytest.mark.parametrize("nr", [5, 32, 64, 256, 300])
+@pytest.mark.parametrize("transposed", [False, True])
+def test_dsmult_tile(hip, nr, transposed):
+    """bidmat_dsmultTile / TileT: windows of A, S and C with their parents' strides, aligned
+    and unaligned window origins, accumulate into C, nothing outside the tile touched."""
+    rng = np.random.default_rng(400 + nr + int(transposed))
+    snr, snc = 90, 70
+    lengths = rng.integers(0, 25, size=snc)
+    lengths[11] = 0
+    data, ir, jc = random_csc(rng, snr, snc, lengths=lengths, sort_rows=False)
+    ir[(ir > 2) & (rng.random(ir.size) < 0.3)] = 1          # a heavy row
+    ic = expand_cols(jc)
+    old_seg, old_panel = opt(hip, "seglen", 64), opt(hip, "panel_kb", 16)
+    try:
+        for (aroff, croff) in ((0, 0), (3, 5), (4, 8)):
+            anr, cnr = nr + aroff + 2, nr + croff + 3
+            if transposed:
+                nc, kk, broff, bcoff = 40, 33, 17, 9          # rows 17..56 of S, columns 9..41
+            else:
+                nc, kk, broff, bcoff = 29, 50, 13, 21         # rows 13..62 of S, columns 21..49
+            acoff, ccoff = 2, 1
+            anc, cnc = kk + acoff + 1, nc + ccoff + 2
+            A = rng.standard_normal(anr * anc).astype(np.float32)
+            C0 = rng.standard_normal(cnr * cnc).astype(np.float32)
+            d = Dev(A=A, data=data, ir=ir, ic=ic, Cm=C0)
+            fn = hip.bidmat_dsmultTileT if transposed else hip.bidmat_dsmultTile
+            hip_abi.check(fn(nr, nc, kk, ir.size, d.A.ptr + 4 * (aroff + acoff * anr), anr, d.data.ptr, d.ir.ptr,
+                             d.ic.ptr, broff, bcoff, d.Cm.ptr + 4 * (croff + ccoff * cnr), cnr))
+            got = d.Cm.numpy().reshape(cnc, cnr).T
+            Cref = C0.copy()
+            ref64, sa = oracle.fsmult_tile(A, anr, aroff, acoff, nr, nc, kk, data, ir, jc, broff, bcoff, Cref, cnr,
+                                           croff, ccoff, transposed=transposed)
+            c0 = C0.reshape(cnc, cnr).T
+            win = (slice(croff, croff + nr), slice(ccoff, ccoff + nc))
+            want = ref64.reshape(nc, nr).T + c0[win]
+            assert_close(got[win].ravel(), want.ravel(), (sa.reshape(nc, nr).T + np.abs(c0[win])).ravel(),
+                         "tile nr=%d T=%s off=%d" % (nr, transposed, aroff))
+            assert_close(Cref.reshape(cnc, cnr).T[win].ravel(), want.ravel(),
+                         (sa.reshape(nc, nr).T + np.abs(c0[win])).ravel(), "oracle fp32 tile")
+            mask = np.ones_like(got, dtype=bool)
+            mask[win] = False
+            assert np.array_equal(got[mask], c0[mask])            # outside the tile: untouched
+            d.free()
+    finally:
+        opt(hip, "seglen", old_seg), opt(hip, "panel_kb", old_panel)
+
+
+def test_dsmult_tile_whole_matrix_equals_plain_product(hip):
+    rng = np.random.default_rng(450)
+    k, nrows, ncols = 64, 200, 300
+    data, ir, jc = random_csc(rng, nrows, ncols, 0.05)
+    ic = expand_cols(jc)
+    A = rng.standard_normal(k * nrows).astype(np.float32)
+    B = rng.standard_normal(k * ncols).astype(np.float32)
+    d = Dev(A=A, B=B, data=data, ir=ir, ic=ic)
+    d.zeros("C1", k * ncols), d.zeros("C2", k * ncols), d.zeros("G1", k * nrows), d.zeros("G2", k * nrows)
+    hip_abi.check(hip.bidmat_dsmult(k, ncols, ir.size, d.A.ptr, d.data.ptr, d.ir.ptr, d.ic.ptr, d.C1.ptr))
+    hip_abi.check(hip.bidmat_dsmultTile(k, ncols, nrows, ir.size, d.A.ptr, k, d.data.ptr, d.ir.ptr, d.ic.ptr, 0, 0, d.C2.ptr, k))
+    assert np.array_equal(d.C1.numpy(), d.C2.numpy())
+    hip_abi.check(hip.bidmat_dsmultT(k, ncols, ir.size, d.B.ptr, d.data.ptr, d.ir.ptr, d.ic.ptr, d.G1.ptr))
+    hip_abi.check(hip.bidmat_dsmultTileT(k, nrows, ncols, ir.size, d.B.ptr, k, d.data.ptr, d.ir.ptr, d.ic.ptr, 0, 0, d.G2.ptr, k))
+    assert np.array_equal(d.G1.numpy(), d.G2.numpy())
+    d.free()

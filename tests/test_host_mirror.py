@@ -249,3 +249,31 @@ def test_flip_gflop_accounting(hip):
     aa * ss
     g, secs = mats.gflop()
     assert secs > 0 and g == pytest.approx(2 * 64 * s[0].size / secs / 1e9, rel=0.2)
+
+
+@gpu
+def test_tile_mult_and_messages(hip):
+    """GMat.tileMult / tileMultNT (GMat.scala:961-997): windows, argument checks, messages."""
+    rng = np.random.default_rng(13)
+    a = rng.random((12, 40)).astype(np.float32)
+    s = sprand(rng, 35, 30, 0.3)
+    c0 = rng.random((15, 33)).astype(np.float32)
+    aa, ss = GMat.from_numpy(a), GSMat.from_csc(35, 30, *s)
+    S = full(35, 30, *s)
+    cc = GMat.from_numpy(c0)
+    out = aa.tileMult(7, 9, 11, 3, 5, ss, 6, 4, cc, 2, 8)
+    assert out.same(cc)
+    want = c0.astype(np.float64).copy()
+    want[2:9, 8:17] += a.astype(np.float64)[3:10, 5:16] @ S[6:17, 4:13]
+    np.testing.assert_allclose(cc.numpy(), want, rtol=0, atol=EPS)
+    cc = GMat.from_numpy(c0)
+    aa.tileMultNT(6, 10, 8, 1, 7, ss, 5, 9, cc, 4, 3)
+    want = c0.astype(np.float64).copy()
+    want[4:10, 3:13] += a.astype(np.float64)[1:7, 7:15] @ S[5:15, 9:17].T
+    np.testing.assert_allclose(cc.numpy(), want, rtol=0, atol=EPS)
+    with pytest.raises(RuntimeError, match="tileMult: cant have negative offsets or dimensions"):
+        aa.tileMult(7, 9, 11, -1, 5, ss, 6, 4, cc, 2, 8)
+    with pytest.raises(RuntimeError, match="tileMult: tile strays outside matrix dimensions"):
+        aa.tileMult(7, 9, 11, 3, 5, ss, 30, 4, cc, 2, 8)
+    with pytest.raises(RuntimeError, match="tileMultNT: tile strays outside matrix dimensions"):
+        aa.tileMultNT(6, 10, 8, 1, 7, ss, 5, 25, cc, 4, 3)

@@ -266,3 +266,41 @@ def test_tolerance_rule():
     assert oracle.within_tolerance(ref + np.array([5e-5, 5e-4, 5e-4]), ref, sa)[0]      # cancellation-safe
     assert not oracle.within_tolerance(ref + np.array([5e-4, 0, 0]), ref, sa)[0]
     assert not oracle.within_tolerance(np.array([np.nan, 0, 0]), ref, sa)[0]
+
+
+def test_tile_products_against_dense_windows():
+    """tileMult / tileMultNT (FMat.scala:1200-1303): windows of A, S and C."""
+    rng = np.random.default_rng(11)
+    anr, anc, snr, snc, cnr, cnc = 12, 40, 35, 30, 15, 33
+    A = rng.standard_normal(anr * anc).astype(np.float32)
+    data, ir, jc = random_csc(rng, snr, snc, 0.3)
+    S = dense_full(snr, snc, data, ir, jc)
+    A2 = A.reshape(anc, anr).T.astype(np.float64)
+    for ioff in (0, 1):
+        # C[croff:+nr, ccoff:+nc] += A[aroff:+nr, acoff:+kk] * S[broff:+kk, bcoff:+nc]
+        nr, nc, kk, aroff, acoff, broff, bcoff, croff, ccoff = 7, 9, 11, 3, 5, 6, 4, 2, 8
+        C0 = rng.standard_normal(cnr * cnc).astype(np.float32)
+        Cm = C0.copy()
+        ref, sa = oracle.fsmult_tile(A, anr, aroff, acoff, nr, nc, kk, data, ir + ioff, jc + ioff, broff, bcoff,
+                                     Cm, cnr, croff, ccoff, ioff=ioff)
+        want = A2[aroff:aroff + nr, acoff:acoff + kk] @ S[broff:broff + kk, bcoff:bcoff + nc]
+        np.testing.assert_allclose(ref.reshape(nc, nr).T, want, rtol=1e-12, atol=1e-12)
+        full_want = C0.reshape(cnc, cnr).T.astype(np.float64).copy()
+        full_want[croff:croff + nr, ccoff:ccoff + nc] += want
+        np.testing.assert_allclose(Cm.reshape(cnc, cnr).T, full_want, rtol=1e-5, atol=1e-5)   # nothing outside the tile moved
+        # C[.., ccoff:+nc] += A[aroff:+nr, acoff:+kk] * S[broff:+nc, bcoff:+kk]^T
+        nr, nc, kk, aroff, acoff, broff, bcoff, croff, ccoff = 6, 10, 8, 1, 7, 5, 9, 4, 3
+        Cm = C0.copy()
+        ref, sa = oracle.fsmult_tile(A, anr, aroff, acoff, nr, nc, kk, data, ir + ioff, jc + ioff, broff, bcoff,
+                                     Cm, cnr, croff, ccoff, ioff=ioff, transposed=True)
+        want = A2[aroff:aroff + nr, acoff:acoff + kk] @ S[broff:broff + nc, bcoff:bcoff + kk].T
+        np.testing.assert_allclose(ref.reshape(nc, nr).T, want, rtol=1e-12, atol=1e-12)
+        full_want = C0.reshape(cnc, cnr).T.astype(np.float64).copy()
+        full_want[croff:croff + nr, ccoff:ccoff + nc] += want
+        np.testing.assert_allclose(Cm.reshape(cnc, cnr).T, full_want, rtol=1e-5, atol=1e-5)
+    # a tile that covers everything is the plain product, bit for bit
+    k = 5
+    Af = rng.standard_normal(k * snr).astype(np.float32)
+    Cm = np.zeros(k * snc, dtype=np.float32)
+    oracle.fsmult_tile(Af, k, 0, 0, k, snc, snr, data, ir, jc, 0, 0, Cm, k, 0, 0)
+    assert np.array_equal(Cm, oracle.fsmult(Af, k, data, ir, jc))
