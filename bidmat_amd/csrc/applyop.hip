@@ -56,6 +56,27 @@ __global__ __launch_bounds__(BM_BLOCK) void k_apply_full4(const float4* __restri
     }
 }
 
+// Dense transpose through a padded LDS tile: in is nrows x ncols (column-major, leading dimension
+// ldi), out is ncols x nrows (leading dimension ldo). Reads and writes are both coalesced.
+constexpr int TT = 32;
+__global__ __launch_bounds__(BM_BLOCK) void k_transpose(int nrows, int ncols, const float* __restrict__ in, int ldi,
+                                                        float* __restrict__ out, int ldo) {
+    __shared__ float tile[TT][TT + 1];
+    const int tx = threadIdx.x & (TT - 1), ty = threadIdx.x / TT;     // 32 x 8 threads
+    const long long r0 = (long long)blockIdx.x * TT, c0 = (long long)blockIdx.y * TT;
+#pragma unroll
+    for (int j = ty; j < TT; j += BM_BLOCK / TT) {
+        const long long r = r0 + tx, c = c0 + j;
+        if (r < nrows && c < ncols) tile[j][tx] = in[(size_t)c * ldi + r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = ty; j < TT; j += BM_BLOCK / TT) {
+        const long long c = c0 + tx, r = r0 + j;                      // out[c, r] = in[r, c]
+        if (r < nrows && c < ncols) out[(size_t)r * ldo + c] = tile[tx][j];
+    }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 inline unsigned grid_for(long long n) {
@@ -93,6 +114,23 @@ hipError_t apply_impl(const float* A, int ma, const float* B, int mb, float* C, 
 }
 
 }  // namespace
+
+hipError_t transpose(int nrows, int ncols, const float* in, int ldi, float* out, int ldo, hipStream_t s) {
+    if (nrows <= 0 || ncols <= 0) return hipSuccess;
+    const long long bx = ((long long)nrows + TT - 1) / TT, by = ((long long)ncols + TT - 1) / TT;
+    if (by > 65535) {
+        // very wide inputs: walk the columns in slabs the grid's y dimension can hold
+        const int slab = 65535 * TT;
+        for (long long c = 0; c < ncols; c += slab) {
+            const int nc = (int)((ncols - c) < slab ? (ncols - c) : slab);
+            hipError_t e = transpose(nrows, nc, in + (size_t)c * ldi, ldi, out + c, ldo, s);
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(k_transpose, dim3((unsigned)bx, (unsigned)by), dim3(BM_BLOCK), 0, s, nrows, ncols, in, ldi, out, ldo);
+    return hipGetLastError();
+}
 
 // Same case analysis, in the same order, as apply_binop (Operators.cu:529-553).
 hipError_t applyop(const float* A, int Anr, int Anc, const float* B, int Bnr, int Bnc, float* C,

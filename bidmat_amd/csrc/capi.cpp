@@ -314,6 +314,49 @@ API int bidmat_spsum_rows_plan(bidmat_plan* plan, const float* Sdata, float* out
     return (int)run_spsum_rows(plan, Sdata, out, beta, as_stream(stream));
 }
 
+API int bidmat_transpose(int nrows, int ncols, const float* in, int ldi, float* out, int ldo, void* stream) {
+    if (nrows < 0 || ncols < 0 || ldi < nrows || ldo < ncols) return kInvalid;
+    if (nrows == 0 || ncols == 0) return 0;
+    if (!in || !out) return kInvalid;
+    return (int)bm::transpose(nrows, ncols, in, ldi, out, ldo, as_stream(stream));
+}
+
+API int bidmat_sdtmult_csc(int nrows, int ncols, int nnz, int p, const float* Sdata, const int* Sir,
+                           const int* Sjc, const float* A, int lda, float* C, int ldc, void* stream) {
+    if (nrows < 0 || ncols < 0 || nnz < 0 || p < 0 || lda < nrows || ldc < ncols) return kInvalid;
+    if (ncols == 0 || p == 0) return 0;
+    if (!Sjc || !C || (nnz > 0 && (!Sdata || !Sir || !A))) return kInvalid;
+    hipStream_t s = as_stream(stream);
+    hipError_t err;
+    // At = A^T (p x nrows), Ct = At * S (p x ncols), C = Ct^T
+    float* At = (float*)bm::ws_get(bm::WS_TRANS_IN, sizeof(float) * (size_t)p * (size_t)(nrows > 0 ? nrows : 1), &err);
+    if (!At) return (int)err;
+    float* Ct = (float*)bm::ws_get(bm::WS_TRANS_OUT, sizeof(float) * (size_t)p * (size_t)ncols, &err);
+    if (!Ct) return (int)err;
+    if ((err = bm::transpose(nrows, p, A, lda, At, p, s)) != hipSuccess) return (int)err;
+    if ((err = bm::dsmult_csc(p, ncols, nnz, At, Sdata, Sir, Sjc, Ct, 0, s)) != hipSuccess) return (int)err;
+    return (int)bm::transpose(p, ncols, Ct, p, C, ldc, s);
+}
+
+API int bidmat_sdmult_plan(bidmat_plan* plan, int p, const float* Sdata, const float* A, int lda, float* C,
+                           int ldc, void* stream) {
+    if (!plan || p < 0) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (lda < plan->ncols || ldc < plan->nrows) return kInvalid;
+    if (plan->nrows == 0 || p == 0) return 0;
+    if (!C || (plan->nnz > 0 && (!Sdata || !A))) return kInvalid;
+    hipStream_t s = as_stream(stream);
+    hipError_t err;
+    // At = A^T (p x ncols), Ct = At *^ S (p x nrows), C = Ct^T
+    float* At = (float*)bm::ws_get(bm::WS_TRANS_IN, sizeof(float) * (size_t)p * (size_t)(plan->ncols > 0 ? plan->ncols : 1), &err);
+    if (!At) return (int)err;
+    float* Ct = (float*)bm::ws_get(bm::WS_TRANS_OUT, sizeof(float) * (size_t)p * (size_t)plan->nrows, &err);
+    if (!Ct) return (int)err;
+    if ((err = bm::transpose(plan->ncols, p, A, lda, At, p, s)) != hipSuccess) return (int)err;
+    if ((err = run_dsmultT(plan, p, At, Sdata, Ct, 0, s)) != hipSuccess) return (int)err;
+    return (int)bm::transpose(p, plan->nrows, Ct, p, C, ldc, s);
+}
+
 API int bidmat_csc_expand_cols(int ncols, int nnz, const int* Sjc, int* Sic, void* stream) {
     if (ncols < 0 || nnz < 0) return kInvalid;
     if (nnz == 0) return 0;

@@ -74,4 +74,7 @@ hipError_t reduce2op(int nrows, int ncols, const float* A, float* B, float initv
 hipError_t applyop(const float* A, int Anr, int Anc, const float* B, int Bnr, int Bnc, float* C,
                    int opn, hipStream_t s);
 
+// out (ncols x nrows, leading dimension ldo) = transpose of in (nrows x ncols, leading dimension ldi)
+hipError_t transpose(int nrows, int ncols, const float* in, int ldi, float* out, int ldo, hipStream_t s);
+
 }  // namespace bm

@@ -14,6 +14,8 @@ enum WsSlot {
     WS_SCAN,          // int[...]      block sums of the scan
     WS_MISC,          // small scalars (max row, fingerprints)
     WS_REDUCE,        // float[...]    partials of the dense reductions
+    WS_TRANS_IN,      // float[...]    transposed dense operand of S*A / S^T*A
+    WS_TRANS_OUT,     // float[...]    transposed result of S*A / S^T*A
     WS_NSLOTS
 };
 

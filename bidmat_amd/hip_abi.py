@@ -37,6 +37,9 @@ SIGNATURES = {
     "bidmat_spsum_rows_plan": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "bidmat_csc_expand_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
     "bidmat_coo_compress_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
+    "bidmat_sdtmult_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int, vp, C.c_int, vp]),
+    "bidmat_sdmult_plan": (C.c_int, [vp, C.c_int, vp, vp, C.c_int, vp, C.c_int, vp]),
+    "bidmat_transpose": (C.c_int, [C.c_int, C.c_int, vp, C.c_int, vp, C.c_int, vp]),
     "bidmat_applyop_flat": (C.c_int, [vp, vp, vp, C.c_longlong, C.c_int, vp]),
     # memory / runtime
     "bidmat_device_count": (C.c_int, [c_int_p]),

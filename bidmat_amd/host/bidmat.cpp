@@ -415,6 +415,26 @@ GMatP GSMat::sum(int n, GMatP oldmat) {
     return out;
 }
 
+GMatP GSMat::SDMult(const GMatP& a, GMatP omat) {
+    if (ncols != a->nrows) fail("SDMult dimensions mismatch");
+    GMatP out = GMat::newOrCheckGMat(nrows, a->ncols, omat, GUID, a->GUID, opHash("SDMult"));
+    int err = bidmat_sdmult_plan(plan(a->ncols), a->ncols, pdata, a->pdata, a->nrows, out->pdata, out->nrows, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("HIP error in GSMAT.SDMult ") + bidmat_error_string(err));
+    Mat::nflops += 2LL * nnz0 * a->ncols;
+    return out;
+}
+
+GMatP GSMat::SDTMult(const GMatP& a, GMatP omat) {
+    if (nrows != a->nrows) fail("SDTMult dimensions mismatch");
+    GMatP out = GMat::newOrCheckGMat(ncols, a->ncols, omat, GUID, a->GUID, opHash("SDTMult"));
+    int err = bidmat_sdtmult_csc(nrows, ncols, nnz0, a->ncols, pdata, pir, pjc, a->pdata, a->nrows, out->pdata, out->nrows, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("HIP error in GSMAT.SDTMult ") + bidmat_error_string(err));
+    Mat::nflops += 2LL * nnz0 * a->ncols;
+    return out;
+}
+
 GSMatP GSMat::DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat) {
     if (A->nrows != B->nrows || C->nrows != A->ncols || C->ncols != B->ncols)
         fail(fmt("dimensions mismatch %d,%d  %d,%d  %d,%d", A->nrows, A->ncols, B->nrows, B->ncols, C->nrows, C->ncols));
@@ -449,6 +469,8 @@ GSMatP GSMat::withValues(const GMatP& vals) const {
 GMatP operator*(const GMatP& a, const GSMatP& s) { return a->GSMult(s, nullptr); }
 GMatP xT(const GMatP& a, const GSMatP& s) { return a->GSMultT(s, nullptr); }
 GMatP operator/(const GMatP& a, const GMatP& b) { return a->gOp(b, nullptr, op_div); }
+GMatP operator*(const GSMatP& s, const GMatP& a) { return s->SDMult(a, nullptr); }
+GMatP Tx(const GSMatP& s, const GMatP& a) { return s->SDTMult(a, nullptr); }
 GSMatP DDS(const GMatP& a, const GMatP& b, const GSMatP& c, GSMatP omat) { return GSMat::DDS(a, b, c, omat); }
 GMatP sum(const GSMatP& s, int n, GMatP omat) { return s->sum(n, omat); }
 GMatP sum(const GMatP& a, int n, GMatP omat) { return a->reduceOp(omat, n, 0.f, op_add); }

@@ -142,6 +142,8 @@ public:
     GSMat& clear();
     void free();
     GMatP sum(int n, GMatP oldmat);                              // GSMat.scala:250-261
+    GMatP SDMult(const GMatP& a, GMatP omat);                    // this * a    (GSMat.scala:265-289)
+    GMatP SDTMult(const GMatP& a, GMatP omat);                   // this ^* a   (GSMat.scala:291-313)
     static GSMatP DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat);   // GSMat.scala:649-667
     // a sparse matrix with this pattern and other values (the V./R step keeps V's pattern)
     GSMatP withValues(const GMatP& vals) const;
@@ -155,6 +157,8 @@ public:
 // ---- operators (GMat.scala:1684-1688, 1972-1976) and free functions
 GMatP operator*(const GMatP& a, const GSMatP& s);                 // a * s
 GMatP xT(const GMatP& a, const GSMatP& s);                        // a *^ s  (alias xT in the reference)
+GMatP operator*(const GSMatP& s, const GMatP& a);                 // s * a   (GSMat.scala:334)
+GMatP Tx(const GSMatP& s, const GMatP& a);                        // s ^* a  (GSMat.scala:335-336)
 GMatP operator/(const GMatP& a, const GMatP& b);                  // elementwise
 GSMatP DDS(const GMatP& a, const GMatP& b, const GSMatP& c, GSMatP omat = nullptr);
 GMatP sum(const GSMatP& s, int n = 0, GMatP omat = nullptr);      // SFunctions.scala:10-15

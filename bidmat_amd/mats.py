@@ -31,7 +31,7 @@ def _load():
         L = C.CDLL(LIB_PATH)
         for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
                      "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
-                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult"):
+                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult"):
             getattr(L, name).restype = vp
         L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
         L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
@@ -39,6 +39,7 @@ def _load():
         for name in ("bmh_mult", "bmh_madd", "bmh_multT", "bmh_maddT"):
             getattr(L, name).argtypes = [vp, vp, vp]
         L.bmh_dds.argtypes = [vp, vp, vp, vp]
+        L.bmh_sdmult.argtypes = [vp, vp, vp, C.c_int]
         L.bmh_tile_mult.argtypes = [vp] + [C.c_int] * 5 + [vp, C.c_int, C.c_int, vp, C.c_int, C.c_int, C.c_int]
         L.bmh_sum_sparse.argtypes = [vp, C.c_int, vp]
         L.bmh_sum_dense.argtypes = [vp, C.c_int, vp]
@@ -224,6 +225,18 @@ class GSMat(_Handle):
 
     def contents(self):
         return GMat(_load().bmh_contents(self._h))
+
+    def __mul__(self, a):                 # s * a   (sparse times dense)
+        return GMat(_load().bmh_sdmult(self._h, a._h, None, 0))
+
+    def SDMult(self, a, out=None):
+        return GMat(_load().bmh_sdmult(self._h, a._h, out._h if out else None, 0))
+
+    def Tx(self, a):                      # s ^* a  (sparse-transpose times dense)
+        return GMat(_load().bmh_sdmult(self._h, a._h, None, 1))
+
+    def SDTMult(self, a, out=None):
+        return GMat(_load().bmh_sdmult(self._h, a._h, out._h if out else None, 1))
 
     def with_values(self, vals):
         return GSMat(_load().bmh_with_values(self._h, vals._h))

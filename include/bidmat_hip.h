@@ -145,6 +145,19 @@ int bidmat_csc_expand_cols(int ncols, int nnz, const int *Sjc, int *Sic, void *s
  * and SparseMat.compressInds (SparseMat.scala:857-868). Enqueues on stream. */
 int bidmat_coo_compress_cols(int ncols, int nnz, const int *Sic, int *Sjc, void *stream);
 
+/* Sparse times dense, the other operand order (GSMat.SDMult / SDTMult, GSMat.scala:265-313, which
+ * call cusparseScsrmm with alpha = 1, beta = 0):
+ *   bidmat_sdtmult_csc:  C (ncols x p) = S^T * A,  A is nrows x p   (S ^* A)
+ *   bidmat_sdmult_plan:  C (nrows x p) = S * A,    A is ncols x p   (S * A), needs the row plan
+ * A and C are column-major with leading dimensions lda / ldc.  Implemented on the gather
+ * kernels through dense transposes ((S^T A)^T = A^T S, (S A)^T = A^T S^T) in library workspace. */
+int bidmat_sdtmult_csc(int nrows, int ncols, int nnz, int p, const float *Sdata, const int *Sir,
+                       const int *Sjc, const float *A, int lda, float *C, int ldc, void *stream);
+int bidmat_sdmult_plan(bidmat_plan *plan, int p, const float *Sdata, const float *A, int lda, float *C,
+                       int ldc, void *stream);
+/* out (ncols x nrows, leading dimension ldo) = transpose of in (nrows x ncols, leading dim ldi). */
+int bidmat_transpose(int nrows, int ncols, const float *in, int ldi, float *out, int ldo, void *stream);
+
 /* Elementwise on flat arrays with a stream (the V./R step on GSMat.contents). */
 int bidmat_applyop_flat(const float *A, const float *B, float *C, long long n, int opn,
                         void *stream);

@@ -557,3 +557,51 @@ def test_dsmult_tile_whole_matrix_equals_plain_product(hip):
     hip_abi.check(hip.bidmat_dsmultTileT(k, nrows, ncols, ir.size, d.B.ptr, k, d.data.ptr, d.ir.ptr, d.ic.ptr, 0, 0, d.G2.ptr, k))
     assert np.array_equal(d.G1.numpy(), d.G2.numpy())
     d.free()
+
+
+# ------------------------------------------------------------------------------ sparse x dense
+@pytest.mark.parametrize("p", [1, 7, 64, 200])
+def test_sparse_times_dense(hip, p):
+    """S*A and S^T*A through the C ABI, windows via lda / ldc, against fp64 dense products."""
+    rng = np.random.default_rng(500 + p)
+    m, n = 150, 230
+    data, ir, jc = random_csc(rng, m, n, 0.06)
+    S = dense_full(m, n, data, ir, jc)
+    d = Dev(data=data, ir=ir, jc=jc)
+    plan = make_plan(hip, m, n, ir.size, d.ir, d.jc, p)
+    # S * A: A is n x p inside a parent with leading dimension n + 3
+    lda, ldc = n + 3, m + 2
+    Ap = rng.standard_normal(lda * p).astype(np.float32)
+    d.put("A", Ap), d.put("Cm", np.full(ldc * p, 7.0, dtype=np.float32))
+    hip_abi.check(hip.bidmat_sdmult_plan(plan, p, d.data.ptr, d.A.ptr, lda, d.Cm.ptr, ldc, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    got = d.Cm.numpy().reshape(p, ldc).T
+    A2 = Ap.reshape(p, lda).T[:n].astype(np.float64)
+    want, sa = S @ A2, np.abs(S) @ np.abs(A2)
+    assert_close(got[:m].ravel(), want.ravel(), sa.ravel(), "S*A p=%d" % p)
+    assert np.all(got[m:] == 7.0)                       # padding rows of the parent untouched
+    # S^T * A: A is m x p
+    lda, ldc = m + 1, n + 5
+    Ap = rng.standard_normal(lda * p).astype(np.float32)
+    d.put("A2", Ap), d.put("C2", np.full(ldc * p, 7.0, dtype=np.float32))
+    hip_abi.check(hip.bidmat_sdtmult_csc(m, n, ir.size, p, d.data.ptr, d.ir.ptr, d.jc.ptr, d.A2.ptr, lda, d.C2.ptr, ldc, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    got = d.C2.numpy().reshape(p, ldc).T
+    A2 = Ap.reshape(p, lda).T[:m].astype(np.float64)
+    want, sa = S.T @ A2, np.abs(S).T @ np.abs(A2)
+    assert_close(got[:n].ravel(), want.ravel(), sa.ravel(), "S^T*A p=%d" % p)
+    assert np.all(got[n:] == 7.0)
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    d.free()
+
+
+def test_transpose(hip):
+    rng = np.random.default_rng(510)
+    for (nr_, nc_) in ((1, 1), (5, 70), (33, 31), (257, 64), (64, 1000)):
+        a = rng.standard_normal((nr_, nc_)).astype(np.float32)
+        d = Dev(a=np.asfortranarray(a).ravel(order="F"))
+        d.zeros("t", nr_ * nc_)
+        hip_abi.check(hip.bidmat_transpose(nr_, nc_, d.a.ptr, nr_, d.t.ptr, nc_, None))
+        hip_abi.check(hip.bidmat_synchronize())
+        assert np.array_equal(d.t.numpy().reshape(nr_, nc_).T, a.T)
+        d.free()

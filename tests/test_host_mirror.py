@@ -277,3 +277,26 @@ def test_tile_mult_and_messages(hip):
         aa.tileMult(7, 9, 11, 3, 5, ss, 30, 4, cc, 2, 8)
     with pytest.raises(RuntimeError, match="tileMultNT: tile strays outside matrix dimensions"):
         aa.tileMultNT(6, 10, 8, 1, 7, ss, 5, 25, cc, 4, 3)
+
+
+@gpu
+def test_sparse_times_dense_both_orders(hip):
+    """'support matrix multiplication' GSMat * GMat half (GSMatTest.scala:55-63) and
+    'support matrix ^*' (GSMatTest.scala:85-94)."""
+    rng = np.random.default_rng(14)
+    a = sprand(rng, nr, nk, 0.2)
+    b = rng.random((nk, nc)).astype(np.float32)
+    aa, bb = GSMat.from_csc(nr, nk, *a), GMat.from_numpy(b)
+    before = Mat.nflops()
+    cc = aa * bb
+    assert cc.mytype == "GMat" and cc.shape == (nr, nc)
+    assert Mat.nflops() - before == 2 * a[0].size * nc
+    np.testing.assert_allclose(cc.numpy(), full(nr, nk, *a) @ b.astype(np.float64), rtol=0, atol=EPS)
+    a2 = sprand(rng, nk, nr, 0.2)
+    cc = GSMat.from_csc(nk, nr, *a2).Tx(bb)
+    assert cc.mytype == "GMat" and cc.shape == (nr, nc)
+    np.testing.assert_allclose(cc.numpy(), full(nk, nr, *a2).T @ b.astype(np.float64), rtol=0, atol=EPS)
+    with pytest.raises(RuntimeError, match="SDMult dimensions mismatch"):
+        aa * GMat.from_numpy(rng.random((nk + 1, nc)).astype(np.float32))
+    with pytest.raises(RuntimeError, match="SDTMult dimensions mismatch"):
+        aa.Tx(bb)
