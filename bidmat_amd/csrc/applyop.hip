@@ -56,6 +56,16 @@ __global__ __launch_bounds__(BM_BLOCK) void k_apply_full4(const float4* __restri
     }
 }
 
+// Sparse values op edge vector, in place: A[i] = op(A[i], B[idx[i]]) (GATHER) or op(A[i], B[0]).
+template <int OP, bool GATHER>
+__global__ __launch_bounds__(BM_BLOCK) void k_sdop(long long nnz, float* __restrict__ A, const int* __restrict__ idx,
+                                                   const float* __restrict__ B) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    const float bval = GATHER ? 0.f : B[0];
+    for (; i < nnz; i += stride) A[i] = binop<OP>(A[i], GATHER ? B[idx[i]] : bval);
+}
+
 // Dense transpose through a padded LDS tile: in is nrows x ncols (column-major, leading dimension
 // ldi), out is ncols x nrows (leading dimension ldo). Reads and writes are both coalesced.
 constexpr int TT = 32;
@@ -114,6 +124,22 @@ hipError_t apply_impl(const float* A, int ma, const float* B, int mb, float* C, 
 }
 
 }  // namespace
+
+hipError_t sdop(long long nnz, float* A, const int* idx, const float* B, int len, int opn, hipStream_t s) {
+    if (nnz <= 0) return hipSuccess;
+    dim3 grid(grid_for(nnz)), block(BM_BLOCK);
+    switch (opn) {
+#define BM_OP(N_)                                                                                          \
+    case N_:                                                                                               \
+        if (len > 1) hipLaunchKernelGGL((k_sdop<N_, true>), grid, block, 0, s, nnz, A, idx, B);            \
+        else hipLaunchKernelGGL((k_sdop<N_, false>), grid, block, 0, s, nnz, A, idx, B);                   \
+        return hipGetLastError();
+    BM_OP(0) BM_OP(1) BM_OP(2) BM_OP(3) BM_OP(4) BM_OP(5) BM_OP(6) BM_OP(7)
+    BM_OP(8) BM_OP(9) BM_OP(10) BM_OP(11) BM_OP(12) BM_OP(13) BM_OP(14)
+#undef BM_OP
+    default: return hipErrorInvalidValue;
+    }
+}
 
 hipError_t transpose(int nrows, int ncols, const float* in, int ldi, float* out, int ldo, hipStream_t s) {
     if (nrows <= 0 || ncols <= 0) return hipSuccess;

@@ -189,6 +189,22 @@ API int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float* A, int 
     return finish_blocking(err);
 }
 
+API int bidmat_sdoprow(int nrows, int ncols, int nnz, float* A, const int* Aic, const float* B, int len, int opn) {
+    if (nrows < 0 || ncols < 0 || nnz < 0 || opn < 0 || opn > 14) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!A || !B || (len > 1 && !Aic)) return kInvalid;
+    if (len > 1 && len < ncols) return kInvalid;         // a row vector has one entry per column
+    return finish_blocking(bm::sdop(nnz, A, Aic, B, len, opn, nullptr));
+}
+
+API int bidmat_sdopcol(int nrows, int ncols, int nnz, float* A, const int* Air, const float* B, int len, int opn) {
+    if (nrows < 0 || ncols < 0 || nnz < 0 || opn < 0 || opn > 14) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!A || !B || (len > 1 && !Air)) return kInvalid;
+    if (len > 1 && len < nrows) return kInvalid;         // a column vector has one entry per row
+    return finish_blocking(bm::sdop(nnz, A, Air, B, len, opn, nullptr));
+}
+
 API int bidmat_dds(int nrows, int nnz, const float* A, const float* B, const int* Cir,
                    const int* Cic, float* P) {
     if (nrows < 0 || nnz < 0) return kInvalid;

@@ -31,6 +31,13 @@ JFN(jint, dsmultTile)(JNIEnv*, jclass, jint nr, jint nc, jint kk, jint nnz, jlon
         return bidmat_dsmultTileT(nr, nc, kk, nnz, P(const float, A), lda, P(const float, Bdata), P(const int, Bir), P(const int, Bic), broff, bcoff, P(float, C), ldc);
     return bidmat_dsmultTile(nr, nc, kk, nnz, P(const float, A), lda, P(const float, Bdata), P(const int, Bir), P(const int, Bic), broff, bcoff, P(float, C), ldc);
 }
+// replace Java_edu_berkeley_bid_CUMAT_sdoprow / sdopcol
+JFN(jint, sdoprow)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong A, jlong Aic, jlong B, jint len, jint op) {
+    return bidmat_sdoprow(nr, nc, nnz, P(float, A), P(const int, Aic), P(const float, B), len, op);
+}
+JFN(jint, sdopcol)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong A, jlong Air, jlong B, jint len, jint op) {
+    return bidmat_sdopcol(nr, nc, nnz, P(float, A), P(const int, Air), P(const float, B), len, op);
+}
 // replaces Java_edu_berkeley_bid_CUMAT_dds (BIDMat_CUMAT.cpp:774-785)
 JFN(jint, dds)(JNIEnv*, jclass, jint nr, jint nnz, jlong A, jlong B, jlong Cir, jlong Cic, jlong Pv) {
     return bidmat_dds(nr, nnz, P(const float, A), P(const float, B), P(const int, Cir), P(const int, Cic), P(float, Pv));

@@ -74,6 +74,8 @@ hipError_t reduce2op(int nrows, int ncols, const float* A, float* B, float initv
 hipError_t applyop(const float* A, int Anr, int Anc, const float* B, int Bnr, int Bnc, float* C,
                    int opn, hipStream_t s);
 
+// A[i] = op(A[i], len > 1 ? B[idx[i]] : B[0]) over the nnz stored values (in place)
+hipError_t sdop(long long nnz, float* A, const int* idx, const float* B, int len, int opn, hipStream_t s);
 // out (ncols x nrows, leading dimension ldo) = transpose of in (nrows x ncols, leading dimension ldi)
 hipError_t transpose(int nrows, int ncols, const float* in, int ldi, float* out, int ldo, hipStream_t s);
 

@@ -20,6 +20,8 @@ SIGNATURES = {
     "bidmat_dsmultT": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp]),
     "bidmat_dsmultTile": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, vp, vp, vp, C.c_int, C.c_int, vp, C.c_int]),
     "bidmat_dsmultTileT": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, vp, vp, vp, C.c_int, C.c_int, vp, C.c_int]),
+    "bidmat_sdoprow": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, C.c_int, C.c_int]),
+    "bidmat_sdopcol": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, C.c_int, C.c_int]),
     "bidmat_dds": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp, vp]),
     "bidmat_spsum": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int]),
     "bidmat_reduce1op": (C.c_int, [C.c_int, C.c_int, vp, vp, C.c_float, C.c_int]),

@@ -415,6 +415,30 @@ GMatP GSMat::sum(int n, GMatP oldmat) {
     return out;
 }
 
+GSMatP GSMat::copy(GSMatP omat, long long key1, long long key2) {
+    GSMatP out = newOrCheckGSMat(nrows, ncols, nnz0, realnnz, omat, GUID, key1, key2, opHash("copy"));
+    if (out.get() != this) {
+        hipcheck(bidmat_memcpy_d2d(out->pir, pir, (long long)sizeof(int) * nnz0), "GSMat.copy");
+        hipcheck(bidmat_memcpy_d2d(out->pic, pic, (long long)sizeof(int) * nnz0), "GSMat.copy");
+        hipcheck(bidmat_memcpy_d2d(out->pjc, pjc, (long long)sizeof(int) * ((long long)ncols + 1)), "GSMat.copy");
+        hipcheck(bidmat_memcpy_d2d(out->pdata, pdata, (long long)sizeof(float) * nnz0), "GSMat.copy");
+        out->planHolder = planHolder;
+    }
+    return out;
+}
+
+GSMatP GSMat::GSDop(const GMatP& b, GSMatP omat, int op) {
+    if (b->nrows > 1 && b->ncols > 1) fail("Sorry only edge operators supported for GSMat op GMat");
+    if (b->nrows != nrows && b->ncols != ncols && b->length() > 1) fail("GSMat op GMat: dimensions mismatch");
+    Mat::nflops += nnz0;
+    GSMatP out = copy(omat, b->GUID, op);
+    int err;
+    if (b->ncols > 1) err = bidmat_sdoprow(nrows, ncols, nnz0, out->pdata, out->pic, b->pdata, (int)b->length(), op);
+    else err = bidmat_sdopcol(nrows, ncols, nnz0, out->pdata, out->pir, b->pdata, (int)b->length(), op);
+    if (err != 0) fail(std::string("HIP error in GSMat.GSDop ") + bidmat_error_string(err));
+    return out;
+}
+
 GMatP GSMat::SDMult(const GMatP& a, GMatP omat) {
     if (ncols != a->nrows) fail("SDMult dimensions mismatch");
     GMatP out = GMat::newOrCheckGMat(nrows, a->ncols, omat, GUID, a->GUID, opHash("SDMult"));

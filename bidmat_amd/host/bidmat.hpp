@@ -142,6 +142,8 @@ public:
     GSMat& clear();
     void free();
     GMatP sum(int n, GMatP oldmat);                              // GSMat.scala:250-261
+    GSMatP GSDop(const GMatP& b, GSMatP omat, int op);           // this op edge vector (GSMat.scala:315-330)
+    GSMatP copy(GSMatP omat, long long key1, long long key2);    // GSMat.copy / copyTo
     GMatP SDMult(const GMatP& a, GMatP omat);                    // this * a    (GSMat.scala:265-289)
     GMatP SDTMult(const GMatP& a, GMatP omat);                   // this ^* a   (GSMat.scala:291-313)
     static GSMatP DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat);   // GSMat.scala:649-667

@@ -91,6 +91,9 @@ API void* bmh_tile_mult(void* a, int nr, int nc, int kk, int aroff, int acoff, v
 API void* bmh_sdmult(void* s, void* a, void* out, int transposed) {
     return guard_ptr([&] { return wrap(transposed ? S(s)->SDTMult(G(a), G(out)) : S(s)->SDMult(G(a), G(out))); });
 }
+API void* bmh_gsdop(void* s, void* b, void* out, int op) {
+    return guard_ptr([&] { return wrap(S(s)->GSDop(G(b), S(out), op)); });
+}
 API void* bmh_dds(void* a, void* b, void* c, void* out) {
     return guard_ptr([&] { return wrap(GSMat::DDS(G(a), G(b), S(c), S(out))); });
 }

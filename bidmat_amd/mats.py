@@ -31,7 +31,7 @@ def _load():
         L = C.CDLL(LIB_PATH)
         for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
                      "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
-                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult"):
+                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop"):
             getattr(L, name).restype = vp
         L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
         L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
@@ -40,6 +40,7 @@ def _load():
             getattr(L, name).argtypes = [vp, vp, vp]
         L.bmh_dds.argtypes = [vp, vp, vp, vp]
         L.bmh_sdmult.argtypes = [vp, vp, vp, C.c_int]
+        L.bmh_gsdop.argtypes = [vp, vp, vp, C.c_int]
         L.bmh_tile_mult.argtypes = [vp] + [C.c_int] * 5 + [vp, C.c_int, C.c_int, vp, C.c_int, C.c_int, C.c_int]
         L.bmh_sum_sparse.argtypes = [vp, C.c_int, vp]
         L.bmh_sum_dense.argtypes = [vp, C.c_int, vp]
@@ -225,6 +226,9 @@ class GSMat(_Handle):
 
     def contents(self):
         return GMat(_load().bmh_contents(self._h))
+
+    def GSDop(self, b, op, out=None):     # s op edge-vector (row vector, column vector or 1x1)
+        return GSMat(_load().bmh_gsdop(self._h, b._h, out._h if out else None, op))
 
     def __mul__(self, a):                 # s * a   (sparse times dense)
         return GMat(_load().bmh_sdmult(self._h, a._h, None, 0))

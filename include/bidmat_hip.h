@@ -66,6 +66,14 @@ int bidmat_dsmultTile(int nr, int nc, int kk, int nnz, const float *A, int lda, 
 int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float *A, int lda, const float *Bdata,
                        const int *Bir, const int *Bic, int broff, int bcoff, float *C, int ldc);
 
+/* Sparse matrix (its nnz stored values A, in place) op edge vector:
+ *   bidmat_sdoprow: A[i] = op(A[i], B[Aic[i]])  (B a row vector, one entry per column), or op(A[i], B[0]) if len <= 1
+ *   bidmat_sdopcol: A[i] = op(A[i], B[Air[i]])  (B a column vector, one entry per row), same scalar rule.
+ * Replace `int sdoprow/sdopcol(int nrows,int ncols,int nnz,float*A,int*Aic|Air,float*B,int len,int opn)`
+ * (Operators.cu:585-647; CUMAT.java:135,139; caller GSMat.GSDop, GSMat.scala:315-330). All 15 ops. */
+int bidmat_sdoprow(int nrows, int ncols, int nnz, float *A, const int *Aic, const float *B, int len, int opn);
+int bidmat_sdopcol(int nrows, int ncols, int nnz, float *A, const int *Air, const float *B, int len, int opn);
+
 /* P[j] += dot(A[:,Cir[j]], B[:,Cic[j]]).  Replaces `int dds(int nrows,int nnz,float*A,float*B,
  * int*Cir,int*Cic,float*P)` (Arith.cu:381-389; CUMAT.java:211; caller GSMat.scala:663). */
 int bidmat_dds(int nrows, int nnz, const float *A, const float *B, const int *Cir,

@@ -300,3 +300,29 @@ def test_sparse_times_dense_both_orders(hip):
         aa * GMat.from_numpy(rng.random((nk + 1, nc)).astype(np.float32))
     with pytest.raises(RuntimeError, match="SDTMult dimensions mismatch"):
         aa.Tx(bb)
+
+
+@gpu
+@pytest.mark.parametrize("op,fn", [(0, np.add), (1, np.subtract), (2, np.multiply), (3, np.divide), (10, np.maximum), (11, np.minimum)])
+def test_sparse_op_edge_vector(hip, op, fn):
+    """GSMat op GMat for row vectors, column vectors and scalars (GSMat.GSDop; the reference's
+    testEwise family, GSMatTest.scala:96-280): the op touches the stored values only."""
+    rng = np.random.default_rng(15 + op)
+    data, ir, jc = sprand(rng, nr, nc, 0.3)
+    aa = GSMat.from_csc(nr, nc, data, ir, jc)
+    cols = np.repeat(np.arange(nc), np.diff(jc))
+    row = (rng.random((1, nc)) + 0.5).astype(np.float32)
+    col = (rng.random((nr, 1)) + 0.5).astype(np.float32)
+    val = (rng.random((1, 1)) + 0.5).astype(np.float32)
+    for b, pick in ((row, row[0, cols]), (col, col[ir - 1, 0]), (val, np.full(data.size, val[0, 0], np.float32))):
+        before = Mat.nflops()
+        out = aa.GSDop(GMat.from_numpy(b), op)
+        assert out.mytype == "GSMat" and Mat.nflops() - before == data.size
+        vals, oir, ojc = out.to_csc()
+        assert np.array_equal(oir, ir) and np.array_equal(ojc, jc)
+        assert np.array_equal(vals, fn(data, pick).astype(np.float32))
+    assert np.array_equal(aa.to_csc()[0], data)          # the operand itself is not modified
+    with pytest.raises(RuntimeError, match="only edge operators supported"):
+        aa.GSDop(GMat.from_numpy(rng.random((nr, nc)).astype(np.float32)), op)
+    with pytest.raises(RuntimeError, match="dimensions mismatch"):
+        aa.GSDop(GMat.from_numpy(rng.random((1, nc + 1)).astype(np.float32)), op)
