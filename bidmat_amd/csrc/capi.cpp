@@ -430,6 +430,14 @@ API int bidmat_memcpy_d2d(void* dst, const void* src, long long bytes) {
     if (bytes < 0 || (bytes > 0 && (!dst || !src))) return kInvalid;
     return bytes ? (int)hipMemcpy(dst, src, (size_t)bytes, hipMemcpyDeviceToDevice) : 0;
 }
+API int bidmat_memcpy_h2d_async(void* dst, const void* src, long long bytes, void* stream) {
+    if (bytes < 0 || (bytes > 0 && (!dst || !src))) return kInvalid;
+    return bytes ? (int)hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyHostToDevice, as_stream(stream)) : 0;
+}
+API int bidmat_memcpy_d2h_async(void* dst, const void* src, long long bytes, void* stream) {
+    if (bytes < 0 || (bytes > 0 && (!dst || !src))) return kInvalid;
+    return bytes ? (int)hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToHost, as_stream(stream)) : 0;
+}
 API int bidmat_memset(void* dptr, int value, long long bytes) {
     if (bytes < 0 || (bytes > 0 && !dptr)) return kInvalid;
     if (!bytes) return 0;

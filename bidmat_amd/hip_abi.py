@@ -52,6 +52,8 @@ SIGNATURES = {
     "bidmat_memcpy_h2d": (C.c_int, [vp, vp, C.c_longlong]),
     "bidmat_memcpy_d2h": (C.c_int, [vp, vp, C.c_longlong]),
     "bidmat_memcpy_d2d": (C.c_int, [vp, vp, C.c_longlong]),
+    "bidmat_memcpy_h2d_async": (C.c_int, [vp, vp, C.c_longlong, vp]),
+    "bidmat_memcpy_d2h_async": (C.c_int, [vp, vp, C.c_longlong, vp]),
     "bidmat_memset": (C.c_int, [vp, C.c_int, C.c_longlong]),
     "bidmat_mem_info": (C.c_int, [C.POINTER(C.c_longlong), C.POINTER(C.c_longlong)]),
     "bidmat_synchronize": (C.c_int, []),

@@ -168,6 +168,20 @@ GMatP sum(const GMatP& a, int n = 0, GMatP omat = nullptr);       // GFunctions.
 // host reference path: FMat * SMat, FMat *^ SMat, DDS on host are NOT provided here (the CPU
 // restatement of those loops lives with the tests); these mirror only the GPU dispatch.
 
+// ---- matrix files (HMat.scala): little-endian int32 header [type, nrows, ncols, nnz], then
+// for a sparse float matrix (type 231) jc[ncols+1], ir[nnz], data[nnz] with 0-based indices on
+// disk (HMat.scala:1232-1266, 1444-1480); for a dense float matrix (type 130) the column-major
+// floats (HMat.scala:337-399, 876-891). Names ending in .gz are gzip streams; .lz4 is refused.
+namespace HMat {
+SMat loadSMat(const std::string& fname);
+void saveSMat(const std::string& fname, const SMat& m);
+FMat loadFMat(const std::string& fname);
+void saveFMat(const std::string& fname, const FMat& m);
+// Reads a type-231 file straight into a GSMat: chunks go through two pinned staging buffers and
+// asynchronous copies, so reading the file and crossing PCIe overlap.
+GSMatP loadGSMat(const std::string& fname);
+}  // namespace HMat
+
 // timers (MatFunctions.scala:19-51)
 void flip();
 std::pair<float, float> flop();

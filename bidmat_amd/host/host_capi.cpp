@@ -106,6 +106,40 @@ API void* bmh_gop(void* a, void* b, void* out, int op) { return guard_ptr([&] { 
 API void* bmh_contents(void* s) { return guard_ptr([&] { GMatP v = S(s)->contents(); v->keepalive = S(s); return wrap(v); }); }
 API void* bmh_with_values(void* s, void* vals) { return guard_ptr([&] { return wrap(S(s)->withValues(G(vals))); }); }
 
+// ---- matrix files (host arrays carry Mat::ioneBased)
+API int bmh_save_smat(const char* fname, int nr, int nc, int nnz, const float* data, const int* ir, const int* jc) {
+    return guard_int([&] {
+        SMat a(nr, nc, nnz);
+        memcpy(a.data.data(), data, sizeof(float) * (size_t)nnz);
+        memcpy(a.ir.data(), ir, sizeof(int) * (size_t)nnz);
+        memcpy(a.jc.data(), jc, sizeof(int) * ((size_t)nc + 1));
+        HMat::saveSMat(fname, a);
+    });
+}
+// two calls: first with null arrays to learn the sizes, then with arrays to fill
+API int bmh_load_smat(const char* fname, int* nr, int* nc, int* nnz, float* data, int* ir, int* jc) {
+    return guard_int([&] {
+        SMat a = HMat::loadSMat(fname);
+        *nr = a.nrows; *nc = a.ncols; *nnz = a.nnz();
+        if (data) {
+            memcpy(data, a.data.data(), sizeof(float) * a.data.size());
+            memcpy(ir, a.ir.data(), sizeof(int) * a.ir.size());
+            memcpy(jc, a.jc.data(), sizeof(int) * a.jc.size());
+        }
+    });
+}
+API int bmh_save_fmat(const char* fname, int nr, int nc, const float* data) {
+    return guard_int([&] { HMat::saveFMat(fname, FMat(nr, nc, data)); });
+}
+API int bmh_load_fmat(const char* fname, int* nr, int* nc, float* data) {
+    return guard_int([&] {
+        FMat a = HMat::loadFMat(fname);
+        *nr = a.nrows; *nc = a.ncols;
+        if (data) memcpy(data, a.data.data(), sizeof(float) * a.data.size());
+    });
+}
+API void* bmh_load_gsmat(const char* fname) { return guard_ptr([&] { return wrap(HMat::loadGSMat(fname)); }); }
+
 API long long bmh_nflops() { return Mat::nflops.load(); }
 API void bmh_flip() { flip(); }
 API double bmh_gflop(float* secs) { auto r = gflop(); if (secs) *secs = r.second; return r.first; }

@@ -31,7 +31,7 @@ def _load():
         L = C.CDLL(LIB_PATH)
         for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
                      "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
-                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop"):
+                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop", "bmh_load_gsmat"):
             getattr(L, name).restype = vp
         L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
         L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
@@ -41,6 +41,12 @@ def _load():
         L.bmh_dds.argtypes = [vp, vp, vp, vp]
         L.bmh_sdmult.argtypes = [vp, vp, vp, C.c_int]
         L.bmh_gsdop.argtypes = [vp, vp, vp, C.c_int]
+        L.bmh_load_gsmat.argtypes = [C.c_char_p]
+        ip = C.POINTER(C.c_int)
+        L.bmh_save_smat.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, vp, vp, vp]
+        L.bmh_load_smat.argtypes = [C.c_char_p, ip, ip, ip, vp, vp, vp]
+        L.bmh_save_fmat.argtypes = [C.c_char_p, C.c_int, C.c_int, vp]
+        L.bmh_load_fmat.argtypes = [C.c_char_p, ip, ip, vp]
         L.bmh_tile_mult.argtypes = [vp] + [C.c_int] * 5 + [vp, C.c_int, C.c_int, vp, C.c_int, C.c_int, C.c_int]
         L.bmh_sum_sparse.argtypes = [vp, C.c_int, vp]
         L.bmh_sum_dense.argtypes = [vp, C.c_int, vp]
@@ -257,6 +263,52 @@ def sum(a, n=0, out=None):      # noqa: A001  (the reference's name)
     if isinstance(a, GSMat):
         return a.sum(n, out)
     return GMat(_load().bmh_sum_dense(a._h, n, out._h if out else None))
+
+
+def saveSMat(fname, nrows, ncols, data, ir, jc):
+    """HMat.saveSMat: host SMat arrays (base Mat.ioneBased) to a type-231 file (0-based on disk)."""
+    data = np.ascontiguousarray(data, dtype=np.float32)
+    ir = np.ascontiguousarray(ir, dtype=np.int32)
+    jc = np.ascontiguousarray(jc, dtype=np.int32)
+    if _load().bmh_save_smat(os.fsencode(fname), nrows, ncols, data.size, data.ctypes.data, ir.ctypes.data, jc.ctypes.data) != 0:
+        raise RuntimeError(_load().bmh_last_error().decode())
+
+
+def loadSMat(fname):
+    """HMat.loadSMat: returns (nrows, ncols, data, ir, jc) with indices in base Mat.ioneBased."""
+    nr, nc, nnz = C.c_int(), C.c_int(), C.c_int()
+    L = _load()
+    if L.bmh_load_smat(os.fsencode(fname), C.byref(nr), C.byref(nc), C.byref(nnz), None, None, None) != 0:
+        raise RuntimeError(L.bmh_last_error().decode())
+    data = np.empty(nnz.value, np.float32)
+    ir = np.empty(nnz.value, np.int32)
+    jc = np.empty(nc.value + 1, np.int32)
+    if L.bmh_load_smat(os.fsencode(fname), C.byref(nr), C.byref(nc), C.byref(nnz), data.ctypes.data, ir.ctypes.data, jc.ctypes.data) != 0:
+        raise RuntimeError(L.bmh_last_error().decode())
+    return nr.value, nc.value, data, ir, jc
+
+
+def saveFMat(fname, a):
+    a = np.asfortranarray(a, dtype=np.float32)
+    flat = np.ascontiguousarray(a.ravel(order="F"))
+    if _load().bmh_save_fmat(os.fsencode(fname), a.shape[0], a.shape[1], flat.ctypes.data) != 0:
+        raise RuntimeError(_load().bmh_last_error().decode())
+
+
+def loadFMat(fname):
+    nr, nc = C.c_int(), C.c_int()
+    L = _load()
+    if L.bmh_load_fmat(os.fsencode(fname), C.byref(nr), C.byref(nc), None) != 0:
+        raise RuntimeError(L.bmh_last_error().decode())
+    out = np.empty(nr.value * nc.value, np.float32)
+    if L.bmh_load_fmat(os.fsencode(fname), C.byref(nr), C.byref(nc), out.ctypes.data) != 0:
+        raise RuntimeError(L.bmh_last_error().decode())
+    return out.reshape(nc.value, nr.value).T
+
+
+def loadGSMat(fname):
+    """A type-231 file straight onto the device (pinned, double-buffered upload)."""
+    return GSMat(_load().bmh_load_gsmat(os.fsencode(fname)))
 
 
 def smat_check(nrows, ncols, ir, jc):

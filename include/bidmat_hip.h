@@ -186,6 +186,9 @@ int bidmat_memcpy_d2d(void *dst, const void *src, long long bytes);
 int bidmat_memset(void *dptr, int value, long long bytes);
 int bidmat_mem_info(long long *free_bytes, long long *total_bytes);
 int bidmat_synchronize(void);
+/* Asynchronous copies between PINNED host memory (bidmat_host_alloc) and the device on a stream. */
+int bidmat_memcpy_h2d_async(void *dst, const void *src_pinned, long long bytes, void *stream);
+int bidmat_memcpy_d2h_async(void *dst_pinned, const void *src, long long bytes, void *stream);
 /* Pinned host staging buffers (allocated, never registered). */
 int bidmat_host_alloc(void **hptr, long long bytes);
 int bidmat_host_free(void *hptr);
