@@ -14,7 +14,9 @@ roofline object of the DDS kernel and the CPU baseline ride along.
 
 The other workloads (C1: A*S k=32; C4: A*S k=1024 with Pareto columns; C5: the NMF update
 chain at k=128, ~400 M nonzeros) are the remaining BASELINE.json configurations; they are
-parity-test cases and are timed only on request.
+parity-test cases and are timed only on request. "next" times the callers either side of the
+path on the headline pattern (tile products, S*A / S^T*A, sparse op edge vector, file load);
+"footprint" sweeps the gather kernels over the gathered footprint (where L1 / L2 / HBM serve).
 """
 import argparse
 import ctypes as C
@@ -60,7 +62,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="headline", choices=["headline", "C1", "C4", "C5"])
+    ap.add_argument("--workload", default="headline", choices=["headline", "C1", "C4", "C5", "next", "footprint"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows/columns of the pattern (testing)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-sample", type=float, default=1.0,
@@ -87,6 +89,11 @@ def main():
     cus = C.c_int(0)
     mem = C.c_longlong(0)
     hip_abi.check(lib.bidmat_device_info(arch, 64, C.byref(cus), C.byref(mem)))
+
+    if args.workload == "footprint":
+        return footprint_sweep(lib, args)
+    if args.workload == "next":
+        return next_rows(lib, args)
 
     t0 = time.time()
     cfg = gen.config("HEAD" if args.workload == "headline" else args.workload, args.scale)
@@ -258,6 +265,118 @@ def main():
         out["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_sample)
 
     print(json.dumps(out))
+
+
+def _timed(lib, fn, stream, reps, warm=2):
+    from bidmat_amd import hip_abi
+    for _ in range(warm):
+        hip_abi.check(fn())
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    hip_abi.check(lib.bidmat_event_create(C.byref(e0)))
+    hip_abi.check(lib.bidmat_event_create(C.byref(e1)))
+    hip_abi.check(lib.bidmat_event_record(e0, stream))
+    for _ in range(reps):
+        hip_abi.check(fn())
+    hip_abi.check(lib.bidmat_event_record(e1, stream))
+    hip_abi.check(lib.bidmat_stream_synchronize(stream))
+    hip_abi.check(lib.bidmat_synchronize())
+    ms = C.c_float(0)
+    hip_abi.check(lib.bidmat_event_elapsed_ms(e0, e1, C.byref(ms)))
+    return ms.value / reps
+
+
+def footprint_sweep(lib, args):
+    """DDS and A*S at k=256 on 100 000 columns x 200 nonzeros whose rows are uniform over R rows:
+    R KiB of gathered footprint, so the sweep shows what L1, L2, the Infinity Cache and HBM deliver."""
+    from bidmat_amd import hip_abi
+    from bidmat_amd.device import DeviceArray
+    k, ncols, L = 256, 100000, 200
+    nnz = ncols * L
+    rng = np.random.default_rng(0)
+    stream = C.c_void_p()
+    hip_abi.check(lib.bidmat_stream_create(C.byref(stream)))
+    d_A = DeviceArray.from_numpy(rng.random(k * (1 << 20), dtype=np.float32))
+    d_B = DeviceArray.from_numpy(rng.random(k * ncols, dtype=np.float32))
+    d_v = DeviceArray.from_numpy(rng.random(nnz, dtype=np.float32))
+    d_jc = DeviceArray.from_numpy((np.arange(ncols + 1) * L).astype(np.int32))
+    d_P, d_C = DeviceArray(nnz, np.float32), DeviceArray(k * ncols, np.float32)
+    rows = []
+    for R in (16, 64, 256, 1024, 2048, 4096, 8192, 16384, 65536, 262144, 1048576):
+        d_ir = DeviceArray.from_numpy(rng.integers(0, R, size=nnz).astype(np.int32))
+        t_dds = _timed(lib, lambda: lib.bidmat_dds_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_P.ptr, 0, stream), stream, 5)
+        t_as = _timed(lib, lambda: lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream), stream, 5)
+        b = nnz * (4 * k + 8)
+        rows.append({"rows": R, "footprint_KiB": R * k * 4 // 1024, "dds_ms": round(t_dds, 3),
+                     "dds_TBps": round(b / t_dds / 1e9, 2), "dsmult_ms": round(t_as, 3),
+                     "dsmult_TBps": round(b / t_as / 1e9, 2)})
+        d_ir.free()
+    print(json.dumps({"metric": "gather throughput vs gathered footprint (algorithmic TB/s), k=256, 20M nnz",
+                      "unit": "TB/s", "n_gpus": 1, "sweep": rows}))
+
+
+def next_rows(lib, args):
+    """The callers either side of the path, on the headline pattern (k = p = 256)."""
+    import tempfile
+    from bidmat_amd import gen, hip_abi, mats
+    from bidmat_amd.device import DeviceArray
+    cfg = gen.config("HEAD", args.scale)
+    k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
+    ir, jc, vals = cfg["ir"], cfg["jc"], cfg["vals"]
+    nnz = int(ir.size)
+    stream = None            # these entries are the blocking, reference-shaped ones or take the default stream
+    d_ir, d_jc, d_v = DeviceArray.from_numpy(ir), DeviceArray.from_numpy(jc), DeviceArray.from_numpy(vals)
+    d_ic = DeviceArray(nnz, np.int32)
+    hip_abi.check(lib.bidmat_csc_expand_cols(ncols, nnz, d_jc.ptr, d_ic.ptr, None))
+    d_A, d_AT = DeviceArray.from_numpy(cfg["A"]), DeviceArray.from_numpy(cfg["A_T"])
+    d_C, d_G = DeviceArray(k * ncols, np.float32), DeviceArray(k * nrows, np.float32)
+    hip_abi.check(lib.bidmat_memset(d_C.ptr, 0, d_C.nbytes))
+    hip_abi.check(lib.bidmat_memset(d_G.ptr, 0, d_G.nbytes))
+    out = {}
+    reps = max(1, args.steps // 2)
+    # tile products over the middle half of the rows and columns (reference-shaped, blocking)
+    r0, nr_, c0, nc_ = nrows // 4, nrows // 2, ncols // 4, ncols // 2
+    inside = int(np.count_nonzero((ir[jc[c0]:jc[c0 + nc_]] >= r0) & (ir[jc[c0]:jc[c0 + nc_]] < r0 + nr_)))
+    t = _timed(lib, lambda: lib.bidmat_dsmultTile(k, nc_, nr_, nnz, d_A.ptr + 4 * k * r0, k, d_v.ptr, d_ir.ptr, d_ic.ptr,
+                                                   r0, c0, d_C.ptr, k), stream, reps, 1)
+    out["dsmultTile"] = {"ms": round(t, 3), "nnz_in_tile": inside, "GBps": round((inside * 4 * k + int(jc[c0 + nc_] - jc[c0]) * 8 + nc_ * 4 * k) / t / 1e6, 1)}
+    t = _timed(lib, lambda: lib.bidmat_dsmultTileT(k, nr_, nc_, nnz, d_AT.ptr + 4 * k * c0, k, d_v.ptr, d_ir.ptr, d_ic.ptr,
+                                                    r0, c0, d_G.ptr, k), stream, reps, 1)
+    out["dsmultTileT"] = {"ms": round(t, 3), "nnz_in_tile": inside, "GBps": round((inside * 4 * k + nnz * 8 + nr_ * 4 * k) / t / 1e6, 1)}
+    # S^T * A and S * A with p = 256 dense columns
+    p = k
+    plan = C.c_void_p()
+    hip_abi.check(lib.bidmat_plan_create(nrows, ncols, nnz, d_ir.ptr, d_jc.ptr, p, C.byref(plan)))
+    d_X = DeviceArray.from_numpy(gen.normal(nrows * p, 71))
+    d_Y = DeviceArray(ncols * p, np.float32)
+    t = _timed(lib, lambda: lib.bidmat_sdtmult_csc(nrows, ncols, nnz, p, d_v.ptr, d_ir.ptr, d_jc.ptr, d_X.ptr, nrows, d_Y.ptr, ncols, None), stream, reps, 1)
+    b = alg_bytes("dsmult", p, nnz, nrows, ncols) + 8 * p * (nrows + ncols)
+    out["SDTMult (S^T*A)"] = {"ms": round(t, 3), "GBps": round(b / t / 1e6, 1)}
+    t = _timed(lib, lambda: lib.bidmat_sdmult_plan(plan, p, d_v.ptr, d_Y.ptr, ncols, d_X.ptr, nrows, None), stream, reps, 1)
+    b = alg_bytes("dsmultT", p, nnz, nrows, ncols) + 8 * p * (nrows + ncols)
+    out["SDMult (S*A)"] = {"ms": round(t, 3), "GBps": round(b / t / 1e6, 1)}
+    # sparse op edge vectors (in place on a copy of the values)
+    d_w = DeviceArray.from_numpy(vals)
+    d_row, d_col = DeviceArray.from_numpy(gen.uniform(ncols, 72, 0.5, 1.5)), DeviceArray.from_numpy(gen.uniform(nrows, 73, 0.5, 1.5))
+    t = _timed(lib, lambda: lib.bidmat_sdoprow(nrows, ncols, nnz, d_w.ptr, d_ic.ptr, d_row.ptr, ncols, 2), stream, reps, 1)
+    out["sdoprow"] = {"ms": round(t, 3), "GBps": round(12.0 * nnz / t / 1e6, 1)}
+    t = _timed(lib, lambda: lib.bidmat_sdopcol(nrows, ncols, nnz, d_w.ptr, d_ir.ptr, d_col.ptr, nrows, 2), stream, reps, 1)
+    out["sdopcol"] = {"ms": round(t, 3), "GBps": round(12.0 * nnz / t / 1e6, 1)}
+    # file -> device (pinned, double-buffered) against host arrays -> device (pageable copies)
+    with tempfile.TemporaryDirectory() as tmp:
+        f = os.path.join(tmp, "pattern.smat")
+        mats.saveSMat(f, nrows, ncols, vals, ir + 1, jc + 1)
+        size = os.path.getsize(f)
+        t0 = time.perf_counter()
+        g = mats.loadGSMat(f)
+        t_load = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        g2 = mats.GSMat.from_csc(nrows, ncols, vals, ir + 1, jc + 1)
+        t_from = time.perf_counter() - t0
+        out["loadGSMat"] = {"file_GB": round(size / 1e9, 3), "s": round(t_load, 3), "GBps": round(size / t_load / 1e9, 2)}
+        out["GSMat.fromSMat"] = {"s": round(t_from, 3), "GBps": round(size / t_from / 1e9, 2)}
+        del g, g2
+    print(json.dumps({"metric": "callers either side of the path on the headline pattern", "unit": "GB/s", "n_gpus": 1,
+                      "config": {"k": k, "nrows": nrows, "ncols": ncols, "nnz": nnz, "scale": args.scale}, "ops": out}))
 
 
 def cpu_baseline(workload, cfg, frac):
