@@ -357,6 +357,7 @@ EXPORT void oracle_spsum_f64(int nrows, int ncols, const float *data, const int 
                              const int *jc, int ioff, int dim, double *ref, double *sumabs)
 {
     int i, j;
+    (void)nrows;
     for (i = 0; i < ncols; i++) {
         for (j = jc[i] - ioff; j < jc[i + 1] - ioff; j++) {
             int o = (dim == 1) ? i : ir[j] - ioff;
