@@ -20,14 +20,29 @@ struct DevBuf {
 };
 
 
+// Row histogram. The first HIST_LDS_ROWS rows are counted in a per-workgroup LDS copy that is
+// flushed once at the end (popular rows tend to carry small indices in count-sorted vocabularies,
+// and even when they do not this only costs the flush); all other rows go straight to global
+// integer atomics. The counts do not depend on the order of the increments.
+constexpr int HIST_LDS_ROWS = 16384;
 __global__ __launch_bounds__(BM_BLOCK) void k_row_hist(int nnz, int nrows, const int* __restrict__ ir,
                                                        int* __restrict__ cnt, int* __restrict__ bad) {
+    __shared__ int local[HIST_LDS_ROWS];
+    for (int i = threadIdx.x; i < HIST_LDS_ROWS; i += BM_BLOCK) local[i] = 0;
+    __syncthreads();
     long long j = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long stride = (long long)gridDim.x * BM_BLOCK;
     for (; j < nnz; j += stride) {
         const int r = ir[j];
         if (r < 0 || r >= nrows) *bad = 1;
+        else if (r < HIST_LDS_ROWS) atomicAdd(&local[r], 1);
         else atomicAdd(&cnt[r], 1);
+    }
+    __syncthreads();
+    const int lim = nrows < HIST_LDS_ROWS ? nrows : HIST_LDS_ROWS;
+    for (int i = threadIdx.x; i < lim; i += BM_BLOCK) {
+        const int v = local[i];
+        if (v) atomicAdd(&cnt[i], v);
     }
 }
 
@@ -83,7 +98,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __re
                                                    const int* __restrict__ hrow, int nheavy, int p8,
                                                    int* __restrict__ pc, int* __restrict__ segstart,
                                                    unsigned* __restrict__ segrow, int* __restrict__ segid,
-                                                   int* __restrict__ class_count) {
+                                                   unsigned char* __restrict__ segclass) {
     long long p = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long stride = (long long)gridDim.x * BM_BLOCK;
     const unsigned per_xcd = (unsigned)p8 * (unsigned)nheavy;     // keys per XCD group
@@ -96,10 +111,20 @@ __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __re
             segstart[sidx] = (int)p;
             segrow[sidx] = key >= light_base ? key - light_base : (unsigned)hrow[key % (unsigned)nheavy];
             segid[sidx] = sidx;
-            // segments per XCD group (integer atomics: the counts do not depend on the order)
-            atomicAdd(&class_count[key >= light_base ? 8 : (int)(key / per_xcd)], 1);
+            segclass[sidx] = (unsigned char)(key >= light_base ? 8 : (int)(key / per_xcd));
         }
     }
+}
+
+// Segments are sorted by key, so their XCD class is non-decreasing: class c starts at the first
+// segment whose class is >= c. start[0..8] must be preset to nseg.
+__global__ __launch_bounds__(BM_BLOCK) void k_class_bounds(int nseg, const unsigned char* __restrict__ segclass,
+                                                           int* __restrict__ start) {
+    const long long s = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    if (s >= nseg) return;
+    const int cls = segclass[s];
+    const int prev = s == 0 ? -1 : (int)segclass[s - 1];
+    for (int c = prev + 1; c <= cls; ++c) start[c] = (int)s;
 }
 
 inline unsigned grid_for(long long n, int maxblocks = 16384) {
@@ -185,7 +210,8 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     // 1. row histogram (integer atomics: the counts do not depend on the order)
     PB_CHECK(fill_i32(cnt.as<int>(), nrows, 0, s));
     PB_CHECK(fill_i32(bad.as<int>(), 1, 0, s));
-    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, nrows, ir, cnt.as<int>(), bad.as<int>());
+    // few, long-lived workgroups: every one flushes its LDS histogram once at the end
+    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, ir, cnt.as<int>(), bad.as<int>());
     int h_bad = 0;
     PB_CHECK(hipMemcpy(&h_bad, bad.p, sizeof(int), hipMemcpyDeviceToHost));
     if (h_bad) { (void)plan_free(plan); return hipErrorInvalidValue; }
@@ -247,8 +273,10 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     plan->nseg = nseg;
 
     DevBuf segid, segrow_sorted, class_count;
+    DevBuf segclass;
     PB_CHECK(class_count.alloc(sizeof(int) * 9));
-    PB_CHECK(fill_i32(class_count.as<int>(), 9, 0, s));
+    PB_CHECK(fill_i32(class_count.as<int>(), 9, nseg, s));
+    PB_CHECK(segclass.alloc((size_t)(nseg > 0 ? nseg : 1)));
     PB_CHECK(hipMalloc((void**)&plan->segrow, sizeof(int) * (size_t)(nseg > 0 ? nseg : 1)));
     unsigned* const segrow_u = reinterpret_cast<unsigned*>(plan->segrow);
     PB_CHECK(segid.alloc(sizeof(int) * (size_t)nseg));
@@ -259,14 +287,11 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out.as<unsigned>(), plan->perm,
                        ic.as<int>(), flag.as<int>(), segidx.as<int>(), hrow.as<int>(), nheavy > 0 ? nheavy : 1,
                        nheavy > 0 ? p8 : 0, plan->pc, plan->segstart, segrow_u, segid.as<int>(),
-                       class_count.as<int>());
+                       segclass.as<unsigned char>());
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
-    {
-        int h_count[9];
-        PB_CHECK(hipMemcpy(h_count, class_count.p, sizeof(h_count), hipMemcpyDeviceToHost));
-        plan->xcd_start[0] = 0;
-        for (int x = 0; x < 8; ++x) plan->xcd_start[x + 1] = plan->xcd_start[x] + h_count[x];
-    }
+    hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg,
+                       segclass.as<unsigned char>(), class_count.as<int>());
+    PB_CHECK(hipMemcpy(plan->xcd_start, class_count.p, sizeof(int) * 9, hipMemcpyDeviceToHost));
 
     // 5. a row's segments, in ascending segment order (stable sort by row)
     {
