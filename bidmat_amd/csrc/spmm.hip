@@ -375,8 +375,8 @@ hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, co
     if (rowsel.on) { a.segrow = segrow; a.row_off = rowsel.off; a.row_len = rowsel.len; }
     int maxheavy = 0;
     for (int x = 0; x < 9; ++x) a.xcd_start[x] = xcd_start[x];
-    for (int x = 0; x < 8; ++x) maxheavy = std::max(maxheavy, xcd_start[x + 1] - xcd_start[x]);
-    const long long nlight = (long long)nseg - xcd_start[8];
+    for (int x = 0; x < 8; ++x) maxheavy = std::max(maxheavy, a.xcd_start[x + 1] - a.xcd_start[x]);
+    const long long nlight = (long long)nseg - a.xcd_start[8];
     // waves per XCD, rounded up to whole workgroups, times 8 XCDs
     const long long per_xcd = (long long)maxheavy + (nlight + 7) / 8;
     const long long blocks_per_xcd = (per_xcd + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
