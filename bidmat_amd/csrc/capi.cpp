@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <list>
+#include <memory>
 #include <mutex>
 
 #define API extern "C" __attribute__((visibility("default")))
@@ -47,14 +48,16 @@ struct CacheEntry {
     int device;
     int ncols, nnz, nrows, k_hint;
     unsigned long long fa, fb;
-    bidmat_plan* plan;
+    std::shared_ptr<bidmat_plan> plan;      // callers hold a reference while they use the plan
 };
+using PlanRef = std::shared_ptr<bidmat_plan>;
+PlanRef own(bidmat_plan* p) { return PlanRef(p, [](bidmat_plan* q) { (void)bm::plan_free(q); }); }
 std::mutex g_cache_mu;
 std::list<CacheEntry> g_cache;          // most recently used first
 constexpr size_t kMaxCachedPlans = 4;
 
-hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_hint, bidmat_plan** out) {
-    *out = nullptr;
+hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_hint, PlanRef* out) {
+    out->reset();
     hipError_t err;
     int dev = 0;
     if ((err = hipGetDevice(&dev)) != hipSuccess) return err;
@@ -85,12 +88,9 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     if ((err = bm::coo_compress_cols(ncols, nnz, ic, jc, s)) != hipSuccess) return err;
     bidmat_plan* p = nullptr;
     if ((err = bm::plan_build(nrows, ncols, nnz, ir, jc, k_hint, &p)) != hipSuccess) return err;
-    while (g_cache.size() >= kMaxCachedPlans) {
-        (void)bm::plan_free(g_cache.back().plan);
-        g_cache.pop_back();
-    }
-    g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, h[0], h[1], p});
-    *out = p;
+    while (g_cache.size() >= kMaxCachedPlans) g_cache.pop_back();   // freed when its last user lets go
+    g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, h[0], h[1], own(p)});
+    *out = g_cache.front().plan;
     return hipSuccess;
 }
 
@@ -138,9 +138,9 @@ API int bidmat_dsmultT(int nrows, int ncols, int nnz, const float* A, const floa
     if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
     if (nrows == 0 || ncols == 0 || nnz == 0) return 0;
     if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
-    bidmat_plan* plan = nullptr;
+    PlanRef plan;
     hipError_t err = cached_plan(ncols, nnz, Bir, Bic, nrows, &plan);
-    if (err == hipSuccess) err = run_dsmultT(plan, nrows, A, Bdata, C, 1, nullptr);
+    if (err == hipSuccess) err = run_dsmultT(plan.get(), nrows, A, Bdata, C, 1, nullptr);
     return finish_blocking(err);
 }
 
@@ -174,12 +174,12 @@ API int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float* A, int 
     hipError_t err = hipMemcpy(&last, Bic + (nnz - 1), sizeof(int), hipMemcpyDeviceToHost);
     if (err != hipSuccess) return (int)err;
     if (last < 0 || last == 0x7fffffff) return kInvalid;
-    bidmat_plan* plan = nullptr;
+    PlanRef plan;
     err = cached_plan(last + 1, nnz, Bir, Bic, nr, &plan);
     if (err != hipSuccess) return finish_blocking(err);
     if (broff >= plan->nrows) return 0;                  // the tile holds no stored row
     const int nrows_eff = nc < plan->nrows - broff ? nc : plan->nrows - broff;
-    err = bm::plan_reserve_partial(plan, nr);
+    err = bm::plan_reserve_partial(plan.get(), nr);
     if (err == hipSuccess)
         err = bm::gather_segments_ex(nr, lda, plan->nseg, plan->xcd_start, A, Bdata, plan->pc, plan->perm,
                                      plan->segstart, plan->partial, bm::Window{1, bcoff, kk}, plan->segrow,
@@ -235,10 +235,10 @@ API int bidmat_spsum(int nrows, int ncols, int nnz, const int* Air, const int* A
         err = bm::coo_compress_cols(ncols, nnz, Aic, jc, nullptr);
         if (err == hipSuccess) err = bm::spsum_cols(ncols, nnz, P, jc, B, 1, nullptr);
     } else {
-        bidmat_plan* plan = nullptr;
+        PlanRef plan;
         err = cached_plan(ncols, nnz, Air, Aic, 0, &plan);
         if (err == hipSuccess && plan->nrows > nrows) err = hipErrorInvalidValue;   // row index outside B
-        if (err == hipSuccess) err = run_spsum_rows(plan, P, B, 1, nullptr);
+        if (err == hipSuccess) err = run_spsum_rows(plan.get(), P, B, 1, nullptr);
     }
     return finish_blocking(err);
 }
@@ -541,7 +541,7 @@ API int bidmat_release_caches(void) {
     {
         std::lock_guard<std::mutex> lock(g_cache_mu);
         for (auto it = g_cache.begin(); it != g_cache.end();) {
-            if (it->device == dev) { (void)bm::plan_free(it->plan); it = g_cache.erase(it); }
+            if (it->device == dev) it = g_cache.erase(it);
             else ++it;
         }
     }
