@@ -47,21 +47,26 @@ struct GatherArgs {
 template <int V, int LPN>
 struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw < 1 ? 1 : (raw > LPN ? LPN : raw); };
 
-template <int W, int V, int LPN, bool PLAN, bool FULL, bool TILE>
-__device__ __forceinline__ void gather_chunk(const GatherArgs& a, int j0, int rem, int g, int l,
-                                             const int (&eld)[V], Vec<W> (&acc)[V]) {
-    constexpr int NG = 64 / LPN;
-    constexpr int U = Unroll<V, LPN>::U;
-    // lane (g,l) holds nonzero q = l*NG + g of the chunk, so group g meets its nonzeros
-    // q = it*NG + g in lane l == it of its own group.
-    const int q = l * NG + g;
-    int myrow = 0;
-    float myval = 0.f;
-    if (FULL || q < rem) {
-        const int p = j0 + q;
+// Loads this lane's nonzero of a chunk: lane (g,l) holds nonzero q = l*NG + g, so group g meets
+// its nonzeros q = it*NG + g in lane l == it of its own group. Lanes past `rem` keep (0, 0).
+template <bool PLAN>
+__device__ __forceinline__ void load_chunk(const GatherArgs& a, int j0, int ahead, int rem, int q, int& myrow,
+                                           float& myval) {
+    myrow = 0;
+    myval = 0.f;
+    if (q < rem) {
+        const int p = j0 + ahead + q;
         myrow = a.idx[p];
         myval = PLAN ? a.vals[a.perm[p]] : a.vals[p];
     }
+}
+
+template <int W, int V, int LPN, bool FULL, bool TILE>
+__device__ __forceinline__ void gather_chunk(const GatherArgs& a, int myrow, float myval, int rem, int g, int l,
+                                             const int (&eld)[V], Vec<W> (&acc)[V]) {
+    constexpr int NG = 64 / LPN;
+    constexpr int U = Unroll<V, LPN>::U;
+    const int q = l * NG + g;
     unsigned long long inmask = ~0ULL;
     if (TILE) {
         // window filter: nonzeros outside the tile contribute nothing (their lane keeps index 0)
@@ -72,6 +77,9 @@ __device__ __forceinline__ void gather_chunk(const GatherArgs& a, int j0, int re
         inmask = __ballot(inside);
     }
     const int niter = FULL ? LPN : (rem + NG - 1) / NG;
+    // One round of U gathers at a time: unrolled further, the compiler hoists every load of the
+    // chunk and the register count collapses the occupancy (256 VGPRs at LPN = 32).
+#pragma unroll 1
     for (int it0 = 0; it0 < niter; it0 += U) {
         Vec<W> av[U][V];
         float vv[U];
@@ -187,13 +195,28 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
             eld[i] = ev[i] ? est[i] : 0;     // lanes past k re-read element 0; never stored
             acc[i] = Vec<W>::zero();
         }
-        int j0 = jstart;
-        if (a.win_on) {
-            for (; j0 + 64 <= jend; j0 += 64) gather_chunk<W, V, LPN, PLAN, true, true>(a, j0, 64, g, l, eld, acc);
-            if (j0 < jend) gather_chunk<W, V, LPN, PLAN, false, true>(a, j0, jend - j0, g, l, eld, acc);
-        } else {
-            for (; j0 + 64 <= jend; j0 += 64) gather_chunk<W, V, LPN, PLAN, true, false>(a, j0, 64, g, l, eld, acc);
-            if (j0 < jend) gather_chunk<W, V, LPN, PLAN, false, false>(a, j0, jend - j0, g, l, eld, acc);
+        // The next chunk's indices and values are requested before the current chunk's gathers,
+        // so their latency overlaps the gathers instead of preceding them.
+        const int q = l * (64 / LPN) + g;
+        int rem = jend - jstart, j0 = jstart;
+        int crow;
+        float cval;
+        load_chunk<PLAN>(a, j0, 0, rem, q, crow, cval);
+        while (rem > 0) {
+            int nrow;
+            float nval;
+            load_chunk<PLAN>(a, j0, 64, rem - 64, q, nrow, nval);
+            if (a.win_on) {
+                if (rem >= 64) gather_chunk<W, V, LPN, true, true>(a, crow, cval, 64, g, l, eld, acc);
+                else gather_chunk<W, V, LPN, false, true>(a, crow, cval, rem, g, l, eld, acc);
+            } else {
+                if (rem >= 64) gather_chunk<W, V, LPN, true, false>(a, crow, cval, 64, g, l, eld, acc);
+                else gather_chunk<W, V, LPN, false, false>(a, crow, cval, rem, g, l, eld, acc);
+            }
+            crow = nrow;
+            cval = nval;
+            j0 += 64;
+            rem -= 64;
         }
 
 #pragma unroll
@@ -255,7 +278,16 @@ __global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int ldc, in
     for (int el = l * W; el < k; el += lpr * W) {
         float* o = C + (size_t)row * ldc + el;
         Vec<W> acc = beta ? Vec<W>::load(o) : Vec<W>::zero();
-        for (int q = s; q < e; ++q) acc.add(Vec<W>::load(partial + (size_t)rowseg[q] * k + el));
+        // eight partials in flight at a time; the additions keep their segment order
+        int q = s;
+        for (; q + 8 <= e; q += 8) {
+            Vec<W> p[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) p[u] = Vec<W>::load(partial + (size_t)rowseg[q + u] * k + el);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc.add(p[u]);
+        }
+        for (; q < e; ++q) acc.add(Vec<W>::load(partial + (size_t)rowseg[q] * k + el));
         acc.store(o);
     }
 }
