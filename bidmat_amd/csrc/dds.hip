@@ -31,14 +31,12 @@ template <int V, int LPN>
 struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw < 1 ? 1 : (raw > LPN ? LPN : raw); };
 
 template <int W, int V, int LPN, bool EXACT, bool FULL>
-__device__ __forceinline__ void dds_chunk(const DdsArgs& a, int j0, int rem, int g, int l,
+__device__ __forceinline__ void dds_chunk(const DdsArgs& a, int myrow, int j0, int rem, int g, int l,
                                           const int (&eld)[V], const bool (&ev)[V],
                                           const Vec<W> (&b)[V], bool accumulate) {
     constexpr int NG = 64 / LPN;
     constexpr int U = Unroll<V, LPN>::U;
     const int q = l * NG + g;            // the nonzero of this chunk whose result this lane keeps
-    int myrow = 0;
-    if (FULL || q < rem) myrow = a.ir[j0 + q];
     float res = 0.f;
     const int niter = FULL ? LPN : (rem + NG - 1) / NG;
     for (int it0 = 0; it0 < niter; it0 += U) {
@@ -116,10 +114,18 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
             b[i] = ev[i] ? Vec<W>::load(bp + e) : Vec<W>::zero();
         }
         const bool accumulate = (a.beta != 0) || (k0 > 0);
-        int j0 = jstart;
-        for (; j0 + 64 <= jend; j0 += 64)
-            dds_chunk<W, V, LPN, EXACT, true>(a, j0, 64, g, l, eld, ev, b, accumulate);
-        if (j0 < jend) dds_chunk<W, V, LPN, EXACT, false>(a, j0, jend - j0, g, l, eld, ev, b, accumulate);
+        // The next chunk's row indices are requested before the current chunk's gathers.
+        const int q = l * (64 / LPN) + g;
+        int j0 = jstart, rem = jend - jstart;
+        int crow = (q < rem) ? a.ir[j0 + q] : 0;
+        while (rem > 0) {
+            const int nrow = (q < rem - 64) ? a.ir[j0 + 64 + q] : 0;
+            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a, crow, j0, 64, g, l, eld, ev, b, accumulate);
+            else dds_chunk<W, V, LPN, EXACT, false>(a, crow, j0, rem, g, l, eld, ev, b, accumulate);
+            crow = nrow;
+            j0 += 64;
+            rem -= 64;
+        }
     }
 }
 
