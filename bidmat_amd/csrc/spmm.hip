@@ -254,6 +254,38 @@ __global__ __launch_bounds__(BM_BLOCK) void k_overflow_reduce(int k, int ldc, in
     }
 }
 
+// Overflow table of a small or medium matrix in two launches: out[c] = number of extra segments
+// in the columns before c, out[ncols] = their total. Pass 1 scans each block of 256 columns and
+// leaves block-local prefixes and block totals; in pass 2 every block sums the totals of the blocks
+// before it (at most OVF2_MAX_BLOCKS of them) and shifts its prefixes.
+constexpr int OVF2_MAX_BLOCKS = 1024;
+__global__ __launch_bounds__(BM_BLOCK) void k_overflow_local(int ncols, const int* __restrict__ jc, int seglen,
+                                                             int* __restrict__ out, int* __restrict__ bsum) {
+    __shared__ int smem[8];
+    const long long c = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    int extra = 0;
+    if (c < ncols) {
+        const int len = jc[c + 1] - jc[c];
+        if (len > seglen) extra = (len - 1) / seglen;
+    }
+    int total;
+    const int ex = block_exclusive_scan_256(extra, total, smem);
+    if (c < ncols) out[c] = ex;
+    if (threadIdx.x == 0) bsum[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(BM_BLOCK) void k_overflow_shift(int ncols, int* __restrict__ out,
+                                                             const int* __restrict__ bsum) {
+    __shared__ int smem[8];
+    int before = 0;
+    for (int b = threadIdx.x; b < (int)blockIdx.x; b += BM_BLOCK) before += bsum[b];
+    int total;
+    (void)block_exclusive_scan_256(before, total, smem);      // total = sum over the whole block
+    const long long c = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    if (c < ncols) out[c] += total;
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) out[ncols] = total + bsum[blockIdx.x];
+}
+
 __global__ __launch_bounds__(BM_BLOCK) void k_extra_segments(int ncols, const int* __restrict__ jc, int seglen,
                                                              int* __restrict__ extra) {
     const long long c = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
@@ -329,11 +361,18 @@ hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, i
     hipError_t err;
     int* buf = (int*)ws_get(WS_OVF, sizeof(int) * (2 * (size_t)ncols + 2), &err);
     if (!buf) return err;
+    unsigned nblk = (unsigned)(((long long)ncols + BM_BLOCK - 1) / BM_BLOCK);
+    if (nblk <= (unsigned)OVF2_MAX_BLOCKS) {
+        int* bsum = buf + ncols + 1;
+        hipLaunchKernelGGL(k_overflow_local, dim3(nblk), dim3(BM_BLOCK), 0, s, ncols, jc, seglen, buf, bsum);
+        hipLaunchKernelGGL(k_overflow_shift, dim3(nblk), dim3(BM_BLOCK), 0, s, ncols, buf, bsum);
+        *d_ovf = buf;
+        return hipGetLastError();
+    }
     int* tmp = (int*)ws_get(WS_SCAN, sizeof(int) * scan_tmp_ints(ncols), &err);
     if (!tmp) return err;
     int* extra = buf;
     int* ovf = buf + ncols + 1;
-    unsigned nblk = (unsigned)(((long long)ncols + BM_BLOCK - 1) / BM_BLOCK);
     hipLaunchKernelGGL(k_extra_segments, dim3(nblk), dim3(BM_BLOCK), 0, s, ncols, jc, seglen, extra);
     err = scan_exclusive_i32(extra, ovf, ncols, tmp, s);
     if (err != hipSuccess) return err;
