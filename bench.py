@@ -236,6 +236,11 @@ def main():
         "bytes_per_launch": r_bytes, "avg_launch_ms": round(r_avg, 4),
     }
 
+    if roofline["traffic"]:
+        # the kernel's measured HBM-side rate: the utilisation figure that cannot exceed 1
+        roofline["traffic_GBps"] = round(roofline["traffic"] / r_avg / 1e6, 1)
+        roofline["traffic_frac"] = round(roofline["traffic"] / r_avg / 1e6 / HBM_PEAK_GBS, 4)
+
     out = {
         "metric": metric, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,

@@ -76,7 +76,9 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
 
     std::lock_guard<std::mutex> lock(g_cache_mu);
     for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
-        if (it->device == dev && it->ncols == ncols && it->nnz == nnz && it->nrows == nrows &&
+        // panels are sized for k_hint: a request that names k only takes a plan built for that k
+        const bool k_ok = k_hint <= 0 || (it->k_hint > 0 ? it->k_hint : 256) == k_hint;
+        if (k_ok && it->device == dev && it->ncols == ncols && it->nnz == nnz && it->nrows == nrows &&
             it->fa == h[0] && it->fb == h[1]) {
             g_cache.splice(g_cache.begin(), g_cache, it);
             *out = g_cache.front().plan;
