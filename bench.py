@@ -123,14 +123,19 @@ def main():
     d_v = up(cfg["vals"])
     keep = [d_ir, d_jc, d_v]
     plan = C.c_void_p()
-    t_plan = [None]
+    t_plan = [None, None]
 
     def build_plan():
-        hip_abi.check(lib.bidmat_synchronize())
-        t = time.time()
-        hip_abi.check(lib.bidmat_plan_create(nrows, ncols, nnz, d_ir.ptr, d_jc.ptr, k, C.byref(plan)), "plan_create")
-        hip_abi.check(lib.bidmat_synchronize())
-        t_plan[0] = time.time() - t
+        # first build in the process (pays one-off costs: kernel loading, workspace growth), then
+        # the build a caller sees from the second pattern on
+        for i in range(2):
+            if plan.value:
+                hip_abi.check(lib.bidmat_plan_destroy(plan))
+            hip_abi.check(lib.bidmat_synchronize())
+            t = time.time()
+            hip_abi.check(lib.bidmat_plan_create(nrows, ncols, nnz, d_ir.ptr, d_jc.ptr, k, C.byref(plan)), "plan_create")
+            hip_abi.check(lib.bidmat_synchronize())
+            t_plan[i] = time.time() - t
 
     # ---- the ops of one step: (name, kind, launcher)
     if args.workload == "headline":
@@ -258,7 +263,7 @@ def main():
                 "step_GBps_incl_h2d": round(total_bytes / (ms_per_step * 1e-3 + h2d["s"]) / 1e9, 1)},
     }
     if t_plan[0] is not None:
-        out["plan"] = {"build_ms": round(t_plan[0] * 1e3, 2), "segments": lib.bidmat_plan_segments(plan),
+        out["plan"] = {"first_build_ms": round(t_plan[0] * 1e3, 2), "build_ms": round(t_plan[1] * 1e3, 2), "segments": lib.bidmat_plan_segments(plan),
                        "bytes": lib.bidmat_plan_bytes(plan)}
     if args.workload == "C5":      # the dense row sums of H, timed apart from the chain
         e0, e1 = ev(), ev()

@@ -74,6 +74,79 @@ __device__ __forceinline__ float group_allsum(float x) {
     return x;
 }
 
+// Sums U values per lane over aligned groups of N lanes at once (U in {2,4,8}, N >= 8, N >= U).
+// The first log2(U) butterfly steps are "transposed": instead of every lane adding up all U
+// values, partners split them, each keeping the half selected by one bit of its slot label, so
+// the work halves per step; the remaining steps are a plain butterfly on the one value left.
+// Afterwards lane l holds the complete group sum of slot slot_label(l). Every sum is formed by
+// the same tree of additions as group_allsum<N>, so the bits are the same.
+//
+// The steps' partners are lane^1, lane^2, 7-lane (within 8), 15-lane (within 16), lane^16,
+// lane^32. A label whose bit t flips exactly under step t and under no later step is
+//   bit0 = l0 ^ l2, bit1 = l1 ^ l2, bit2 = l2 ^ l3          (l0..l3 = low bits of the lane).
+__device__ __forceinline__ int slot_label(int l) {
+    return ((l ^ (l >> 2)) & 1) | ((((l >> 1) ^ (l >> 2)) & 1) << 1) | ((((l >> 2) ^ (l >> 3)) & 1) << 2);
+}
+// Which of the U consecutive lanes it0 .. it0+U-1 (it0 a multiple of U) carries slot u.
+template <int U>
+__device__ __forceinline__ int slot_offset(int u, int it0) {
+    if constexpr (U == 8) {
+        const int b3 = (it0 >> 3) & 1;
+        const int b2 = ((u >> 2) & 1) ^ b3, b0 = (u & 1) ^ b2, b1 = ((u >> 1) & 1) ^ b2;
+        return b0 | (b1 << 1) | (b2 << 2);
+    } else if constexpr (U == 4) {
+        const int b2 = (it0 >> 2) & 1;
+        return ((u & 1) ^ b2) | ((((u >> 1) & 1) ^ b2) << 1);
+    } else if constexpr (U == 2) {
+        return (u & 1) ^ ((it0 >> 2) & 1);
+    } else {
+        return 0;
+    }
+}
+template <int N, int U>
+__device__ __forceinline__ float group_multisum(const float (&s)[U], int label) {
+    static_assert(U == 2 || U == 4 || U == 8, "U must be 2, 4 or 8");
+    static_assert(N >= 8 && N >= U, "group too small");
+    float a[U / 2];
+    {
+        const bool hi = label & 1;
+#pragma unroll
+        for (int i = 0; i < U / 2; ++i) {
+            const float keep = hi ? s[2 * i + 1] : s[2 * i];
+            const float send = hi ? s[2 * i] : s[2 * i + 1];
+            a[i] = keep + dpp_mov<DPP_QUAD_XOR1>(send);
+        }
+    }
+    float x;
+    if constexpr (U >= 4) {
+        float b[U / 4];
+        const bool hi = label & 2;
+#pragma unroll
+        for (int i = 0; i < U / 4; ++i) {
+            const float keep = hi ? a[2 * i + 1] : a[2 * i];
+            const float send = hi ? a[2 * i] : a[2 * i + 1];
+            b[i] = keep + dpp_mov<DPP_QUAD_XOR2>(send);
+        }
+        if constexpr (U == 8) {
+            const bool hi2 = label & 4;
+            const float keep = hi2 ? b[1] : b[0];
+            const float send = hi2 ? b[0] : b[1];
+            x = keep + dpp_mov<DPP_ROW_HALF_MIRROR>(send);
+        } else {
+            x = b[0];
+            x += dpp_mov<DPP_ROW_HALF_MIRROR>(x);
+        }
+    } else {
+        x = a[0];
+        x += dpp_mov<DPP_QUAD_XOR2>(x);
+        x += dpp_mov<DPP_ROW_HALF_MIRROR>(x);
+    }
+    if (N >= 16) x += dpp_mov<DPP_ROW_MIRROR>(x);
+    if (N >= 32) x += __shfl_xor(x, 16, 64);
+    if (N >= 64) x += __shfl_xor(x, 32, 64);
+    return x;
+}
+
 // Read lane `src` (a wave-uniform or per-lane index) of x.
 __device__ __forceinline__ int lane_read(int x, int src) { return __shfl(x, src, 64); }
 __device__ __forceinline__ float lane_read(float x, int src) { return __shfl(x, src, 64); }

@@ -31,26 +31,31 @@ template <int V, int LPN>
 struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw < 1 ? 1 : (raw > LPN ? LPN : raw); };
 
 template <int W, int V, int LPN, bool EXACT, bool FULL>
-__device__ __forceinline__ void dds_chunk(const DdsArgs& a, int myrow, int j0, int rem, int g, int l,
-                                          const int (&eld)[V], const bool (&ev)[V],
+__device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, int myrow, float* o, int rem, int g,
+                                          int l, const int (&eld)[V], const bool (&ev)[V],
                                           const Vec<W> (&b)[V], bool accumulate) {
     constexpr int NG = 64 / LPN;
     constexpr int U = Unroll<V, LPN>::U;
     const int q = l * NG + g;            // the nonzero of this chunk whose result this lane keeps
     float res = 0.f;
     const int niter = FULL ? LPN : (rem + NG - 1) / NG;
+    constexpr bool MULTI = (LPN >= 8) && (U >= 2);       // U dot products reduced together
+    const int label = slot_label(l);
+#pragma unroll 1
     for (int it0 = 0; it0 < niter; it0 += U) {
         Vec<W> av[U][V];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int it = it0 + u;
+            // slot u of the round belongs to the nonzero kept by lane it0 + slot_offset(u)
+            const int it = it0 + (MULTI ? slot_offset<U>(u, it0) : u);
             int r;
             if constexpr (LPN == 64) r = __builtin_amdgcn_readlane(myrow, it);
             else r = lane_read(myrow, g * LPN + it);
-            const float* ap = a.A + (size_t)r * (size_t)a.k;
+            const float* ap = A + (size_t)r * (size_t)k;
 #pragma unroll
             for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
         }
+        float sums[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float s = 0.f;
@@ -60,14 +65,20 @@ __device__ __forceinline__ void dds_chunk(const DdsArgs& a, int myrow, int j0, i
                 if (!EXACT) x = ev[i] ? x : Vec<W>::zero();   // lanes past k contribute nothing
                 s = x.dotacc(b[i], s);
             }
-            s = group_allsum<LPN>(s);
-            res = (l == it0 + u) ? s : res;
+            sums[u] = s;
+        }
+        if constexpr (MULTI) {
+            const float red = group_multisum<LPN, U>(sums, label);
+            res = (l / U == it0 / U) ? red : res;
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float s = group_allsum<LPN>(sums[u]);
+                res = (l == it0 + u) ? s : res;
+            }
         }
     }
-    if (FULL || q < rem) {
-        float* o = a.P + j0 + q;
-        *o = accumulate ? (*o + res) : res;
-    }
+    if (FULL || q < rem) *o = accumulate ? (*o + res) : res;      // o: where this lane's nonzero goes
 }
 
 template <int W, int V, int LPN, bool EXACT>
@@ -120,8 +131,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
         int crow = (q < rem) ? a.ir[j0 + q] : 0;
         while (rem > 0) {
             const int nrow = (q < rem - 64) ? a.ir[j0 + 64 + q] : 0;
-            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a, crow, j0, 64, g, l, eld, ev, b, accumulate);
-            else dds_chunk<W, V, LPN, EXACT, false>(a, crow, j0, rem, g, l, eld, ev, b, accumulate);
+            float* o = a.P + j0 + q;
+            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate);
+            else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate);
             crow = nrow;
             j0 += 64;
             rem -= 64;

@@ -5,20 +5,30 @@
 #include "common.hpp"
 #include "kernels.hpp"
 #include "scan.hpp"
+#include "workspace.hpp"
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
+#include <mutex>
 #include <new>
 
 namespace bm {
 namespace {
 
-struct DevBuf {
-    void* p = nullptr;
-    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 256); }
-    ~DevBuf() { if (p) (void)hipFree(p); }
-    template <typename T> T* as() { return static_cast<T*>(p); }
+// Carves 256-byte aligned pieces out of one allocation.
+struct Arena {
+    char* base = nullptr;
+    size_t used = 0;
+    static size_t round(size_t b) { return (b + 255) & ~size_t(255); }
+    template <typename T> T* take(size_t count) {
+        T* p = base ? reinterpret_cast<T*>(base + used) : nullptr;
+        used += round(sizeof(T) * (count ? count : 1));
+        return p;
+    }
 };
 
+// Build temporaries up to this size stay in the library's workspace for the next build;
+// larger ones are given back at once.
+constexpr size_t kKeepArenaBytes = size_t(512) << 20;
 
 // Row histogram. The first HIST_LDS_ROWS rows are counted in a per-workgroup LDS copy that is
 // flushed once at the end (popular rows tend to carry small indices in count-sorted vocabularies,
@@ -145,7 +155,7 @@ inline int bits_for(unsigned long long maxval) {
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
     hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->pc, p->perm, p->segstart, p->segrow, p->rowptr, p->rowseg, p->partial};
+    void* bufs[] = {p->block_nnz, p->block_seg, p->partial};
     for (void* b : bufs)
         if (b && (f = hipFree(b)) != hipSuccess) e = f;
     delete p;
@@ -175,22 +185,51 @@ hipError_t plan_reserve_partial(bidmat_plan* p, int k) {
 hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,
                       bidmat_plan** out) {
     *out = nullptr;
+    // builds share the workspace arena of their device: one at a time
+    static std::mutex build_mu;
+    std::lock_guard<std::mutex> build_lock(build_mu);
     bidmat_plan* plan = new (std::nothrow) bidmat_plan();
     if (!plan) return hipErrorOutOfMemory;
     hipStream_t s = nullptr;
     PB_CHECK(hipGetDevice(&plan->device));
     plan->nrows = nrows; plan->ncols = ncols; plan->nnz = nnz;
     plan->seglen = opt_seglen();
+    {
+        // small patterns: shorter segments, so that the gather stage still has a few waves for
+        // every wave slot of the device
+        long long want = ((long long)nnz / 32768 / 64) * 64;
+        if (want < 64) want = 64;
+        if (want < plan->seglen) plan->seglen = (int)want;
+    }
     if (k_hint <= 0) k_hint = 256;
     long long pcols = (long long)opt_panel_kb() * 1024 / (4LL * k_hint);
     if (pcols < 64) pcols = 64;
     if (pcols > ncols) pcols = ncols > 0 ? ncols : 1;
+    if (ncols >= 8 * 64) {
+        // panels are dealt to the 8 XCDs round-robin: a multiple of 8 keeps them all equally busy
+        long long np = (ncols + pcols - 1) / pcols;
+        np = ((np + 7) / 8) * 8;
+        pcols = (ncols + np - 1) / np;
+    }
     plan->panel_cols = (int)pcols;
     plan->npanels = ncols > 0 ? (int)(((long long)ncols + pcols - 1) / pcols) : 1;
     const int p8 = (plan->npanels + 7) / 8;          // panels per XCD group
 
-    PB_CHECK(hipMalloc((void**)&plan->rowptr, sizeof(int) * ((size_t)nrows + 1)));
-    plan->index_bytes += sizeof(int) * ((size_t)nrows + 1);
+    // memory the plan keeps, part 1: everything whose size is known now
+    {
+        Arena own;
+        for (int pass = 0; pass < 2; ++pass) {
+            own.used = 0;
+            plan->rowptr = own.take<int>((size_t)nrows + 1);
+            plan->perm = own.take<int>((size_t)nnz);
+            plan->pc = own.take<int>((size_t)nnz);
+            if (pass == 0) {
+                PB_CHECK(hipMalloc(&plan->block_nnz, own.used));
+                own.base = static_cast<char*>(plan->block_nnz);
+                plan->index_bytes += own.used;
+            }
+        }
+    }
     if (nnz == 0 || nrows == 0 || ncols == 0) {
         PB_CHECK(fill_i32(plan->rowptr, (long long)nrows + 1, 0, s));
         PB_CHECK(hipStreamSynchronize(s));
@@ -198,115 +237,144 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         return hipSuccess;
     }
 
-    DevBuf cnt, hflag, hrank, hrow, scantmp, bad, keys_in, keys_out, pos_in, ic, flag, segidx;
-    PB_CHECK(cnt.alloc(sizeof(int) * (size_t)nrows));
-    PB_CHECK(hflag.alloc(sizeof(int) * (size_t)nrows));
-    PB_CHECK(hrank.alloc(sizeof(int) * ((size_t)nrows + 1)));
-    PB_CHECK(hrow.alloc(sizeof(int) * (size_t)nrows));
-    size_t scan_n = (size_t)(nnz > nrows ? nnz : nrows);
-    PB_CHECK(scantmp.alloc(sizeof(int) * scan_tmp_ints((long long)scan_n)));
-    PB_CHECK(bad.alloc(sizeof(int)));
+    // temporaries: one arena out of the library's workspace
+    const size_t scan_n = (size_t)(nnz > nrows ? nnz : nrows);
+    const unsigned long long maxkey_bound = 8ULL * (unsigned long long)p8 * (unsigned long long)nrows + (unsigned long long)nrows;
+    const int rbits = bits_for((unsigned long long)nrows);
+    size_t sort_bytes = 0;
+    {
+        // both sorts share one scratch area, sized for the larger request (the second sort has
+        // at most nnz items)
+        size_t b1 = 0, b2 = 0;
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b1, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
+                                           (int*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b2, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
+                                           (int*)nullptr, (size_t)nnz, 0, rbits, s));
+        sort_bytes = b1 > b2 ? b1 : b2;
+    }
+    Arena tmp;
+    int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *scantmp = nullptr, *class_count = nullptr;
+    int *pos_in = nullptr, *ic = nullptr, *flag = nullptr, *segidx = nullptr;
+    unsigned *keys_in = nullptr, *keys_out = nullptr;
+    unsigned char* segclass = nullptr;
+    char* sorttmp = nullptr;
+    for (int pass = 0; pass < 2; ++pass) {
+        tmp.used = 0;
+        cnt = tmp.take<int>((size_t)nrows);
+        hflag = tmp.take<int>((size_t)nrows);
+        hrank = tmp.take<int>((size_t)nrows + 2);        // [nrows] = number of heavy rows, [nrows+1] = bad-index flag
+        hrow = tmp.take<int>((size_t)nrows);
+        scantmp = tmp.take<int>(scan_tmp_ints((long long)scan_n));
+        class_count = tmp.take<int>(9);
+        keys_in = tmp.take<unsigned>((size_t)nnz);       // later: ids of the segments
+        keys_out = tmp.take<unsigned>((size_t)nnz);
+        pos_in = tmp.take<int>((size_t)nnz);             // later: segment rows in sorted order
+        ic = tmp.take<int>((size_t)nnz);
+        flag = tmp.take<int>((size_t)nnz);
+        segidx = tmp.take<int>((size_t)nnz + 1);
+        segclass = tmp.take<unsigned char>((size_t)nnz);
+        sorttmp = tmp.take<char>(sort_bytes);
+        if (pass == 0) {
+            hipError_t werr;
+            tmp.base = static_cast<char*>(ws_get(WS_PLAN, tmp.used, &werr));
+            if (!tmp.base) { (void)plan_free(plan); return werr; }
+        }
+    }
+    const size_t arena_bytes = tmp.used;
+    int* const bad = hrank + nrows + 1;
 
     // 1. row histogram (integer atomics: the counts do not depend on the order)
-    PB_CHECK(fill_i32(cnt.as<int>(), nrows, 0, s));
-    PB_CHECK(fill_i32(bad.as<int>(), 1, 0, s));
+    PB_CHECK(fill_i32(cnt, nrows, 0, s));
+    PB_CHECK(fill_i32(hrank + nrows, 2, 0, s));
     // few, long-lived workgroups: every one flushes its LDS histogram once at the end
-    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, ir, cnt.as<int>(), bad.as<int>());
-    int h_bad = 0;
-    PB_CHECK(hipMemcpy(&h_bad, bad.p, sizeof(int), hipMemcpyDeviceToHost));
-    if (h_bad) { (void)plan_free(plan); return hipErrorInvalidValue; }
+    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, ir, cnt, bad);
 
     // 2. heavy rows and their ranks
     int nheavy = 0;
+    int h2[2] = {0, 0};                                  // {number of heavy rows, bad-index flag}
     if (plan->npanels >= 2) {
         long long thresh = (long long)plan->npanels * opt_heavy_min();
         if (thresh > 0x7fffffffLL) thresh = 0x7fffffffLL;
-        hipLaunchKernelGGL(k_heavy_flag, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, cnt.as<int>(), (int)thresh, hflag.as<int>());
-        PB_CHECK(scan_exclusive_i32(hflag.as<int>(), hrank.as<int>(), nrows, scantmp.as<int>(), s));
-        PB_CHECK(hipMemcpy(&nheavy, hrank.as<int>() + nrows, sizeof(int), hipMemcpyDeviceToHost));
+        hipLaunchKernelGGL(k_heavy_flag, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, cnt, (int)thresh, hflag);
+        // the scan writes hrank[0..nrows]; the bad-index flag sits behind it
+        PB_CHECK(scan_exclusive_i32(hflag, hrank, nrows, scantmp, s));
+    }
+    PB_CHECK(hipMemcpy(h2, hrank + nrows, sizeof(h2), hipMemcpyDeviceToHost));
+    if (h2[1]) { (void)plan_free(plan); return hipErrorInvalidValue; }
+    if (plan->npanels >= 2) {
+        nheavy = h2[0];
         // keys must fit 32 bits
         if (8ULL * (unsigned long long)p8 * (unsigned long long)nheavy + (unsigned long long)nrows > 0xffffffffULL) nheavy = 0;
     }
     if (nheavy == 0) {
-        PB_CHECK(fill_i32(hflag.as<int>(), nrows, 0, s));
-        PB_CHECK(fill_i32(hrank.as<int>(), (long long)nrows + 1, 0, s));
+        PB_CHECK(fill_i32(hflag, nrows, 0, s));
+        PB_CHECK(fill_i32(hrank, (long long)nrows + 1, 0, s));
     } else {
-        hipLaunchKernelGGL(k_heavy_rows, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, hflag.as<int>(), hrank.as<int>(), hrow.as<int>());
+        hipLaunchKernelGGL(k_heavy_rows, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, hflag, hrank, hrow);
     }
     plan->nheavy = nheavy;
 
     // 3. keys + stable radix sort
-    PB_CHECK(keys_in.alloc(sizeof(unsigned) * (size_t)nnz));
-    PB_CHECK(keys_out.alloc(sizeof(unsigned) * (size_t)nnz));
-    PB_CHECK(pos_in.alloc(sizeof(int) * (size_t)nnz));
-    PB_CHECK(hipMalloc((void**)&plan->perm, sizeof(int) * (size_t)nnz));
-    PB_CHECK(hipMalloc((void**)&plan->pc, sizeof(int) * (size_t)nnz));
-    plan->index_bytes += 2 * sizeof(int) * (size_t)nnz;
     {
         long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
         hipLaunchKernelGGL(k_make_keys, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nrows, jc, ir,
-                           hflag.as<int>(), hrank.as<int>(), nheavy, plan->npanels, plan->panel_cols, p8,
-                           keys_in.as<unsigned>(), pos_in.as<int>());
+                           hflag, hrank, nheavy, plan->npanels, plan->panel_cols, p8, keys_in, pos_in);
     }
     const unsigned long long maxkey = 8ULL * (unsigned long long)p8 * nheavy + (unsigned long long)nrows;
     const int end_bit = bits_for(maxkey);
     {
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in.as<unsigned>(), keys_out.as<unsigned>(),
-                                           pos_in.as<int>(), plan->perm, (size_t)nnz, 0, end_bit, s));
-        DevBuf sorttmp;
-        PB_CHECK(sorttmp.alloc(tmp_bytes));
-        PB_CHECK(rocprim::radix_sort_pairs(sorttmp.p, tmp_bytes, keys_in.as<unsigned>(), keys_out.as<unsigned>(),
-                                           pos_in.as<int>(), plan->perm, (size_t)nnz, 0, end_bit, s));
-        PB_CHECK(hipStreamSynchronize(s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in, keys_out, pos_in, plan->perm, (size_t)nnz, 0, end_bit, s));
+        if (tmp_bytes > sort_bytes) { (void)plan_free(plan); return hipErrorOutOfMemory; }
+        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, keys_in, keys_out, pos_in, plan->perm, (size_t)nnz, 0, end_bit, s));
     }
 
     // 4. segment boundaries
-    PB_CHECK(ic.alloc(sizeof(int) * (size_t)nnz));
-    PB_CHECK(csc_expand_cols(ncols, nnz, jc, ic.as<int>(), s));
-    PB_CHECK(flag.alloc(sizeof(int) * (size_t)nnz));
-    PB_CHECK(segidx.alloc(sizeof(int) * ((size_t)nnz + 1)));
-    hipLaunchKernelGGL(k_boundaries, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, plan->seglen, keys_out.as<unsigned>(), flag.as<int>());
-    PB_CHECK(scan_exclusive_i32(flag.as<int>(), segidx.as<int>(), nnz, scantmp.as<int>(), s));
+    PB_CHECK(csc_expand_cols(ncols, nnz, jc, ic, s));
+    hipLaunchKernelGGL(k_boundaries, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, plan->seglen, keys_out, flag);
+    PB_CHECK(scan_exclusive_i32(flag, segidx, nnz, scantmp, s));
     int nseg = 0;
-    PB_CHECK(hipMemcpy(&nseg, segidx.as<int>() + nnz, sizeof(int), hipMemcpyDeviceToHost));
+    PB_CHECK(hipMemcpy(&nseg, segidx + nnz, sizeof(int), hipMemcpyDeviceToHost));
     plan->nseg = nseg;
 
-    DevBuf segid, segrow_sorted, class_count;
-    DevBuf segclass;
-    PB_CHECK(class_count.alloc(sizeof(int) * 9));
-    PB_CHECK(fill_i32(class_count.as<int>(), 9, nseg, s));
-    PB_CHECK(segclass.alloc((size_t)(nseg > 0 ? nseg : 1)));
-    PB_CHECK(hipMalloc((void**)&plan->segrow, sizeof(int) * (size_t)(nseg > 0 ? nseg : 1)));
+    // memory the plan keeps, part 2: the segment tables
+    {
+        Arena own;
+        for (int pass = 0; pass < 2; ++pass) {
+            own.used = 0;
+            plan->segstart = own.take<int>((size_t)nseg + 1);
+            plan->segrow = own.take<int>((size_t)nseg);
+            plan->rowseg = own.take<int>((size_t)nseg);
+            if (pass == 0) {
+                PB_CHECK(hipMalloc(&plan->block_seg, own.used));
+                own.base = static_cast<char*>(plan->block_seg);
+                plan->index_bytes += own.used;
+            }
+        }
+    }
+    // the sort's inputs are dead by now: their space holds the segment ids and the sorted rows
+    int* const segid = reinterpret_cast<int*>(keys_in);
+    unsigned* const segrow_sorted = reinterpret_cast<unsigned*>(pos_in);
     unsigned* const segrow_u = reinterpret_cast<unsigned*>(plan->segrow);
-    PB_CHECK(segid.alloc(sizeof(int) * (size_t)nseg));
-    PB_CHECK(segrow_sorted.alloc(sizeof(unsigned) * (size_t)nseg));
-    PB_CHECK(hipMalloc((void**)&plan->segstart, sizeof(int) * ((size_t)nseg + 1)));
-    PB_CHECK(hipMalloc((void**)&plan->rowseg, sizeof(int) * (size_t)nseg));
-    plan->index_bytes += sizeof(int) * (3 * (size_t)nseg + 1);
-    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out.as<unsigned>(), plan->perm,
-                       ic.as<int>(), flag.as<int>(), segidx.as<int>(), hrow.as<int>(), nheavy > 0 ? nheavy : 1,
-                       nheavy > 0 ? p8 : 0, plan->pc, plan->segstart, segrow_u, segid.as<int>(),
-                       segclass.as<unsigned char>());
+    PB_CHECK(fill_i32(class_count, 9, nseg, s));
+    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out, plan->perm,
+                       ic, flag, segidx, hrow, nheavy > 0 ? nheavy : 1,
+                       nheavy > 0 ? p8 : 0, plan->pc, plan->segstart, segrow_u, segid, segclass);
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
-    hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg,
-                       segclass.as<unsigned char>(), class_count.as<int>());
-    PB_CHECK(hipMemcpy(plan->xcd_start, class_count.p, sizeof(int) * 9, hipMemcpyDeviceToHost));
+    hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg, segclass, class_count);
+    PB_CHECK(hipMemcpy(plan->xcd_start, class_count, sizeof(int) * 9, hipMemcpyDeviceToHost));
 
     // 5. a row's segments, in ascending segment order (stable sort by row)
     {
-        const int rbits = bits_for((unsigned long long)nrows);
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, segrow_u, segrow_sorted.as<unsigned>(),
-                                           segid.as<int>(), plan->rowseg, (size_t)nseg, 0, rbits, s));
-        DevBuf sorttmp;
-        PB_CHECK(sorttmp.alloc(tmp_bytes));
-        PB_CHECK(rocprim::radix_sort_pairs(sorttmp.p, tmp_bytes, segrow_u, segrow_sorted.as<unsigned>(),
-                                           segid.as<int>(), plan->rowseg, (size_t)nseg, 0, rbits, s));
-        PB_CHECK(coo_compress_cols(nrows, nseg, reinterpret_cast<const int*>(segrow_sorted.as<unsigned>()), plan->rowptr, s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
+        if (tmp_bytes > sort_bytes) { (void)plan_free(plan); return hipErrorOutOfMemory; }
+        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
+        PB_CHECK(coo_compress_cols(nrows, nseg, reinterpret_cast<const int*>(segrow_sorted), plan->rowptr, s));
         PB_CHECK(hipStreamSynchronize(s));
     }
     PB_CHECK(hipGetLastError());
+    if (arena_bytes > kKeepArenaBytes) PB_CHECK(ws_drop(WS_PLAN));
     *out = plan;
     return hipSuccess;
 }

@@ -29,6 +29,8 @@ struct bidmat_plan {
     int* segrow = nullptr;   // [nseg]   row of each segment
     int* rowptr = nullptr;   // [nrows+1] range of a row's segments in rowseg
     int* rowseg = nullptr;   // [nseg]   segment ids grouped by row, ascending within a row
+    void* block_nnz = nullptr;   // owns pc, perm, rowptr
+    void* block_seg = nullptr;   // owns segstart, segrow, rowseg
     float* partial = nullptr;
     size_t partial_floats = 0;
     size_t index_bytes = 0;

@@ -48,6 +48,20 @@ void* ws_get(WsSlot slot, size_t bytes, hipError_t* err) {
     return s.ptr;
 }
 
+hipError_t ws_drop(WsSlot slot) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_mu);
+    Slot& s = g_slots[dev][slot];
+    if (s.ptr) {
+        e = hipFree(s.ptr);
+        s.ptr = nullptr; s.bytes = 0;
+    }
+    return e;
+}
+
 hipError_t ws_release() {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);

@@ -16,12 +16,15 @@ enum WsSlot {
     WS_REDUCE,        // float[...]    partials of the dense reductions
     WS_TRANS_IN,      // float[...]    transposed dense operand of S*A / S^T*A
     WS_TRANS_OUT,     // float[...]    transposed result of S*A / S^T*A
+    WS_PLAN,          // bytes         temporaries of a plan build (dropped again when large)
     WS_NSLOTS
 };
 
 // Returns a device buffer of at least `bytes` for `slot` on the current device (nullptr and
 // *err set on failure). Growing a slot frees the old buffer after a device synchronise.
 void* ws_get(WsSlot slot, size_t bytes, hipError_t* err);
+// Frees one slot of the current device.
+hipError_t ws_drop(WsSlot slot);
 // Frees every slot of the current device.
 hipError_t ws_release();
 // Total bytes currently held on the current device.
