@@ -48,11 +48,28 @@ __global__ __launch_bounds__(BM_BLOCK) void k_apply(const float* __restrict__ A,
 template <int OP>
 __global__ __launch_bounds__(BM_BLOCK) void k_apply_full4(const float4* __restrict__ A, const float4* __restrict__ B,
                                                           float4* __restrict__ C, long long n4) {
-    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    const long long stride = (long long)gridDim.x * BM_BLOCK;
-    for (; i < n4; i += stride) {
-        const float4 a = A[i], b = B[i];
-        C[i] = make_float4(binop<OP>(a.x, b.x), binop<OP>(a.y, b.y), binop<OP>(a.z, b.z), binop<OP>(a.w, b.w));
+    // a workgroup walks tiles of 4 x 256 vectors: four independent 128-bit loads per operand in
+    // flight per thread, neighbouring in memory
+    constexpr int UN = 4;
+    long long i = (long long)blockIdx.x * (UN * BM_BLOCK) + threadIdx.x;
+    const long long stride = (long long)gridDim.x * (UN * BM_BLOCK);
+    for (; i + (UN - 1) * BM_BLOCK < n4; i += stride) {
+        float4 a[UN], b[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) { a[u] = A[i + u * BM_BLOCK]; b[u] = B[i + u * BM_BLOCK]; }
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            C[i + u * BM_BLOCK] = make_float4(binop<OP>(a[u].x, b[u].x), binop<OP>(a[u].y, b[u].y),
+                                              binop<OP>(a[u].z, b[u].z), binop<OP>(a[u].w, b[u].w));
+    }
+    // the last, partial tile
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const long long j = i + u * BM_BLOCK;
+        if (j < n4) {
+            const float4 a = A[j], b = B[j];
+            C[j] = make_float4(binop<OP>(a.x, b.x), binop<OP>(a.y, b.y), binop<OP>(a.z, b.z), binop<OP>(a.w, b.w));
+        }
     }
 }
 
@@ -104,7 +121,7 @@ hipError_t apply_impl(const float* A, int ma, const float* B, int mb, float* C, 
         long long n4 = 0;
         if (aligned16(A) && aligned16(B) && aligned16(C)) {
             n4 = n / 4;
-            if (n4 > 0) hipLaunchKernelGGL(k_apply_full4<OP>, dim3(grid_for(n4)), dim3(BM_BLOCK), 0, s,
+            if (n4 > 0) hipLaunchKernelGGL(k_apply_full4<OP>, dim3(grid_for((n4 + 3) / 4)), dim3(BM_BLOCK), 0, s,
                                            (const float4*)A, (const float4*)B, (float4*)C, n4);
         }
         long long done = n4 * 4;

@@ -453,6 +453,21 @@ def test_applyop_flat_div_on_values(hip):
     d.free()
 
 
+@pytest.mark.parametrize("n", [1, 3, 5, 4 * 1023, 4 * 1024, 4 * 1024 + 4, 4 * 1025 + 1, 4 * 2048, 4 * 2048 + 7,
+                               4 * 1024 * 16384 + 4 * 100 + 2])
+def test_applyop_flat_tile_edges(hip, n):
+    """Sizes around the 4 x 256-vector tiles of the streaming kernel, and one larger than the grid."""
+    rng = np.random.default_rng(n % 1000)
+    A = rng.random(n).astype(np.float32)
+    B = rng.random(n).astype(np.float32) + 0.5
+    d = Dev(A=A, B=B)
+    d.zeros("Cm", n)
+    hip_abi.check(hip.bidmat_applyop_flat(d.A.ptr, d.B.ptr, d.Cm.ptr, n, 1, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert np.array_equal(d.Cm.numpy(), A - B)
+    d.free()
+
+
 # ------------------------------------------------------------------------------ CSC utilities
 def test_expand_and_compress_cols(hip):
     rng = np.random.default_rng(95)
