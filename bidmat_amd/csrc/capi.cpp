@@ -64,10 +64,8 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     hipStream_t s = nullptr;
     unsigned long long* d_misc = (unsigned long long*)bm::ws_get(bm::WS_MISC, 64, &err);
     if (!d_misc) return err;
-    // misc layout: [0..1] fingerprints, [2] (as int) max row
-    if ((err = bm::fingerprint(ir, nnz, ic, nnz, d_misc, s)) != hipSuccess) return err;
-    int* d_max = reinterpret_cast<int*>(d_misc + 2);
-    if ((err = bm::int_max(ir, nnz, d_max, s)) != hipSuccess) return err;
+    // misc layout: [0..1] digests of ir and ic, [2] (as int) max row
+    if ((err = bm::pattern_digest(ir, ic, nnz, d_misc, s)) != hipSuccess) return err;
     unsigned long long h[3];
     if ((err = hipMemcpy(h, d_misc, sizeof(h), hipMemcpyDeviceToHost)) != hipSuccess) return err;
     int maxrow;

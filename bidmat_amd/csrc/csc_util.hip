@@ -38,35 +38,61 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fill(T* __restrict__ out, long lon
     for (; i < n; i += stride) out[i] = v;
 }
 
-__global__ __launch_bounds__(BM_BLOCK) void k_int_max(const int* __restrict__ in, long long n, int* out) {
-    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    const long long stride = (long long)gridDim.x * BM_BLOCK;
+// Weight of position i in the digest: odd, and different positions get unrelated weights.
+__device__ __forceinline__ unsigned pos_weight(unsigned i) {
+    unsigned x = (i + 1u) * 0x9E3779B1u;
+    x ^= x >> 15; x *= 0x85EBCA77u;
+    x ^= x >> 13;
+    return x | 1u;
+}
+
+// One pass over both index arrays of a pattern: digests sum_i weight(i) * (value_i + c) of ir and
+// of ic (64-bit integer sums: position-sensitive, independent of the order in which threads
+// contribute) and the largest row index. A workgroup walks tiles of 4 x 256 positions with four
+// loads per array in flight per thread. out: [0] digest of ir, [1] digest of ic, [2] (int) max.
+__global__ __launch_bounds__(BM_BLOCK) void k_pattern_digest(const int* __restrict__ ir, const int* __restrict__ ic,
+                                                             long long n, unsigned long long* out) {
+    constexpr int UN = 4;
+    long long i = (long long)blockIdx.x * (UN * BM_BLOCK) + threadIdx.x;
+    const long long stride = (long long)gridDim.x * (UN * BM_BLOCK);
+    unsigned long long ha = 0, hb = 0;
     int m = -1;
-    for (; i < n; i += stride) m = max(m, in[i]);
+    for (; i < n; i += stride) {
+        int r[UN], c[UN];
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) m = max(m, __shfl_xor(m, d, 64));
-    if ((threadIdx.x & 63) == 0 && m >= 0) atomicMax(out, m);
+        for (int u = 0; u < UN; ++u) {
+            const long long j = i + u * BM_BLOCK;
+            r[u] = j < n ? ir[j] : -1;
+            c[u] = j < n ? ic[j] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const long long j = i + u * BM_BLOCK;
+            if (j < n) {
+                const unsigned long long w = pos_weight((unsigned)j);
+                ha += w * (unsigned long long)((unsigned)r[u] + 0x7F4A7C15u);
+                hb += w * (unsigned long long)((unsigned)c[u] + 0x2545F491u);
+                m = max(m, r[u]);
+            }
+        }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        ha += __shfl_xor(ha, d, 64);
+        hb += __shfl_xor(hb, d, 64);
+        m = max(m, __shfl_xor(m, d, 64));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        atomicAdd(out, ha);
+        atomicAdd(out + 1, hb);
+        if (m >= 0) atomicMax(reinterpret_cast<int*>(out + 2), m);
+    }
 }
 
-__device__ __forceinline__ unsigned long long mix64(unsigned long long x) {
-    x ^= x >> 33; x *= 0xff51afd7ed558ccdULL;
-    x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ULL;
-    x ^= x >> 33;
-    return x;
-}
-
-// Sum over positions of mix(position, value): position-sensitive, and the integer sum does
-// not depend on the order in which threads contribute.
-__global__ __launch_bounds__(BM_BLOCK) void k_fingerprint(const int* __restrict__ in, long long n,
-                                                          unsigned long long* out) {
-    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    const long long stride = (long long)gridDim.x * BM_BLOCK;
-    unsigned long long h = 0;
-    for (; i < n; i += stride)
-        h += mix64(((unsigned long long)i << 32) ^ (unsigned long long)(unsigned)in[i] ^ 0x9e3779b97f4a7c15ULL);
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) h += __shfl_xor(h, d, 64);
-    if ((threadIdx.x & 63) == 0) atomicAdd(out, h);
+// out[0..1] = 0, (int)out[2] = -1
+__global__ void k_digest_init(unsigned long long* out) {
+    if (threadIdx.x < 2) out[threadIdx.x] = 0;
+    if (threadIdx.x == 2) { out[2] = 0; *reinterpret_cast<int*>(out + 2) = -1; }
 }
 
 inline unsigned grid_for(long long n, int maxblocks = 8192) {
@@ -106,19 +132,10 @@ hipError_t fill_i32(int* out, long long n, int v, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t int_max(const int* d_in, long long n, int* d_out, hipStream_t s) {
-    hipError_t e = fill_i32(d_out, 1, -1, s);
-    if (e != hipSuccess || n <= 0) return e;
-    hipLaunchKernelGGL(k_int_max, dim3(grid_for(n, 2048)), dim3(BM_BLOCK), 0, s, d_in, n, d_out);
-    return hipGetLastError();
-}
-
-hipError_t fingerprint(const int* a, long long na, const int* b, long long nb,
-                       unsigned long long* d_out, hipStream_t s) {
-    hipError_t e = fill_i32(reinterpret_cast<int*>(d_out), 4, 0, s);
-    if (e != hipSuccess) return e;
-    if (na > 0) hipLaunchKernelGGL(k_fingerprint, dim3(grid_for(na, 2048)), dim3(BM_BLOCK), 0, s, a, na, d_out);
-    if (nb > 0) hipLaunchKernelGGL(k_fingerprint, dim3(grid_for(nb, 2048)), dim3(BM_BLOCK), 0, s, b, nb, d_out + 1);
+hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s) {
+    hipLaunchKernelGGL(k_digest_init, dim3(1), dim3(64), 0, s, d_out);
+    if (nnz > 0)
+        hipLaunchKernelGGL(k_pattern_digest, dim3(grid_for((nnz + 3) / 4, 2048)), dim3(BM_BLOCK), 0, s, ir, ic, nnz, d_out);
     return hipGetLastError();
 }
 

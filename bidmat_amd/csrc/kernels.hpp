@@ -16,11 +16,9 @@ hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStre
 // out[i] = v for i < n (a kernel, so that callers may record it into a HIP graph)
 hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
 hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);
-// max over an int array (result written to *d_out, a device int; empty -> -1)
-hipError_t int_max(const int* d_in, long long n, int* d_out, hipStream_t s);
-// order-sensitive 64-bit fingerprint of two int arrays (device result, 2 x uint64)
-hipError_t fingerprint(const int* a, long long na, const int* b, long long nb,
-                       unsigned long long* d_out, hipStream_t s);
+// One pass over the two index arrays of a pattern (device result, 3 x uint64): [0], [1] order- and
+// position-sensitive 64-bit digests of ir and ic, [2] (as int) the largest entry of ir (-1: empty).
+hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s);
 
 // ---- overflow-segment table shared by dsmult and dds (spmm.hip)
 // Returns in *d_ovf a device table int[ncols+1] (exclusive scan of the number of extra
