@@ -76,6 +76,34 @@ JFN(jint, dsmultTPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong Sdata
     int e = bidmat_dsmultT_plan(P(bidmat_plan, plan), k, P(const float, A), P(const float, Sdata), P(float, C), beta, nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
+// sparse sums without the per-nonzero column array (GSMat.sum, GSMat.scala:250-261)
+JFN(jint, spsumCols)(JNIEnv*, jclass, jint nc, jint nnz, jlong Sdata, jlong Sjc, jlong out, jint beta) {
+    int e = bidmat_spsum_cols(nc, nnz, P(const float, Sdata), P(const int, Sjc), P(float, out), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jint, spsumRowsPlan)(JNIEnv*, jclass, jlong plan, jlong Sdata, jlong out, jint beta) {
+    int e = bidmat_spsum_rows_plan(P(bidmat_plan, plan), P(const float, Sdata), P(float, out), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+// S^T * A and S * A (replace the cusparseScsrmm calls of GSMat.SDTMult / SDMult, GSMat.scala:265-313)
+JFN(jint, sdtmultCsc)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jint p, jlong Sdata, jlong Sir, jlong Sjc, jlong A,
+                      jint lda, jlong C, jint ldc) {
+    int e = bidmat_sdtmult_csc(nr, nc, nnz, p, P(const float, Sdata), P(const int, Sir), P(const int, Sjc),
+                               P(const float, A), lda, P(float, C), ldc, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jint, sdmultPlan)(JNIEnv*, jclass, jlong plan, jint p, jlong Sdata, jlong A, jint lda, jlong C, jint ldc) {
+    int e = bidmat_sdmult_plan(P(bidmat_plan, plan), p, P(const float, Sdata), P(const float, A), lda, P(float, C), ldc, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jint, setOption)(JNIEnv* env, jclass, jstring name, jlong value) {
+    const char* n = env->GetStringUTFChars(name, nullptr);
+    if (!n) return 1;
+    int e = bidmat_set_option(n, value);
+    env->ReleaseStringUTFChars(name, n);
+    return e;
+}
+JFN(jint, releaseCaches)(JNIEnv*, jclass) { return bidmat_release_caches(); }
 JFN(jint, cscExpandCols)(JNIEnv*, jclass, jint nc, jint nnz, jlong Sjc, jlong Sic) {
     int e = bidmat_csc_expand_cols(nc, nnz, P(const int, Sjc), P(int, Sic), nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
