@@ -21,7 +21,20 @@ __global__ __launch_bounds__(BM_BLOCK) void k_spsum_ranges(int nranges, const fl
     float acc = 0.f;
     if (c < nranges) {
         const int s = ptr[c], e = ptr[c + 1];
-        for (int j = s + l; j < e; j += 16) acc += PERM ? vals[perm[j]] : vals[j];
+        // four loads in flight per lane; the four running sums are combined in a fixed order
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        int j = s + l;
+        for (; j + 48 < e; j += 64) {
+            if (PERM) {
+                const int p0 = perm[j], p1 = perm[j + 16], p2 = perm[j + 32], p3 = perm[j + 48];
+                a0 += vals[p0]; a1 += vals[p1]; a2 += vals[p2]; a3 += vals[p3];
+            } else {
+                const float v0 = vals[j], v1 = vals[j + 16], v2 = vals[j + 32], v3 = vals[j + 48];
+                a0 += v0; a1 += v1; a2 += v2; a3 += v3;
+            }
+        }
+        for (; j < e; j += 16) a0 += PERM ? vals[perm[j]] : vals[j];
+        acc = (a0 + a1) + (a2 + a3);
     }
     acc = group_allsum<16>(acc);
     if (c < nranges && l == 0) out[c] = beta ? out[c] + acc : acc;
