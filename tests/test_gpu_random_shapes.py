@@ -70,3 +70,56 @@ def test_random_case(hip, seed):
     finally:
         for n, v in olds:
             hip_abi.check(hip.bidmat_set_option(n.encode(), v))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_medium_case(hip, seed):
+    """Thousands of columns and rows: several workgroups in the overflow table, plans with many
+    panels (a multiple of 8 of them) and segment lengths adapted to the pattern size."""
+    rng = np.random.default_rng(9500 + seed)
+    k = int(rng.choice([32, 100, 128, 256, 512]))
+    nrows = int(rng.integers(500, 6000))
+    ncols = int(rng.integers(2000, 30000))
+    lengths = rng.poisson(rng.uniform(2, 25), size=ncols).astype(np.int64)
+    for c in rng.integers(0, ncols, size=5):              # a few long columns
+        lengths[c] = int(rng.integers(1500, 6000))
+    jc = np.zeros(ncols + 1, dtype=np.int32)
+    jc[1:] = np.cumsum(lengths)
+    nnz = int(jc[-1])
+    # Zipf-like rows (repeats inside a column allowed), unsorted for odd seeds
+    w = 1.0 / np.arange(1, nrows + 1) ** rng.uniform(0.8, 1.3)
+    ir = rng.choice(nrows, size=nnz, p=w / w.sum()).astype(np.int32)
+    if seed % 2 == 0:
+        ic = np.repeat(np.arange(ncols), lengths)
+        ir = ir[np.lexsort((ir, ic))]
+    data = (1.0 - rng.random(nnz)).astype(np.float32)
+    seglen = int(rng.choice([64, 256, 1024]))
+    panel_kb = int(rng.choice([16, 256, 3072]))
+    heavy_min = int(rng.choice([1, 8]))
+    olds = [(n, hip.bidmat_get_option(n.encode())) for n in ("seglen", "panel_kb", "heavy_min")]
+    for n, v in (("seglen", seglen), ("panel_kb", panel_kb), ("heavy_min", heavy_min)):
+        hip_abi.check(hip.bidmat_set_option(n.encode(), v))
+    try:
+        A = rng.standard_normal(k * nrows).astype(np.float32)
+        B = rng.standard_normal(k * ncols).astype(np.float32)
+        d = Dev(A=A, B=B, data=data, ir=ir, jc=jc)
+        d.zeros("AS", k * ncols), d.zeros("P", nnz), d.zeros("BSt", k * nrows)
+        d.zeros("cs", ncols), d.zeros("rs", nrows)
+        plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+        hip_abi.check(hip.bidmat_dsmult_csc(k, ncols, nnz, d.A.ptr, d.data.ptr, d.ir.ptr, d.jc.ptr, d.AS.ptr, 0, None))
+        hip_abi.check(hip.bidmat_dds_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.P.ptr, 0, None))
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.B.ptr, d.data.ptr, d.BSt.ptr, 0, None))
+        hip_abi.check(hip.bidmat_spsum_cols(ncols, nnz, d.data.ptr, d.jc.ptr, d.cs.ptr, 0, None))
+        hip_abi.check(hip.bidmat_spsum_rows_plan(plan, d.data.ptr, d.rs.ptr, 0, None))
+        hip_abi.check(hip.bidmat_synchronize())
+        tag = "seed=%d k=%d %dx%d nnz=%d seglen=%d panel=%d heavy=%d" % (seed, k, nrows, ncols, nnz, seglen, panel_kb, heavy_min)
+        close(d.AS.numpy(), *oracle.fsmult_f64(A, k, data, ir, jc), "A*S " + tag)
+        close(d.P.numpy(nnz), *oracle.dds_f64(A, B, k, ir, jc), "DDS " + tag)
+        close(d.BSt.numpy(), *oracle.fsmultT_f64(B, k, nrows, data, ir, jc), "A*^S " + tag)
+        close(d.cs.numpy(), *oracle.spsum_f64(nrows, data, ir, jc, 1), "colsum " + tag)
+        close(d.rs.numpy(), *oracle.spsum_f64(nrows, data, ir, jc, 2), "rowsum " + tag)
+        hip_abi.check(hip.bidmat_plan_destroy(plan))
+        d.free()
+    finally:
+        for n, v in olds:
+            hip_abi.check(hip.bidmat_set_option(n.encode(), v))
