@@ -106,7 +106,7 @@ hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* va
 hipError_t run_spsum_rows(bidmat_plan* plan, const float* vals, float* out, int beta, hipStream_t s) {
     hipError_t err;
     if ((err = bm::plan_reserve_partial(plan, 1)) != hipSuccess) return err;
-    if ((err = bm::spsum_segments(plan->nseg, vals, plan->perm, plan->segstart, plan->partial, s)) != hipSuccess)
+    if ((err = bm::spsum_segments(plan->nseg, plan->xcd_start, vals, plan->perm, plan->segstart, plan->partial, s)) != hipSuccess)
         return err;
     return bm::reduce_segments(1, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, out, beta, s);
 }

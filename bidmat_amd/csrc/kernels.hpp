@@ -61,7 +61,7 @@ hipError_t reduce_segments_ex(int k, int ldc, int row0, int nrows, const int* ro
 // ---- sums (sums.hip)
 hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, float* out, int beta,
                       hipStream_t s);
-hipError_t spsum_segments(int nseg, const float* vals, const int* perm, const int* segstart,
+hipError_t spsum_segments(int nseg, const int* xcd_start, const float* vals, const int* perm, const int* segstart,
                           float* partial, hipStream_t s);
 hipError_t reduce1op(int nrows, int ncols, const float* A, float* B, float initv, int opn,
                      hipStream_t s);

@@ -9,10 +9,9 @@ namespace bm {
 namespace {
 
 // ------------------------------------------------------------------ sparse
-// 16 lanes per column (or per plan segment): strided partial sums, DPP butterfly inside the row.
-template <bool PERM>
+// 16 lanes per column: strided partial sums (four loads in flight per lane, combined in a fixed
+// order), DPP butterfly inside the 16-lane row.
 __global__ __launch_bounds__(BM_BLOCK) void k_spsum_ranges(int nranges, const float* __restrict__ vals,
-                                                           const int* __restrict__ perm,
                                                            const int* __restrict__ ptr,
                                                            float* __restrict__ out, int beta) {
     const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
@@ -21,23 +20,47 @@ __global__ __launch_bounds__(BM_BLOCK) void k_spsum_ranges(int nranges, const fl
     float acc = 0.f;
     if (c < nranges) {
         const int s = ptr[c], e = ptr[c + 1];
-        // four loads in flight per lane; the four running sums are combined in a fixed order
         float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
         int j = s + l;
         for (; j + 48 < e; j += 64) {
-            if (PERM) {
-                const int p0 = perm[j], p1 = perm[j + 16], p2 = perm[j + 32], p3 = perm[j + 48];
-                a0 += vals[p0]; a1 += vals[p1]; a2 += vals[p2]; a3 += vals[p3];
-            } else {
-                const float v0 = vals[j], v1 = vals[j + 16], v2 = vals[j + 32], v3 = vals[j + 48];
-                a0 += v0; a1 += v1; a2 += v2; a3 += v3;
-            }
+            const float v0 = vals[j], v1 = vals[j + 16], v2 = vals[j + 32], v3 = vals[j + 48];
+            a0 += v0; a1 += v1; a2 += v2; a3 += v3;
         }
-        for (; j < e; j += 16) a0 += PERM ? vals[perm[j]] : vals[j];
+        for (; j < e; j += 16) a0 += vals[j];
         acc = (a0 + a1) + (a2 + a3);
     }
     acc = group_allsum<16>(acc);
     if (c < nranges && l == 0) out[c] = beta ? out[c] + acc : acc;
+}
+
+// Sums of the plan's segments, walked in the plan's XCD order (workgroup b runs on XCD b % 8 and
+// takes that XCD's group of heavy segments, panel after panel, then every 8th light segment): the
+// values a panel's segments pick through `perm` lie in that panel's columns, a few MiB that stay
+// in the XCD's L2 while all heavy rows of the panel are summed.
+struct XcdStarts { int v[9]; };
+__global__ __launch_bounds__(BM_BLOCK) void k_spsum_plan(int nseg, XcdStarts xs, const float* __restrict__ vals,
+                                                         const int* __restrict__ perm,
+                                                         const int* __restrict__ segstart,
+                                                         float* __restrict__ out) {
+    const int xcd = blockIdx.x & 7;
+    const long long wi = (long long)(blockIdx.x >> 3) * (BM_BLOCK / 16) + (threadIdx.x >> 4);
+    const int l = threadIdx.x & 15;
+    const int hstart = xs.v[xcd], hcount = xs.v[xcd + 1] - hstart;
+    const long long seg = wi < hcount ? hstart + wi : xs.v[8] + (wi - hcount) * 8 + xcd;
+    float acc = 0.f;
+    if (seg < nseg) {
+        const int s = segstart[seg], e = segstart[seg + 1];
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        int j = s + l;
+        for (; j + 48 < e; j += 64) {
+            const int p0 = perm[j], p1 = perm[j + 16], p2 = perm[j + 32], p3 = perm[j + 48];
+            a0 += vals[p0]; a1 += vals[p1]; a2 += vals[p2]; a3 += vals[p3];
+        }
+        for (; j < e; j += 16) a0 += vals[perm[j]];
+        acc = (a0 + a1) + (a2 + a3);
+    }
+    acc = group_allsum<16>(acc);
+    if (seg < nseg && l == 0) out[seg] = acc;
 }
 
 // ------------------------------------------------------------------ dense
@@ -237,16 +260,22 @@ hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, floa
     if (ncols <= 0) return hipSuccess;
     long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(k_spsum_ranges<false>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, vals, nullptr, jc, out, beta);
+    hipLaunchKernelGGL(k_spsum_ranges, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, vals, jc, out, beta);
     return hipGetLastError();
 }
 
-hipError_t spsum_segments(int nseg, const float* vals, const int* perm, const int* segstart,
+hipError_t spsum_segments(int nseg, const int* xcd_start, const float* vals, const int* perm, const int* segstart,
                           float* partial, hipStream_t s) {
     if (nseg <= 0) return hipSuccess;
-    long long nblk = ((long long)nseg * 16 + BM_BLOCK - 1) / BM_BLOCK;
+    XcdStarts xs;
+    int maxheavy = 0;
+    for (int x = 0; x < 9; ++x) xs.v[x] = xcd_start[x];
+    for (int x = 0; x < 8; ++x) maxheavy = xs.v[x + 1] - xs.v[x] > maxheavy ? xs.v[x + 1] - xs.v[x] : maxheavy;
+    const long long nlight = (long long)nseg - xs.v[8];
+    const long long per_xcd = (long long)maxheavy + (nlight + 7) / 8;          // segments per XCD
+    const long long nblk = 8 * ((per_xcd + BM_BLOCK / 16 - 1) / (BM_BLOCK / 16));
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(k_spsum_ranges<true>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, nseg, vals, perm, segstart, partial, 0);
+    hipLaunchKernelGGL(k_spsum_plan, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, nseg, xs, vals, perm, segstart, partial);
     return hipGetLastError();
 }
 
