@@ -380,6 +380,26 @@ API int bidmat_csc_expand_cols(int ncols, int nnz, const int* Sjc, int* Sic, voi
     return (int)bm::csc_expand_cols(ncols, nnz, Sjc, Sic, as_stream(stream));
 }
 
+API int bidmat_csc_colslice_range(int ncols, int col1, int col2, const int* Sjc, int* start, int* nnz) {
+    if (ncols < 0 || col1 < 0 || col2 < col1 || col2 > ncols || !Sjc || !start || !nnz) return kInvalid;
+    int lo = 0, hi = 0;
+    hipError_t e = hipMemcpy(&lo, Sjc + col1, sizeof(int), hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemcpy(&hi, Sjc + col2, sizeof(int), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return (int)e;
+    if (lo < 0 || hi < lo) return kInvalid;
+    *start = lo;
+    *nnz = hi - lo;
+    return 0;
+}
+
+API int bidmat_csc_colslice(int col1, int col2, int start, int nnz, const int* Sjc, const int* Sir, const float* Sdata,
+                            int* out_jc, int* out_ir, int* out_ic, float* out_data, void* stream) {
+    if (col1 < 0 || col2 < col1 || start < 0 || nnz < 0) return kInvalid;
+    if (!Sjc || !out_jc || (nnz > 0 && (!Sir || !Sdata || !out_ir || !out_data))) return kInvalid;
+    return (int)bm::csc_colslice(col2 - col1, start, nnz, Sjc + col1, Sir, Sdata, out_jc, out_ir, out_ic, out_data,
+                                 as_stream(stream));
+}
+
 API int bidmat_coo_compress_cols(int ncols, int nnz, const int* Sic, int* Sjc, void* stream) {
     if (ncols < 0 || nnz < 0) return kInvalid;
     if (!Sjc || (nnz > 0 && !Sic)) return kInvalid;

@@ -95,6 +95,24 @@ __global__ void k_digest_init(unsigned long long* out) {
     if (threadIdx.x == 2) { out[2] = 0; *reinterpret_cast<int*>(out + 2) = -1; }
 }
 
+// Columns [col1, col1+nc) of a CSC matrix as a matrix of its own: nonzero range copied, column
+// pointer rebased to 0, per-nonzero column rebuilt afterwards by k_expand_cols.
+__global__ __launch_bounds__(BM_BLOCK) void k_colslice(int nc, int start, int n, const int* __restrict__ jc_at_col1,
+                                                       const int* __restrict__ ir, const float* __restrict__ data,
+                                                       int* __restrict__ out_jc, int* __restrict__ out_ir,
+                                                       float* __restrict__ out_data) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    const long long lim = n > nc + 1 ? n : nc + 1;
+    for (; i < lim; i += stride) {
+        if (i < n) {
+            out_ir[i] = ir[(long long)start + i];
+            out_data[i] = data[(long long)start + i];
+        }
+        if (i <= nc) out_jc[i] = jc_at_col1[i] - start;
+    }
+}
+
 inline unsigned grid_for(long long n, int maxblocks = 8192) {
     long long b = (n + BM_BLOCK - 1) / BM_BLOCK;
     if (b < 1) b = 1;
@@ -130,6 +148,16 @@ hipError_t fill_i32(int* out, long long n, int v, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_fill<int>, dim3(grid_for(n)), dim3(BM_BLOCK), 0, s, out, n, v);
     return hipGetLastError();
+}
+
+hipError_t csc_colslice(int nc, int start, int n, const int* jc_at_col1, const int* ir, const float* data,
+                        int* out_jc, int* out_ir, int* out_ic, float* out_data, hipStream_t s) {
+    const long long lim = n > nc + 1 ? n : (long long)nc + 1;
+    hipLaunchKernelGGL(k_colslice, dim3(grid_for(lim, 16384)), dim3(BM_BLOCK), 0, s, nc, start, n, jc_at_col1, ir, data,
+                       out_jc, out_ir, out_data);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess && out_ic != nullptr) e = csc_expand_cols(nc, n, out_jc, out_ic, s);
+    return e;
 }
 
 hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s) {

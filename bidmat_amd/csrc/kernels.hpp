@@ -13,6 +13,10 @@ int opt_heavy_min();   // a row is cut by panels when it averages at least this 
 // ---- CSC utilities (csc_util.hip)
 hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);
 hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStream_t s);
+// columns [col1, col1+nc) with n nonzeros starting at position `start`: out_jc (nc+1, rebased),
+// out_ir / out_data (n), out_ic (n, nullable)
+hipError_t csc_colslice(int nc, int start, int n, const int* jc_at_col1, const int* ir, const float* data,
+                        int* out_jc, int* out_ir, int* out_ic, float* out_data, hipStream_t s);
 // out[i] = v for i < n (a kernel, so that callers may record it into a HIP graph)
 hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
 hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);

@@ -427,6 +427,19 @@ GSMatP GSMat::copy(GSMatP omat, long long key1, long long key2) {
     return out;
 }
 
+GSMatP GSMat::colslice(int col1, int col2, GSMatP omat) {
+    if (col1 < 0 || col2 < col1 || col2 > ncols) fail("GSMat.colslice: column range outside the matrix");
+    int starti = 0, newnnz = 0;
+    hipcheck(bidmat_csc_colslice_range(ncols, col1, col2, pjc, &starti, &newnnz), "GSMAT.colslice");
+    const int newncols = col2 - col1;
+    GSMatP out = newOrCheckGSMat(nrows, newncols, newnnz, newnnz, omat, GUID, col1, col2, opHash("colslice"));
+    int err = bidmat_csc_colslice(col1, col2, starti, newnnz, pjc, pir, pdata, out->pjc, out->pir, out->pic, out->pdata, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("HIP error in GSMAT.colslice ") + bidmat_error_string(err));
+    out->planHolder = std::make_shared<PlanHolder>();      // another pattern: any plan is rebuilt on demand
+    return out;
+}
+
 GSMatP GSMat::GSDop(const GMatP& b, GSMatP omat, int op) {
     if (b->nrows > 1 && b->ncols > 1) fail("Sorry only edge operators supported for GSMat op GMat");
     if (b->nrows != nrows && b->ncols != ncols && b->length() > 1) fail("GSMat op GMat: dimensions mismatch");

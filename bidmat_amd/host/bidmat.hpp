@@ -144,6 +144,7 @@ public:
     GMatP sum(int n, GMatP oldmat);                              // GSMat.scala:250-261
     GSMatP GSDop(const GMatP& b, GSMatP omat, int op);           // this op edge vector (GSMat.scala:315-330)
     GSMatP copy(GSMatP omat, long long key1, long long key2);    // GSMat.copy / copyTo
+    GSMatP colslice(int col1, int col2, GSMatP omat = nullptr);  // columns [col1, col2)  (GSMat.scala:77-104)
     GMatP SDMult(const GMatP& a, GMatP omat);                    // this * a    (GSMat.scala:265-289)
     GMatP SDTMult(const GMatP& a, GMatP omat);                   // this ^* a   (GSMat.scala:291-313)
     static GSMatP DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat);   // GSMat.scala:649-667

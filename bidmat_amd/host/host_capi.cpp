@@ -94,6 +94,9 @@ API void* bmh_sdmult(void* s, void* a, void* out, int transposed) {
 API void* bmh_gsdop(void* s, void* b, void* out, int op) {
     return guard_ptr([&] { return wrap(S(s)->GSDop(G(b), S(out), op)); });
 }
+API void* bmh_colslice(void* s, int col1, int col2, void* out) {
+    return guard_ptr([&] { return wrap(S(s)->colslice(col1, col2, S(out))); });
+}
 API void* bmh_dds(void* a, void* b, void* c, void* out) {
     return guard_ptr([&] { return wrap(GSMat::DDS(G(a), G(b), S(c), S(out))); });
 }

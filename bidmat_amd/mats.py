@@ -31,7 +31,7 @@ def _load():
         L = C.CDLL(LIB_PATH)
         for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
                      "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
-                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop", "bmh_load_gsmat"):
+                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop", "bmh_load_gsmat", "bmh_colslice"):
             getattr(L, name).restype = vp
         L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
         L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
@@ -41,6 +41,7 @@ def _load():
         L.bmh_dds.argtypes = [vp, vp, vp, vp]
         L.bmh_sdmult.argtypes = [vp, vp, vp, C.c_int]
         L.bmh_gsdop.argtypes = [vp, vp, vp, C.c_int]
+        L.bmh_colslice.argtypes = [vp, C.c_int, C.c_int, vp]
         L.bmh_load_gsmat.argtypes = [C.c_char_p]
         ip = C.POINTER(C.c_int)
         L.bmh_save_smat.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, vp, vp, vp]
@@ -232,6 +233,9 @@ class GSMat(_Handle):
 
     def contents(self):
         return GMat(_load().bmh_contents(self._h))
+
+    def colslice(self, col1, col2, out=None):     # columns [col1, col2)
+        return GSMat(_load().bmh_colslice(self._h, col1, col2, out._h if out else None))
 
     def GSDop(self, b, op, out=None):     # s op edge-vector (row vector, column vector or 1x1)
         return GSMat(_load().bmh_gsdop(self._h, b._h, out._h if out else None, op))

@@ -149,6 +149,18 @@ int bidmat_spsum_rows_plan(bidmat_plan *plan, const float *Sdata, float *out, in
 /* jc[ncols+1] -> ic[nnz] (per-nonzero column index).  Replaces cusparseXcsr2coo at
  * GSMat.scala:639.  Enqueues on stream. */
 int bidmat_csc_expand_cols(int ncols, int nnz, const int *Sjc, int *Sic, void *stream);
+/* Columns [col1, col2) of a device CSC matrix as a matrix of its own; replaces the four copies
+ * and two index subtractions of GSMat.colslice (GSMat.scala:77-104).  First ask for the range
+ * (blocking: reads Sjc[col1] and Sjc[col2]), allocate the outputs, then slice (enqueue only):
+ * out_jc[0..col2-col1] rebased to 0, out_ir / out_data the nnz nonzeros from position start,
+ * out_ic (nullable) the rebased column of every nonzero.
+ * The product entries do not need a copy for a column range: pass Sjc + col1 with
+ * ncols = col2 - col1 and the unsliced Sir / Sdata (column pointers are absolute positions). */
+int bidmat_csc_colslice_range(int ncols, int col1, int col2, const int *Sjc, int *start, int *nnz);
+int bidmat_csc_colslice(int col1, int col2, int start, int nnz, const int *Sjc, const int *Sir,
+                        const float *Sdata, int *out_jc, int *out_ir, int *out_ic, float *out_data,
+                        void *stream);
+
 /* non-decreasing ic[nnz] -> jc[ncols+1].  Replaces cusparseXcoo2csr at GSMat.scala:698,716
  * and SparseMat.compressInds (SparseMat.scala:857-868). Enqueues on stream. */
 int bidmat_coo_compress_cols(int ncols, int nnz, const int *Sic, int *Sjc, void *stream);

@@ -489,6 +489,53 @@ def test_expand_and_compress_cols(hip):
     d.free()
 
 
+def test_colslice_copy_and_zero_copy_column_ranges(hip):
+    """bidmat_csc_colslice against numpy slicing (bit-exact), and the zero-copy form: the product
+    entries take Sjc + col1 with the unsliced index / value arrays."""
+    rng = np.random.default_rng(96)
+    k, nrows, ncols = 64, 300, 2000
+    lengths = rng.integers(0, 40, size=ncols)
+    lengths[777] = 3000                                         # a split column inside the range
+    data, ir, jc = random_csc(rng, nrows, ncols, lengths=lengths, unique=False)
+    nnz = int(ir.size)
+    A = rng.standard_normal(k * nrows).astype(np.float32)
+    B = rng.standard_normal(k * ncols).astype(np.float32)
+    d = Dev(A=A, B=B, data=data, ir=ir, jc=jc)
+    ref, sa = oracle.fsmult_f64(A, k, data, ir, jc)
+    pref, psa = oracle.dds_f64(A, B, k, ir, jc)
+    for c1, c2 in [(0, ncols), (500, 1200), (776, 778), (1999, 2000), (100, 100)]:
+        start, n = C.c_int(-1), C.c_int(-1)
+        hip_abi.check(hip.bidmat_csc_colslice_range(ncols, c1, c2, d.jc.ptr, C.byref(start), C.byref(n)))
+        assert (start.value, n.value) == (int(jc[c1]), int(jc[c2] - jc[c1]))
+        nc, n = c2 - c1, n.value
+        o = Dev()
+        o.zeros("jc", nc + 1, np.int32), o.zeros("ir", max(n, 1), np.int32), o.zeros("ic", max(n, 1), np.int32)
+        o.zeros("data", max(n, 1))
+        hip_abi.check(hip.bidmat_csc_colslice(c1, c2, start.value, n, d.jc.ptr, d.ir.ptr, d.data.ptr,
+                                              o.jc.ptr, o.ir.ptr, o.ic.ptr, o.data.ptr, None))
+        hip_abi.check(hip.bidmat_synchronize())
+        lo, hi = int(jc[c1]), int(jc[c2])
+        assert np.array_equal(o.jc.numpy(), jc[c1:c2 + 1] - jc[c1])
+        assert np.array_equal(o.ir.numpy(n), ir[lo:hi]) and np.array_equal(o.data.numpy(n), data[lo:hi])
+        assert np.array_equal(o.ic.numpy(n), np.repeat(np.arange(nc, dtype=np.int32), np.diff(jc[c1:c2 + 1])))
+        if nc:
+            # zero-copy: column pointers are absolute positions, so a range of them is a matrix
+            o.zeros("AS", k * nc), o.zeros("P", nnz)
+            hip_abi.check(hip.bidmat_dsmult_csc(k, nc, nnz, d.A.ptr, d.data.ptr, d.ir.ptr, d.jc.ptr + 4 * c1,
+                                                o.AS.ptr, 0, None))
+            hip_abi.check(hip.bidmat_dds_csc(k, nc, nnz, d.A.ptr, d.B.ptr + 4 * k * c1, d.ir.ptr, d.jc.ptr + 4 * c1,
+                                             o.P.ptr, 0, None))
+            hip_abi.check(hip.bidmat_synchronize())
+            assert_close(o.AS.numpy(), ref[k * c1:k * c2], sa[k * c1:k * c2], "A*S on a column range")
+            P = o.P.numpy()                                     # P keeps absolute nonzero positions
+            assert_close(P[lo:hi], pref[lo:hi], psa[lo:hi], "DDS on a column range")
+            assert not P[:lo].any() and not P[hi:].any()
+        o.free()
+    assert hip.bidmat_csc_colslice_range(ncols, 5, 4, d.jc.ptr, C.byref(start), C.byref(C.c_int())) == 1
+    assert hip.bidmat_csc_colslice_range(ncols, 0, ncols + 1, d.jc.ptr, C.byref(start), C.byref(C.c_int())) == 1
+    d.free()
+
+
 # ------------------------------------------------------------------------------ error behaviour
 def test_argument_validation(hip):
     d = Dev(x=np.ones(16, dtype=np.float32), i=np.zeros(16, dtype=np.int32))

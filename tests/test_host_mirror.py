@@ -326,3 +326,36 @@ def test_sparse_op_edge_vector(hip, op, fn):
         aa.GSDop(GMat.from_numpy(rng.random((nr, nc)).astype(np.float32)), op)
     with pytest.raises(RuntimeError, match="dimensions mismatch"):
         aa.GSDop(GMat.from_numpy(rng.random((1, nc + 1)).astype(np.float32)), op)
+
+
+@gpu
+def test_colslice(hip):
+    """GSMat.colslice (GSMat.scala:77-104): the slice is a matrix of its own (pattern bit-exact,
+    column pointer rebased), usable by every product; empty and full ranges; bad ranges throw."""
+    rng = np.random.default_rng(12)
+    m, n, kk = 40, 300, 16
+    s = sprand(rng, m, n, 0.15)
+    ss = GSMat.from_csc(m, n, *s)
+    data, ir, jc = s
+    a = rng.random((kk, m)).astype(np.float32)
+    b = rng.random((kk, 57)).astype(np.float32)
+    aa = GMat.from_numpy(a)
+    for c1, c2 in [(0, n), (17, 74), (0, 1), (n - 1, n), (50, 50)]:
+        sl = ss.colslice(c1, c2)
+        assert sl.mytype == "GSMat" and sl.dims == (m, c2 - c1, int(jc[c2] - jc[c1]))
+        d2, ir2, jc2 = sl.to_csc()
+        lo, hi = jc[c1] - 1, jc[c2] - 1                           # host arrays are 1-based
+        assert np.array_equal(ir2, ir[lo:hi]) and np.array_equal(d2, data[lo:hi])
+        assert np.array_equal(jc2, jc[c1:c2 + 1] - jc[c1] + 1)
+        assert np.array_equal(sl.device_jc(), jc[c1:c2 + 1] - jc[c1])
+        if c2 > c1:
+            want = a.astype(np.float64) @ full(m, n, *s)[:, c1:c2]
+            np.testing.assert_allclose((aa * sl).numpy(), want, rtol=0, atol=EPS)
+    sl = ss.colslice(17, 74)
+    bb = GMat.from_numpy(b)                                       # kk x 57
+    want = b.astype(np.float64) @ full(m, n, *s)[:, 17:74].T      # kk x m
+    np.testing.assert_allclose(bb.xT(sl).numpy(), want, rtol=0, atol=EPS)
+    np.testing.assert_allclose(sl.sum(2).numpy().ravel(), full(m, n, *s)[:, 17:74].sum(axis=1), rtol=0, atol=EPS)
+    for bad in [(-1, 3), (5, 4), (0, n + 1)]:
+        with pytest.raises(RuntimeError, match="colslice"):
+            ss.colslice(*bad)
