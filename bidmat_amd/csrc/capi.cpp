@@ -400,6 +400,20 @@ API int bidmat_csc_colslice(int col1, int col2, int start, int nnz, const int* S
                                  as_stream(stream));
 }
 
+API int bidmat_nhot(int n, int ncols, const int* cats, int* out_ir, int* out_ic, int* out_jc, float* out_data,
+                    int* maxcat) {
+    if (n < 0 || ncols < 0 || (long long)n * ncols > 0x7fffffffLL || !out_jc) return kInvalid;
+    if ((long long)n * ncols > 0 && (!cats || !out_ir || !out_ic || !out_data)) return kInvalid;
+    hipError_t err;
+    int* d_max = (int*)bm::ws_get(bm::WS_MISC, 64, &err);
+    if (!d_max) return (int)err;
+    err = bm::nhot(n, ncols, cats, out_ir, out_ic, out_jc, out_data, d_max, nullptr);
+    int m = -1;
+    if (err == hipSuccess) err = hipMemcpy(&m, d_max, sizeof(int), hipMemcpyDeviceToHost);
+    if (maxcat) *maxcat = m;
+    return finish_blocking(err);
+}
+
 API int bidmat_coo_compress_cols(int ncols, int nnz, const int* Sic, int* Sjc, void* stream) {
     if (ncols < 0 || nnz < 0) return kInvalid;
     if (!Sjc || (nnz > 0 && !Sic)) return kInvalid;

@@ -113,6 +113,30 @@ __global__ __launch_bounds__(BM_BLOCK) void k_colslice(int nc, int start, int n,
     }
 }
 
+// n-hot pattern: column j holds the n row indices cats[j*n .. j*n+n) with value 1 (rows in the
+// given order, repeats allowed); also the largest category, for callers that size the matrix by it.
+__global__ __launch_bounds__(BM_BLOCK) void k_nhot(int n, int ncols, const int* __restrict__ cats,
+                                                   int* __restrict__ ir, int* __restrict__ ic, int* __restrict__ jc,
+                                                   float* __restrict__ data, int* __restrict__ maxcat) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    const long long total = (long long)n * ncols;
+    int m = -1;
+    for (; i < total || i <= ncols; i += stride) {
+        if (i < total) {
+            const int r = cats[i];
+            ir[i] = r;
+            ic[i] = (int)(i / n);
+            data[i] = 1.0f;
+            m = max(m, r);
+        }
+        if (i <= ncols) jc[i] = (int)(i * n);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = max(m, __shfl_xor(m, d, 64));
+    if ((threadIdx.x & 63) == 0 && m >= 0) atomicMax(maxcat, m);
+}
+
 inline unsigned grid_for(long long n, int maxblocks = 8192) {
     long long b = (n + BM_BLOCK - 1) / BM_BLOCK;
     if (b < 1) b = 1;
@@ -158,6 +182,16 @@ hipError_t csc_colslice(int nc, int start, int n, const int* jc_at_col1, const i
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && out_ic != nullptr) e = csc_expand_cols(nc, n, out_jc, out_ic, s);
     return e;
+}
+
+hipError_t nhot(int n, int ncols, const int* cats, int* ir, int* ic, int* jc, float* data, int* d_maxcat,
+                hipStream_t s) {
+    hipError_t e = fill_i32(d_maxcat, 1, -1, s);
+    if (e != hipSuccess) return e;
+    const long long total = (long long)n * ncols;
+    const long long lim = total > (long long)ncols + 1 ? total : (long long)ncols + 1;
+    hipLaunchKernelGGL(k_nhot, dim3(grid_for(lim)), dim3(BM_BLOCK), 0, s, n, ncols, cats, ir, ic, jc, data, d_maxcat);
+    return hipGetLastError();
 }
 
 hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s) {

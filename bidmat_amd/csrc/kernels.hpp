@@ -17,6 +17,9 @@ hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStre
 // out_ir / out_data (n), out_ic (n, nullable)
 hipError_t csc_colslice(int nc, int start, int n, const int* jc_at_col1, const int* ir, const float* data,
                         int* out_jc, int* out_ir, int* out_ic, float* out_data, hipStream_t s);
+// n-hot pattern from an n x ncols category matrix; *d_maxcat (device int) receives the largest category
+hipError_t nhot(int n, int ncols, const int* cats, int* ir, int* ic, int* jc, float* data, int* d_maxcat,
+                hipStream_t s);
 // out[i] = v for i < n (a kernel, so that callers may record it into a HIP graph)
 hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
 hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);

@@ -427,6 +427,28 @@ GSMatP GSMat::copy(GSMatP omat, long long key1, long long key2) {
     return out;
 }
 
+GSMatP GSMat::nHot(const std::vector<int>& cats, int n, int ncols, int ncats0) {
+    if (n < 0 || ncols < 0 || (long long)cats.size() != (long long)n * ncols) fail("GSMat.nHot: category matrix has the wrong size");
+    const int len = n * ncols;
+    void* dcats = nullptr;
+    hipcheck(bidmat_malloc(&dcats, (long long)sizeof(int) * len), "GSMat.nHot");
+    GSMatP out;
+    try {
+        hipcheck(bidmat_memcpy_h2d(dcats, cats.data(), (long long)sizeof(int) * len), "GSMat.nHot category copy error");
+        out = make(ncats0, ncols, len, len);
+        int maxcat = -1;
+        int err = bidmat_nhot(n, ncols, static_cast<const int*>(dcats), out->pir, out->pic, out->pjc, out->pdata, &maxcat);
+        if (err != 0) fail(std::string("HIP error in GSMat.nHot ") + bidmat_error_string(err));
+        if (ncats0 == 0) out->nrows = maxcat + 1;
+        else if (maxcat >= ncats0) fail("GSMat.nHot: category outside the matrix");
+    } catch (...) {
+        (void)bidmat_free(dcats);
+        throw;
+    }
+    hipcheck(bidmat_free(dcats), "GSMat.nHot");
+    return out;
+}
+
 GSMatP GSMat::colslice(int col1, int col2, GSMatP omat) {
     if (col1 < 0 || col2 < col1 || col2 > ncols) fail("GSMat.colslice: column range outside the matrix");
     int starti = 0, newnnz = 0;

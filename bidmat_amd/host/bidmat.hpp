@@ -137,6 +137,9 @@ public:
     std::string mytype() const { return "GSMat"; }
     static GSMatP make(int nr, int nc, int nnz, int realnnz);
     static GSMatP fromSMat(const SMat& a, GSMatP b = nullptr);   // GSMat.scala:620-647
+    // oneHot (n = 1) / nHot: cats is an n x ncols category matrix (column-major, 0-based);
+    // ncats0 == 0: rows = largest category + 1  (GSMat.scala:686-720)
+    static GSMatP nHot(const std::vector<int>& cats, int n, int ncols, int ncats0);
     SMat toSMat() const;                                         // GSMat.scala:108-127
     GMatP contents();                                            // GSMat.scala:21-25
     GSMat& clear();

@@ -94,6 +94,12 @@ API void* bmh_sdmult(void* s, void* a, void* out, int transposed) {
 API void* bmh_gsdop(void* s, void* b, void* out, int op) {
     return guard_ptr([&] { return wrap(S(s)->GSDop(G(b), S(out), op)); });
 }
+API void* bmh_nhot(const int* cats, int n, int ncols, int ncats) {
+    return guard_ptr([&] {
+        std::vector<int> c(cats, cats + (size_t)n * (size_t)ncols);
+        return wrap(GSMat::nHot(c, n, ncols, ncats));
+    });
+}
 API void* bmh_colslice(void* s, int col1, int col2, void* out) {
     return guard_ptr([&] { return wrap(S(s)->colslice(col1, col2, S(out))); });
 }

@@ -31,7 +31,7 @@ def _load():
         L = C.CDLL(LIB_PATH)
         for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
                      "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
-                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop", "bmh_load_gsmat", "bmh_colslice"):
+                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop", "bmh_load_gsmat", "bmh_colslice", "bmh_nhot"):
             getattr(L, name).restype = vp
         L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
         L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
@@ -42,6 +42,7 @@ def _load():
         L.bmh_sdmult.argtypes = [vp, vp, vp, C.c_int]
         L.bmh_gsdop.argtypes = [vp, vp, vp, C.c_int]
         L.bmh_colslice.argtypes = [vp, C.c_int, C.c_int, vp]
+        L.bmh_nhot.argtypes = [vp, C.c_int, C.c_int, C.c_int]
         L.bmh_load_gsmat.argtypes = [C.c_char_p]
         ip = C.POINTER(C.c_int)
         L.bmh_save_smat.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, vp, vp, vp]
@@ -208,6 +209,18 @@ class GSMat(_Handle):
         ir = np.ascontiguousarray(ir, dtype=np.int32)
         jc = np.ascontiguousarray(jc, dtype=np.int32)
         return cls(_load().bmh_gsmat_from_host(nrows, ncols, data.size, data.ctypes.data, ir.ctypes.data, jc.ctypes.data))
+
+    @classmethod
+    def nHot(cls, cats, ncats=0):
+        """GSMat.nHot / oneHot: cats is an n x ncols (or 1-D = one-hot) array of 0-based categories."""
+        cats = np.asarray(cats, dtype=np.int32)
+        if cats.ndim == 1:
+            cats = cats.reshape(1, -1)
+        n, ncols = cats.shape
+        flat = np.ascontiguousarray(cats.T).ravel()                  # column-major
+        return cls(_load().bmh_nhot(flat.ctypes.data, n, ncols, ncats))
+
+    oneHot = nHot
 
     @property
     def dims(self):

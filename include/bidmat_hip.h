@@ -149,6 +149,15 @@ int bidmat_spsum_rows_plan(bidmat_plan *plan, const float *Sdata, float *out, in
 /* jc[ncols+1] -> ic[nnz] (per-nonzero column index).  Replaces cusparseXcsr2coo at
  * GSMat.scala:639.  Enqueues on stream. */
 int bidmat_csc_expand_cols(int ncols, int nnz, const int *Sjc, int *Sic, void *stream);
+/* One-hot / n-hot pattern (GSMat.oneHot / GSMat.nHot, GSMat.scala:686-720): cats is an
+ * n x ncols device int matrix of categories; column j of the result holds rows cats[:, j] in
+ * the given order (not sorted, repeats allowed) with value 1.  Outputs: out_ir, out_ic,
+ * out_data (n*ncols each), out_jc (ncols+1).  *maxcat (host, nullable) receives the largest
+ * category (-1 when empty), which the reference uses as nrows-1 when ncats is not given.
+ * Replaces a D2D copy, setval, initSeq and cusparseXcoo2csr.  Blocking. */
+int bidmat_nhot(int n, int ncols, const int *cats, int *out_ir, int *out_ic, int *out_jc,
+                float *out_data, int *maxcat);
+
 /* Columns [col1, col2) of a device CSC matrix as a matrix of its own; replaces the four copies
  * and two index subtractions of GSMat.colslice (GSMat.scala:77-104).  First ask for the range
  * (blocking: reads Sjc[col1] and Sjc[col2]), allocate the outputs, then slice (enqueue only):

@@ -359,3 +359,38 @@ def test_colslice(hip):
     for bad in [(-1, 3), (5, 4), (0, n + 1)]:
         with pytest.raises(RuntimeError, match="colslice"):
             ss.colslice(*bad)
+
+
+@gpu
+def test_onehot_and_nhot(hip):
+    """GSMat.oneHot / nHot (GSMat.scala:686-720): patterns with unsorted, repeated rows built on the
+    device; A * oneHot(c) is a pure gather (bit-exact), nHot sums the chosen columns."""
+    rng = np.random.default_rng(13)
+    kk, ncats, n = 24, 37, 500
+    a = rng.standard_normal((kk, ncats)).astype(np.float32)
+    aa = GMat.from_numpy(a)
+    c = rng.integers(0, ncats, size=n).astype(np.int32)
+    c[7] = ncats - 1
+    s1 = GSMat.oneHot(c)                                          # ncats from the largest category
+    assert s1.mytype == "GSMat" and s1.dims == (ncats, n, n)
+    assert np.array_equal(s1.device_jc(), np.arange(n + 1))
+    assert np.array_equal((aa * s1).numpy(), a[:, c])             # 1.0f * x added to 0: exact
+    d, ir, jc = s1.to_csc()
+    assert np.array_equal(ir, c + 1) and np.array_equal(d, np.ones(n, np.float32))
+    s1b = GSMat.oneHot(c, 50)
+    assert s1b.dims == (50, n, n)
+    with pytest.raises(RuntimeError, match="category outside"):
+        GSMat.oneHot(c, ncats - 1)
+    # n-hot with rows in arbitrary order and repeats inside a column
+    cats = rng.integers(0, ncats, size=(3, 200)).astype(np.int32)
+    cats[:, 5] = 4
+    s3 = GSMat.nHot(cats, ncats)
+    assert s3.dims == (ncats, 200, 600) and np.array_equal(s3.device_jc(), 3 * np.arange(201))
+    want = sum(a.astype(np.float64)[:, cats[i]] for i in range(3))
+    np.testing.assert_allclose((aa * s3).numpy(), want, rtol=0, atol=EPS)
+    b = rng.standard_normal((kk, 200)).astype(np.float32)
+    wantT = np.zeros((kk, ncats))
+    for i in range(3):
+        np.add.at(wantT.T, cats[i], b.astype(np.float64).T)
+    np.testing.assert_allclose(GMat.from_numpy(b).xT(s3).numpy(), wantT, rtol=0, atol=EPS)
+    np.testing.assert_allclose(s3.sum(2).numpy().ravel(), np.bincount(cats.ravel(), minlength=ncats), rtol=0, atol=EPS)
