@@ -104,6 +104,28 @@ JFN(jint, setOption)(JNIEnv* env, jclass, jstring name, jlong value) {
     return e;
 }
 JFN(jint, releaseCaches)(JNIEnv*, jclass) { return bidmat_release_caches(); }
+// GSMat.oneHot / nHot (GSMat.scala:686-720); returns -(error) or the largest category + 1
+JFN(jint, nhot)(JNIEnv*, jclass, jint n, jint nc, jlong cats, jlong oir, jlong oic, jlong ojc, jlong odata) {
+    int maxcat = -1;
+    int e = bidmat_nhot(n, nc, P(const int, cats), P(int, oir), P(int, oic), P(int, ojc), P(float, odata), &maxcat);
+    return e ? -e : maxcat + 1;
+}
+// GSMat.colslice (GSMat.scala:77-104): range[0] = first nonzero, range[1] = number of nonzeros
+JFN(jint, cscColsliceRange)(JNIEnv* env, jclass, jint nc, jint col1, jint col2, jlong Sjc, jintArray range) {
+    int start = 0, nnz = 0;
+    int e = bidmat_csc_colslice_range(nc, col1, col2, P(const int, Sjc), &start, &nnz);
+    if (e) return e;
+    jint* r = static_cast<jint*>(env->GetPrimitiveArrayCritical(range, nullptr));
+    r[0] = start; r[1] = nnz;
+    env->ReleasePrimitiveArrayCritical(range, r, 0);
+    return 0;
+}
+JFN(jint, cscColslice)(JNIEnv*, jclass, jint col1, jint col2, jint start, jint nnz, jlong Sjc, jlong Sir, jlong Sdata,
+                       jlong ojc, jlong oir, jlong oic, jlong odata) {
+    int e = bidmat_csc_colslice(col1, col2, start, nnz, P(const int, Sjc), P(const int, Sir), P(const float, Sdata),
+                                P(int, ojc), P(int, oir), P(int, oic), P(float, odata), nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
 JFN(jint, cscExpandCols)(JNIEnv*, jclass, jint nc, jint nnz, jlong Sjc, jlong Sic) {
     int e = bidmat_csc_expand_cols(nc, nnz, P(const int, Sjc), P(int, Sic), nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
