@@ -62,19 +62,28 @@ __global__ __launch_bounds__(BM_BLOCK) void k_heavy_flag(int nrows, const int* _
     if (r < nrows) flag[r] = cnt[r] >= thresh ? 1 : 0;
 }
 
-// hrow[hrank[r]] = r for heavy rows
-__global__ __launch_bounds__(BM_BLOCK) void k_heavy_rows(int nrows, const int* __restrict__ flag,
+// hrow[hrank[r]] = r for heavy rows; flag[r] becomes the row's code for the key kernel: its
+// heavy rank, or -1 for a light row (one lookup per nonzero instead of two).
+__global__ __launch_bounds__(BM_BLOCK) void k_heavy_rows(int nrows, int* __restrict__ flag,
                                                          const int* __restrict__ hrank, int* __restrict__ hrow) {
     const long long r = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    if (r < nrows && flag[r]) hrow[hrank[r]] = (int)r;
+    if (r >= nrows) return;
+    if (flag[r]) {
+        const int h = hrank[r];
+        hrow[h] = (int)r;
+        flag[r] = h;
+    } else {
+        flag[r] = -1;
+    }
 }
 
-// 16 lanes per column: key and original position of every nonzero.
+// 16 lanes per column: key of every nonzero, and its (column, original position) as the value
+// that is sorted along with it.
 __global__ __launch_bounds__(BM_BLOCK) void k_make_keys(int ncols, int nrows, const int* __restrict__ jc,
-                                                        const int* __restrict__ ir, const int* __restrict__ flag,
-                                                        const int* __restrict__ hrank, int nheavy, int npanels,
+                                                        const int* __restrict__ ir, const int* __restrict__ hcode,
+                                                        int nheavy, int npanels,
                                                         int panel_cols, int p8, unsigned* __restrict__ keys,
-                                                        int* __restrict__ pos) {
+                                                        unsigned long long* __restrict__ colpos) {
     const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long c = t >> 4;
     const int l = (int)(t & 15);
@@ -88,8 +97,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_make_keys(int ncols, int nrows, co
     for (int j = s + l; j < e; j += 16) {
         int r = ir[j];
         r = r < 0 ? 0 : (r >= nrows ? nrows - 1 : r);
-        keys[j] = flag[r] ? panel * (unsigned)nheavy + (unsigned)hrank[r] : light_base + (unsigned)r;
-        pos[j] = j;
+        const int h = hcode[r];                         // heavy rank, or -1
+        keys[j] = h >= 0 ? panel * (unsigned)nheavy + (unsigned)h : light_base + (unsigned)r;
+        colpos[j] = ((unsigned long long)(unsigned)c << 32) | (unsigned)j;   // travels with the key
     }
 }
 
@@ -101,12 +111,14 @@ __global__ __launch_bounds__(BM_BLOCK) void k_boundaries(int nnz, int seglen, co
         flag[p] = (p == 0 || keys[p] != keys[p - 1] || (p % seglen) == 0) ? 1 : 0;
 }
 
-// Column of every nonzero in plan order; segment tables at the flagged positions.
+// Column and original position of every nonzero in plan order; segment tables at the flagged
+// positions.
 __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __restrict__ keys,
-                                                   const int* __restrict__ perm, const int* __restrict__ ic,
+                                                   const unsigned long long* __restrict__ colpos,
                                                    const int* __restrict__ flag, const int* __restrict__ segidx,
                                                    const int* __restrict__ hrow, int nheavy, int p8,
-                                                   int* __restrict__ pc, int* __restrict__ segstart,
+                                                   int* __restrict__ pc, int* __restrict__ perm,
+                                                   int* __restrict__ segstart,
                                                    unsigned* __restrict__ segrow, int* __restrict__ segid,
                                                    unsigned char* __restrict__ segclass) {
     long long p = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
@@ -114,7 +126,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __re
     const unsigned per_xcd = (unsigned)p8 * (unsigned)nheavy;     // keys per XCD group
     const unsigned light_base = 8u * per_xcd;
     for (; p < nnz; p += stride) {
-        pc[p] = ic[perm[p]];
+        const unsigned long long cp = colpos[p];
+        pc[p] = (int)(cp >> 32);
+        perm[p] = (int)(cp & 0xffffffffULL);
         if (flag[p]) {
             const int sidx = segidx[p];
             const unsigned key = keys[p];
@@ -246,16 +260,17 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         // both sorts share one scratch area, sized for the larger request (the second sort has
         // at most nnz items)
         size_t b1 = 0, b2 = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b1, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
-                                           (int*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b1, (unsigned*)nullptr, (unsigned*)nullptr, (unsigned long long*)nullptr,
+                                           (unsigned long long*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
         PB_CHECK(rocprim::radix_sort_pairs(nullptr, b2, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
                                            (int*)nullptr, (size_t)nnz, 0, rbits, s));
         sort_bytes = b1 > b2 ? b1 : b2;
     }
     Arena tmp;
     int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *scantmp = nullptr, *class_count = nullptr;
-    int *pos_in = nullptr, *ic = nullptr, *flag = nullptr, *segidx = nullptr;
+    int *flag = nullptr, *segidx = nullptr;
     unsigned *keys_in = nullptr, *keys_out = nullptr;
+    unsigned long long *colpos_in = nullptr, *colpos_out = nullptr;
     unsigned char* segclass = nullptr;
     char* sorttmp = nullptr;
     for (int pass = 0; pass < 2; ++pass) {
@@ -268,8 +283,8 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         class_count = tmp.take<int>(9);
         keys_in = tmp.take<unsigned>((size_t)nnz);       // later: ids of the segments
         keys_out = tmp.take<unsigned>((size_t)nnz);
-        pos_in = tmp.take<int>((size_t)nnz);             // later: segment rows in sorted order
-        ic = tmp.take<int>((size_t)nnz);
+        colpos_in = tmp.take<unsigned long long>((size_t)nnz);   // later: segment rows in sorted order
+        colpos_out = tmp.take<unsigned long long>((size_t)nnz);
         flag = tmp.take<int>((size_t)nnz);
         segidx = tmp.take<int>((size_t)nnz + 1);
         segclass = tmp.take<unsigned char>((size_t)nnz);
@@ -307,8 +322,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         if (8ULL * (unsigned long long)p8 * (unsigned long long)nheavy + (unsigned long long)nrows > 0xffffffffULL) nheavy = 0;
     }
     if (nheavy == 0) {
-        PB_CHECK(fill_i32(hflag, nrows, 0, s));
-        PB_CHECK(fill_i32(hrank, (long long)nrows + 1, 0, s));
+        PB_CHECK(fill_i32(hflag, nrows, -1, s));        // every row is light
     } else {
         hipLaunchKernelGGL(k_heavy_rows, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, hflag, hrank, hrow);
     }
@@ -318,19 +332,18 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     {
         long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
         hipLaunchKernelGGL(k_make_keys, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nrows, jc, ir,
-                           hflag, hrank, nheavy, plan->npanels, plan->panel_cols, p8, keys_in, pos_in);
+                           hflag, nheavy, plan->npanels, plan->panel_cols, p8, keys_in, colpos_in);
     }
     const unsigned long long maxkey = 8ULL * (unsigned long long)p8 * nheavy + (unsigned long long)nrows;
     const int end_bit = bits_for(maxkey);
     {
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in, keys_out, pos_in, plan->perm, (size_t)nnz, 0, end_bit, s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in, keys_out, colpos_in, colpos_out, (size_t)nnz, 0, end_bit, s));
         if (tmp_bytes > sort_bytes) { (void)plan_free(plan); return hipErrorOutOfMemory; }
-        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, keys_in, keys_out, pos_in, plan->perm, (size_t)nnz, 0, end_bit, s));
+        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, keys_in, keys_out, colpos_in, colpos_out, (size_t)nnz, 0, end_bit, s));
     }
 
     // 4. segment boundaries
-    PB_CHECK(csc_expand_cols(ncols, nnz, jc, ic, s));
     hipLaunchKernelGGL(k_boundaries, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, plan->seglen, keys_out, flag);
     PB_CHECK(scan_exclusive_i32(flag, segidx, nnz, scantmp, s));
     int nseg = 0;
@@ -354,12 +367,12 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     }
     // the sort's inputs are dead by now: their space holds the segment ids and the sorted rows
     int* const segid = reinterpret_cast<int*>(keys_in);
-    unsigned* const segrow_sorted = reinterpret_cast<unsigned*>(pos_in);
+    unsigned* const segrow_sorted = reinterpret_cast<unsigned*>(colpos_in);
     unsigned* const segrow_u = reinterpret_cast<unsigned*>(plan->segrow);
     PB_CHECK(fill_i32(class_count, 9, nseg, s));
-    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out, plan->perm,
-                       ic, flag, segidx, hrow, nheavy > 0 ? nheavy : 1,
-                       nheavy > 0 ? p8 : 0, plan->pc, plan->segstart, segrow_u, segid, segclass);
+    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out, colpos_out,
+                       flag, segidx, hrow, nheavy > 0 ? nheavy : 1,
+                       nheavy > 0 ? p8 : 0, plan->pc, plan->perm, plan->segstart, segrow_u, segid, segclass);
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
     hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg, segclass, class_count);
     PB_CHECK(hipMemcpy(plan->xcd_start, class_count, sizeof(int) * 9, hipMemcpyDeviceToHost));
