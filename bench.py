@@ -36,7 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # kernel of --calibrate, which moves a known 2 GiB + 1 GiB). The counter runs and their tables are
 # kept in profiles/headline_kernel_trace_and_hbm_counters.txt; a profiler cannot run inside this
 # script, so the figure is reported only for the exact workload it was measured on.
-MEASURED_TRAFFIC_BYTES = {("headline", "dds", 100003320): 41.9e9}
+MEASURED_TRAFFIC_BYTES = {("headline", "dds", 100003320): 41.8e9,
+                          ("C4", "dsmult", 38900534): 163.1e9}   # profiles/other_workloads_kernel_trace_and_hbm_counters.txt
 
 
 def alg_bytes(op, k, nnz, nrows, ncols):
