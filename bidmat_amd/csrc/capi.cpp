@@ -345,9 +345,9 @@ API int bidmat_sdtmult_csc(int nrows, int ncols, int nnz, int p, const float* Sd
     hipStream_t s = as_stream(stream);
     hipError_t err;
     // At = A^T (p x nrows), Ct = At * S (p x ncols), C = Ct^T
-    float* At = (float*)bm::ws_get(bm::WS_TRANS_IN, sizeof(float) * (size_t)p * (size_t)(nrows > 0 ? nrows : 1), &err);
+    float* At = (float*)bm::ws_get(bm::WS_TRANS_IN, sizeof(float) * (size_t)p * (size_t)(nrows > 0 ? nrows : 1), &err, s);
     if (!At) return (int)err;
-    float* Ct = (float*)bm::ws_get(bm::WS_TRANS_OUT, sizeof(float) * (size_t)p * (size_t)ncols, &err);
+    float* Ct = (float*)bm::ws_get(bm::WS_TRANS_OUT, sizeof(float) * (size_t)p * (size_t)ncols, &err, s);
     if (!Ct) return (int)err;
     if ((err = bm::transpose(nrows, p, A, lda, At, p, s)) != hipSuccess) return (int)err;
     if ((err = bm::dsmult_csc(p, ncols, nnz, At, Sdata, Sir, Sjc, Ct, 0, s)) != hipSuccess) return (int)err;
@@ -364,9 +364,9 @@ API int bidmat_sdmult_plan(bidmat_plan* plan, int p, const float* Sdata, const f
     hipStream_t s = as_stream(stream);
     hipError_t err;
     // At = A^T (p x ncols), Ct = At *^ S (p x nrows), C = Ct^T
-    float* At = (float*)bm::ws_get(bm::WS_TRANS_IN, sizeof(float) * (size_t)p * (size_t)(plan->ncols > 0 ? plan->ncols : 1), &err);
+    float* At = (float*)bm::ws_get(bm::WS_TRANS_IN, sizeof(float) * (size_t)p * (size_t)(plan->ncols > 0 ? plan->ncols : 1), &err, s);
     if (!At) return (int)err;
-    float* Ct = (float*)bm::ws_get(bm::WS_TRANS_OUT, sizeof(float) * (size_t)p * (size_t)plan->nrows, &err);
+    float* Ct = (float*)bm::ws_get(bm::WS_TRANS_OUT, sizeof(float) * (size_t)p * (size_t)plan->nrows, &err, s);
     if (!Ct) return (int)err;
     if ((err = bm::transpose(plan->ncols, p, A, lda, At, p, s)) != hipSuccess) return (int)err;
     if ((err = run_dsmultT(plan, p, At, Sdata, Ct, 0, s)) != hipSuccess) return (int)err;
@@ -500,7 +500,13 @@ API int bidmat_stream_create(void** stream) {
     *stream = (e == hipSuccess) ? (void*)s : nullptr;
     return (int)e;
 }
-API int bidmat_stream_destroy(void* stream) { return stream ? (int)hipStreamDestroy(as_stream(stream)) : 0; }
+API int bidmat_stream_destroy(void* stream) {
+    if (!stream) return 0;
+    hipError_t e = hipStreamSynchronize(as_stream(stream));
+    hipError_t f = bm::ws_drop_stream(as_stream(stream));      // the stream's scratch goes with it
+    hipError_t g = hipStreamDestroy(as_stream(stream));
+    return (int)(e != hipSuccess ? e : (f != hipSuccess ? f : g));
+}
 API int bidmat_stream_synchronize(void* stream) { return (int)hipStreamSynchronize(as_stream(stream)); }
 API int bidmat_event_create(void** event) {
     if (!event) return kInvalid;

@@ -359,7 +359,7 @@ hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, i
     *d_ovf = nullptr;
     if (nnz <= seglen || ncols <= 0) return hipSuccess;
     hipError_t err;
-    int* buf = (int*)ws_get(WS_OVF, sizeof(int) * (2 * (size_t)ncols + 2), &err);
+    int* buf = (int*)ws_get(WS_OVF, sizeof(int) * (2 * (size_t)ncols + 2), &err, s);
     if (!buf) return err;
     unsigned nblk = (unsigned)(((long long)ncols + BM_BLOCK - 1) / BM_BLOCK);
     if (nblk <= (unsigned)OVF2_MAX_BLOCKS) {
@@ -369,7 +369,7 @@ hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, i
         *d_ovf = buf;
         return hipGetLastError();
     }
-    int* tmp = (int*)ws_get(WS_SCAN, sizeof(int) * scan_tmp_ints(ncols), &err);
+    int* tmp = (int*)ws_get(WS_SCAN, sizeof(int) * scan_tmp_ints(ncols), &err, s);
     if (!tmp) return err;
     int* extra = buf;
     int* ovf = buf + ncols + 1;
@@ -404,7 +404,7 @@ hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const floa
     long long novf_max = 0;
     if (ovf) {
         novf_max = nnz / seglen;
-        partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err);
+        partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err, s);
         if (!partial) return err;
     }
     const bool al = aligned16(A) && aligned16(C) && aligned16(partial) && lda % 4 == 0 && ldc % 4 == 0;

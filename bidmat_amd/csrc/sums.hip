@@ -190,7 +190,7 @@ hipError_t reduce1_impl(int nrows, int ncols, const float* A, float* B, hipStrea
     float* dst = B;
     if (nchunks > 1) {
         hipError_t err;
-        dst = (float*)ws_get(WS_REDUCE, sizeof(float) * (size_t)nchunks * ncols, &err);
+        dst = (float*)ws_get(WS_REDUCE, sizeof(float) * (size_t)nchunks * ncols, &err, s);
         if (!dst) return err;
     }
     if (vec) hipLaunchKernelGGL((k_reduce_cols<OP, 4>), dim3((unsigned)nblk, (unsigned)nchunks), dim3(BM_BLOCK), 0, s,
@@ -233,7 +233,7 @@ hipError_t reduce2_impl(int nrows, int ncols, const float* A, float* B, hipStrea
             // 1/16 of the one before)
             hipError_t err;
             scratch_floats = need + need / 8 + 4096;
-            scratch = (float*)ws_get(WS_REDUCE, sizeof(float) * scratch_floats, &err);
+            scratch = (float*)ws_get(WS_REDUCE, sizeof(float) * scratch_floats, &err, s);
             if (!scratch) return err;
         }
         if (need > scratch_floats) return hipErrorInvalidValue;

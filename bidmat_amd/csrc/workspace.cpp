@@ -1,14 +1,17 @@
 #include "workspace.hpp"
-#include <mutex>
+#include <array>
 #include <cstdio>
 #include <cstdlib>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace bm {
 
 namespace {
-constexpr int kMaxDevices = 64;
 struct Slot { void* ptr = nullptr; size_t bytes = 0; };
-Slot g_slots[kMaxDevices][WS_NSLOTS];
+using SlotSet = std::array<Slot, WS_NSLOTS>;
+std::map<std::pair<int, hipStream_t>, SlotSet> g_sets;      // (device, stream) -> slots
 std::mutex g_mu;
 
 bool debug_mem() {
@@ -16,16 +19,26 @@ bool debug_mem() {
     if (v < 0) { const char* e = getenv("BIDMAT_DEBUG_MEM"); v = (e && e[0] == '1') ? 1 : 0; }
     return v == 1;
 }
+
+hipError_t free_set(SlotSet& set) {
+    hipError_t e = hipSuccess;
+    for (Slot& s : set) {
+        if (s.ptr) {
+            hipError_t f = hipFree(s.ptr);
+            if (f != hipSuccess) e = f;
+            s.ptr = nullptr; s.bytes = 0;
+        }
+    }
+    return e;
+}
 }  // namespace
 
-void* ws_get(WsSlot slot, size_t bytes, hipError_t* err) {
-    *err = hipSuccess;
+void* ws_get(WsSlot slot, size_t bytes, hipError_t* err, hipStream_t stream) {
     int dev = 0;
     *err = hipGetDevice(&dev);
     if (*err != hipSuccess) return nullptr;
-    if (dev < 0 || dev >= kMaxDevices) { *err = hipErrorInvalidDevice; return nullptr; }
     std::lock_guard<std::mutex> lock(g_mu);
-    Slot& s = g_slots[dev][slot];
+    Slot& s = g_sets[{dev, stream}][slot];
     if (bytes == 0) bytes = 256;
     if (s.bytes >= bytes) return s.ptr;
     if (s.ptr) {
@@ -44,17 +57,19 @@ void* ws_get(WsSlot slot, size_t bytes, hipError_t* err) {
         if (*err != hipSuccess) { s.ptr = nullptr; return nullptr; }
     }
     s.bytes = want;
-    if (debug_mem()) fprintf(stderr, "[bidmathip] workspace slot %d -> %zu bytes on device %d\n", (int)slot, want, dev);
+    if (debug_mem())
+        fprintf(stderr, "[bidmathip] workspace slot %d -> %zu bytes on device %d, stream %p\n", (int)slot, want, dev, (void*)stream);
     return s.ptr;
 }
 
-hipError_t ws_drop(WsSlot slot) {
+hipError_t ws_drop(WsSlot slot, hipStream_t stream) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
     std::lock_guard<std::mutex> lock(g_mu);
-    Slot& s = g_slots[dev][slot];
+    auto it = g_sets.find({dev, stream});
+    if (it == g_sets.end()) return hipSuccess;
+    Slot& s = it->second[slot];
     if (s.ptr) {
         e = hipFree(s.ptr);
         s.ptr = nullptr; s.bytes = 0;
@@ -62,18 +77,30 @@ hipError_t ws_drop(WsSlot slot) {
     return e;
 }
 
+hipError_t ws_drop_stream(hipStream_t stream) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_sets.find({dev, stream});
+    if (it == g_sets.end()) return hipSuccess;
+    e = free_set(it->second);
+    g_sets.erase(it);
+    return e;
+}
+
 hipError_t ws_release() {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
     std::lock_guard<std::mutex> lock(g_mu);
-    for (int i = 0; i < WS_NSLOTS; ++i) {
-        Slot& s = g_slots[dev][i];
-        if (s.ptr) {
-            hipError_t f = hipFree(s.ptr);
+    for (auto it = g_sets.begin(); it != g_sets.end();) {
+        if (it->first.first == dev) {
+            hipError_t f = free_set(it->second);
             if (f != hipSuccess) e = f;
-            s.ptr = nullptr; s.bytes = 0;
+            it = g_sets.erase(it);
+        } else {
+            ++it;
         }
     }
     return e;
@@ -81,10 +108,12 @@ hipError_t ws_release() {
 
 size_t ws_bytes() {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
     std::lock_guard<std::mutex> lock(g_mu);
     size_t t = 0;
-    for (int i = 0; i < WS_NSLOTS; ++i) t += g_slots[dev][i].bytes;
+    for (auto& kv : g_sets)
+        if (kv.first.first == dev)
+            for (const Slot& s : kv.second) t += s.bytes;
     return t;
 }
 

@@ -1,6 +1,6 @@
-// Per-device scratch buffers owned by the library (column-pointer copies, overflow-segment
-// tables, partial sums). Buffers grow on demand and are reused by later calls; calls that
-// share a device are expected to be stream-ordered with respect to each other.
+// Scratch buffers owned by the library (column-pointer copies, overflow-segment tables, partial
+// sums), one set per (device, stream): calls enqueued on different streams never share scratch,
+// calls on one stream are ordered by the stream. Buffers grow on demand and are reused.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stddef.h>
@@ -20,12 +20,15 @@ enum WsSlot {
     WS_NSLOTS
 };
 
-// Returns a device buffer of at least `bytes` for `slot` on the current device (nullptr and
-// *err set on failure). Growing a slot frees the old buffer after a device synchronise.
-void* ws_get(WsSlot slot, size_t bytes, hipError_t* err);
-// Frees one slot of the current device.
-hipError_t ws_drop(WsSlot slot);
-// Frees every slot of the current device.
+// Returns a device buffer of at least `bytes` for `slot` of `stream` on the current device
+// (nullptr and *err set on failure). Growing a slot frees the old buffer, which waits for the
+// device first.
+void* ws_get(WsSlot slot, size_t bytes, hipError_t* err, hipStream_t stream = nullptr);
+// Frees one slot of `stream` on the current device.
+hipError_t ws_drop(WsSlot slot, hipStream_t stream = nullptr);
+// Frees every slot of `stream` on the current device (called when a stream is destroyed).
+hipError_t ws_drop_stream(hipStream_t stream);
+// Frees every slot of every stream of the current device.
 hipError_t ws_release();
 // Total bytes currently held on the current device.
 size_t ws_bytes();

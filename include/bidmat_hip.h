@@ -17,7 +17,9 @@
  *   - entry points WITHOUT a stream argument block until the result is complete, like the
  *     reference's launchers (cudaStreamSynchronize, MatKernel.hpp:15).  Entry points WITH
  *     a `stream` argument (a hipStream_t passed as void*, NULL = default stream) only
- *     enqueue work.
+ *     enqueue work.  The library's scratch buffers are kept per (device, stream): calls on
+ *     different streams may overlap; calls that use the same plan handle share its
+ *     partial-sum buffer and must be ordered with each other.
  *   - results are deterministic: no floating-point atomics anywhere.
  */
 #ifndef BIDMAT_HIP_H

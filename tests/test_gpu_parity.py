@@ -536,6 +536,35 @@ def test_colslice_copy_and_zero_copy_column_ranges(hip):
     d.free()
 
 
+def test_two_streams_do_not_share_scratch(hip):
+    """Products with split columns enqueued back to back on two streams (each needs its own
+    overflow table and partial sums while the other is still running)."""
+    rng = np.random.default_rng(97)
+    k = 128
+    cases = []
+    for nrows, ncols in [(3000, 6000), (2500, 5000)]:
+        lengths = rng.integers(0, 30, size=ncols)
+        lengths[rng.integers(0, ncols, size=40)] = 5000          # many split columns
+        data, ir, jc = random_csc(rng, nrows, ncols, lengths=lengths, unique=False)
+        A = rng.standard_normal(k * nrows).astype(np.float32)
+        B = rng.standard_normal(k * ncols).astype(np.float32)
+        d = Dev(A=A, B=B, data=data, ir=ir, jc=jc)
+        d.zeros("AS", k * ncols), d.zeros("P", ir.size)
+        st = C.c_void_p()
+        hip_abi.check(hip.bidmat_stream_create(C.byref(st)))
+        cases.append((d, st, A, B, data, ir, jc, ncols))
+    for rep in range(3):
+        for d, st, A, B, data, ir, jc, ncols in cases:
+            hip_abi.check(hip.bidmat_dsmult_csc(k, ncols, ir.size, d.A.ptr, d.data.ptr, d.ir.ptr, d.jc.ptr, d.AS.ptr, 0, st))
+            hip_abi.check(hip.bidmat_dds_csc(k, ncols, ir.size, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.P.ptr, 0, st))
+    for d, st, A, B, data, ir, jc, ncols in cases:
+        hip_abi.check(hip.bidmat_stream_synchronize(st))
+        assert_close(d.AS.numpy(), *oracle.fsmult_f64(A, k, data, ir, jc), "A*S on its own stream")
+        assert_close(d.P.numpy(), *oracle.dds_f64(A, B, k, ir, jc), "DDS on its own stream")
+        hip_abi.check(hip.bidmat_stream_destroy(st))              # frees that stream's scratch as well
+        d.free()
+
+
 # ------------------------------------------------------------------------------ error behaviour
 def test_argument_validation(hip):
     d = Dev(x=np.ones(16, dtype=np.float32), i=np.zeros(16, dtype=np.int32))
