@@ -279,6 +279,24 @@ def main():
         out["rowsum"] = {"ms_avg": round(t, 4), "GBps": round(b / t / 1e6, 1),
                          "frac_of_hbm_peak": round(b / t / 1e6 / HBM_PEAK_GBS, 4)}
 
+    if args.workload in ("C1", "headline"):
+        # the same step recorded once into a HIP graph and replayed with one launch per step
+        gx = C.c_void_p()
+        hip_abi.check(lib.bidmat_graph_begin_capture(stream))
+        step()
+        hip_abi.check(lib.bidmat_graph_end_capture(stream, C.byref(gx)))
+        reps = 200 if args.workload == "C1" else args.steps
+        for _ in range(3):
+            hip_abi.check(lib.bidmat_graph_launch(gx, stream))
+        e0, e1 = ev(), ev()
+        hip_abi.check(lib.bidmat_event_record(e0, stream))
+        for _ in range(reps):
+            hip_abi.check(lib.bidmat_graph_launch(gx, stream))
+        hip_abi.check(lib.bidmat_event_record(e1, stream))
+        hip_abi.check(lib.bidmat_stream_synchronize(stream))
+        out["graph_replay"] = {"ms_per_step": round(elapsed(e0, e1) / reps, 4), "steps": reps}
+        hip_abi.check(lib.bidmat_graph_destroy(gx))
+
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_sample)
 

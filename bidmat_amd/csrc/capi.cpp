@@ -508,6 +508,32 @@ API int bidmat_stream_destroy(void* stream) {
     return (int)(e != hipSuccess ? e : (f != hipSuccess ? f : g));
 }
 API int bidmat_stream_synchronize(void* stream) { return (int)hipStreamSynchronize(as_stream(stream)); }
+// ---- HIP graphs: record a sequence of stream-taking calls once, replay it with one launch
+API int bidmat_graph_begin_capture(void* stream) {
+    if (!stream) return kInvalid;                  // the default stream cannot be captured
+    return (int)hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal);
+}
+API int bidmat_graph_end_capture(void* stream, void** graph_exec) {
+    if (!stream || !graph_exec) return kInvalid;
+    *graph_exec = nullptr;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(as_stream(stream), &g);
+    if (e != hipSuccess) return (int)e;
+    hipGraphExec_t x = nullptr;
+    e = hipGraphInstantiate(&x, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return (int)e;
+    *graph_exec = (void*)x;
+    return 0;
+}
+API int bidmat_graph_launch(void* graph_exec, void* stream) {
+    if (!graph_exec) return kInvalid;
+    return (int)hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream));
+}
+API int bidmat_graph_destroy(void* graph_exec) {
+    return graph_exec ? (int)hipGraphExecDestroy((hipGraphExec_t)graph_exec) : 0;
+}
+
 API int bidmat_event_create(void** event) {
     if (!event) return kInvalid;
     hipEvent_t ev;

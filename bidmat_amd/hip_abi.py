@@ -65,6 +65,10 @@ SIGNATURES = {
     "bidmat_stream_create": (C.c_int, [C.POINTER(vp)]),
     "bidmat_stream_destroy": (C.c_int, [vp]),
     "bidmat_stream_synchronize": (C.c_int, [vp]),
+    "bidmat_graph_begin_capture": (C.c_int, [vp]),
+    "bidmat_graph_end_capture": (C.c_int, [vp, C.POINTER(vp)]),
+    "bidmat_graph_launch": (C.c_int, [vp, vp]),
+    "bidmat_graph_destroy": (C.c_int, [vp]),
     "bidmat_event_create": (C.c_int, [C.POINTER(vp)]),
     "bidmat_event_destroy": (C.c_int, [vp]),
     "bidmat_event_record": (C.c_int, [vp, vp]),

@@ -215,6 +215,17 @@ int bidmat_memcpy_d2h_async(void *dst_pinned, const void *src, long long bytes, 
 /* Pinned host staging buffers (allocated, never registered). */
 int bidmat_host_alloc(void **hptr, long long bytes);
 int bidmat_host_free(void *hptr);
+/* HIP graphs (no counterpart in the reference, whose launchers block): record the stream-taking
+ * calls issued on `stream` between begin and end, then replay them with one launch per step.
+ * Only kernels are recorded (the library clears memory with fill kernels, never memset nodes).
+ * Nothing may allocate while recording: run the same calls once on the same stream beforehand,
+ * so that the stream's scratch buffers and any plan's partial-sum buffer have their size.  The
+ * recorded pointers and sizes are fixed; the data they point to may change between replays. */
+int bidmat_graph_begin_capture(void *stream);
+int bidmat_graph_end_capture(void *stream, void **graph_exec);
+int bidmat_graph_launch(void *graph_exec, void *stream);
+int bidmat_graph_destroy(void *graph_exec);
+
 /* Streams and events for callers that time or overlap work (benchmark harness). */
 int bidmat_stream_create(void **stream);
 int bidmat_stream_destroy(void *stream);

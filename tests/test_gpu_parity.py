@@ -565,6 +565,56 @@ def test_two_streams_do_not_share_scratch(hip):
         d.free()
 
 
+def test_graph_replay_of_the_three_products(hip):
+    """A*S, DDS and A*^S recorded into one HIP graph; every replay (with eager work and
+    synchronisations in between, and with new values in the same buffers) must give exactly what
+    the eager calls give."""
+    rng = np.random.default_rng(98)
+    k, nrows, ncols = 64, 400, 3000
+    lengths = rng.integers(0, 25, size=ncols)
+    lengths[11] = 2500                                           # overflow segments inside the graph
+    data, ir, jc = random_csc(rng, nrows, ncols, lengths=lengths, unique=False)
+    nnz = int(ir.size)
+    A = rng.standard_normal(k * nrows).astype(np.float32)
+    B = rng.standard_normal(k * ncols).astype(np.float32)
+    d = Dev(A=A, B=B, data=data, ir=ir, jc=jc)
+    for name, n in (("AS", k * ncols), ("P", nnz), ("G", k * nrows), ("AS2", k * ncols), ("P2", nnz), ("G2", k * nrows)):
+        d.zeros(name, n)
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    st = C.c_void_p()
+    hip_abi.check(hip.bidmat_stream_create(C.byref(st)))
+
+    def step(AS, P, G, stream):
+        hip_abi.check(hip.bidmat_dsmult_csc(k, ncols, nnz, d.A.ptr, d.data.ptr, d.ir.ptr, d.jc.ptr, AS.ptr, 0, stream))
+        hip_abi.check(hip.bidmat_dds_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, P.ptr, 0, stream))
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.B.ptr, d.data.ptr, G.ptr, 0, stream))
+
+    step(d.AS, d.P, d.G, st)                                      # warm-up: sizes the stream's scratch
+    hip_abi.check(hip.bidmat_stream_synchronize(st))
+    hip_abi.check(hip.bidmat_graph_begin_capture(st))
+    step(d.AS, d.P, d.G, st)
+    gx = C.c_void_p()
+    hip_abi.check(hip.bidmat_graph_end_capture(st, C.byref(gx)))
+    for rep in range(4):
+        if rep:                                                   # new values in the same buffers
+            newA = rng.standard_normal(k * nrows).astype(np.float32)
+            newv = (1.0 - rng.random(nnz)).astype(np.float32)
+            hip_abi.check(hip.bidmat_memcpy_h2d(d.A.ptr, newA.ctypes.data, newA.nbytes))
+            hip_abi.check(hip.bidmat_memcpy_h2d(d.data.ptr, newv.ctypes.data, newv.nbytes))
+        for buf in (d.AS, d.P, d.G):
+            hip_abi.check(hip.bidmat_memset(buf.ptr, 0xFF, buf.nbytes))
+        hip_abi.check(hip.bidmat_graph_launch(gx, st))
+        hip_abi.check(hip.bidmat_stream_synchronize(st))
+        step(d.AS2, d.P2, d.G2, None)                             # eager, default stream
+        hip_abi.check(hip.bidmat_synchronize())
+        for got, want, what in ((d.AS, d.AS2, "A*S"), (d.P, d.P2, "DDS"), (d.G, d.G2, "A*^S")):
+            assert np.array_equal(got.numpy().view(np.int32), want.numpy().view(np.int32)), "%s replay %d" % (what, rep)
+    hip_abi.check(hip.bidmat_graph_destroy(gx))
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    hip_abi.check(hip.bidmat_stream_destroy(st))
+    d.free()
+
+
 # ------------------------------------------------------------------------------ error behaviour
 def test_argument_validation(hip):
     d = Dev(x=np.ones(16, dtype=np.float32), i=np.zeros(16, dtype=np.int32))
