@@ -77,10 +77,29 @@ __global__ __launch_bounds__(BM_BLOCK) void k_apply_full4(const float4* __restri
 template <int OP, bool GATHER>
 __global__ __launch_bounds__(BM_BLOCK) void k_sdop(long long nnz, float* __restrict__ A, const int* __restrict__ idx,
                                                    const float* __restrict__ B) {
-    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    // tiles of 4 x 256 values per workgroup: four loads (and four dependent gathers) in flight
+    constexpr int UN = 4;
+    long long i = (long long)blockIdx.x * (UN * BM_BLOCK) + threadIdx.x;
+    const long long stride = (long long)gridDim.x * (UN * BM_BLOCK);
     const float bval = GATHER ? 0.f : B[0];
-    for (; i < nnz; i += stride) A[i] = binop<OP>(A[i], GATHER ? B[idx[i]] : bval);
+    for (; i < nnz; i += stride) {
+        float a[UN], b[UN];
+        int ix[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const long long j = i + u * BM_BLOCK;
+            const bool ok = j < nnz;
+            a[u] = ok ? A[j] : 0.f;
+            ix[u] = (GATHER && ok) ? idx[j] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) b[u] = GATHER ? B[ix[u]] : bval;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const long long j = i + u * BM_BLOCK;
+            if (j < nnz) A[j] = binop<OP>(a[u], b[u]);
+        }
+    }
 }
 
 // Dense transpose through a padded LDS tile: in is nrows x ncols (column-major, leading dimension
@@ -144,7 +163,7 @@ hipError_t apply_impl(const float* A, int ma, const float* B, int mb, float* C, 
 
 hipError_t sdop(long long nnz, float* A, const int* idx, const float* B, int len, int opn, hipStream_t s) {
     if (nnz <= 0) return hipSuccess;
-    dim3 grid(grid_for(nnz)), block(BM_BLOCK);
+    dim3 grid(grid_for((nnz + 3) / 4)), block(BM_BLOCK);
     switch (opn) {
 #define BM_OP(N_)                                                                                          \
     case N_:                                                                                               \
