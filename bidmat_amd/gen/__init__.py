@@ -92,7 +92,7 @@ def pattern(nrows, ncols, lengths, rows, seed):
     return ir, jc
 
 
-# The five configurations of BASELINE.json, parameterised by a scale in (0,1] that shrinks the
+# The five benchmark configurations, parameterised by a scale in (0,1] that shrinks the
 # number of columns (and for the big ones the number of rows) but keeps k and the per-column
 # statistics. scale=1 is the full configuration.
 def config(name, scale=1.0):

@@ -1,4 +1,4 @@
-"""Parity at the full sizes of BASELINE.json's configurations, where the oracle cannot run the
+"""Parity at the full sizes of the benchmark configurations, where the oracle cannot run the
 whole problem in seconds: size-independent properties (the Frobenius identity that ties the
 three products together, linearity, sum-of-sums) plus oracle checks on random samples of
 columns / rows / nonzeros of the full-size result.

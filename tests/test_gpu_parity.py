@@ -120,7 +120,7 @@ def test_dsmult_long_columns_split_path(hip, k):
 
 
 def test_dsmult_config1(hip):
-    """BASELINE configs[0]: A 32x4096 N(0,1), S 4096x8192 with exactly 50 nnz per column."""
+    """Benchmark configuration 1: A 32x4096 N(0,1), S 4096x8192 with exactly 50 nnz per column."""
     from bidmat_amd import gen
     c = gen.config("C1")
     k, ncols = c["k"], c["ncols"]

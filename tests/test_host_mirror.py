@@ -211,7 +211,7 @@ def test_index_base_zero_host_matrices(hip):
 
 @gpu
 def test_nmf_multiplicative_update_chain(hip):
-    """The chain of BASELINE configs[4] at a small size: R = DDS(W,H,V); Q = V ./ R on the
+    """The NMF update chain (benchmark configuration 5) at a small size: R = DDS(W,H,V); Q = V ./ R on the
     nonzeros; G = W *^ Q; rs = sum(H, 2)."""
     rng = np.random.default_rng(11)
     k, m, n = 16, 40, 60
