@@ -400,6 +400,20 @@ API int bidmat_csc_colslice(int col1, int col2, int start, int nnz, const int* S
                                  as_stream(stream));
 }
 
+API int bidmat_csc_transpose(int nrows, int ncols, int nnz, const float* Sdata, const int* Sir, const int* Sjc,
+                             float* out_data, int* out_ir, int* out_jc) {
+    if (nrows < 0 || ncols < 0 || nnz < 0 || !out_jc) return kInvalid;
+    if (nnz > 0 && (!Sdata || !Sir || !Sjc || !out_data || !out_ir)) return kInvalid;
+    return finish_blocking(bm::csc_transpose(nrows, ncols, nnz, Sdata, Sir, Sjc, out_data, out_ir, out_jc, nullptr));
+}
+
+API int bidmat_full(const int* ir, const int* ic, const float* data, float* od, int nrows, int ncols, int nnz) {
+    if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!ir || !ic || !data || !od) return kInvalid;
+    return finish_blocking(bm::full_from_coo(nrows, ncols, nnz, ir, ic, data, od, nrows, nullptr));
+}
+
 API int bidmat_nhot(int n, int ncols, const int* cats, int* out_ir, int* out_ic, int* out_jc, float* out_data,
                     int* maxcat) {
     if (n < 0 || ncols < 0 || (long long)n * ncols > 0x7fffffffLL || !out_jc) return kInvalid;

@@ -137,6 +137,19 @@ __global__ __launch_bounds__(BM_BLOCK) void k_nhot(int n, int ncols, const int* 
     if ((threadIdx.x & 63) == 0 && m >= 0) atomicMax(maxcat, m);
 }
 
+// Dense image of a sparse matrix: od[row + col*ld] = value for every stored nonzero (the output is
+// cleared by the caller; where a column stores a row twice, one of the values stays).
+__global__ __launch_bounds__(BM_BLOCK) void k_full(long long nnz, const int* __restrict__ ir, const int* __restrict__ ic,
+                                                   const float* __restrict__ data, float* __restrict__ od,
+                                                   int nrows, int ncols, long long ld) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    for (; i < nnz; i += stride) {
+        const int r = ir[i], c = ic[i];
+        if ((unsigned)r < (unsigned)nrows && (unsigned)c < (unsigned)ncols) od[r + c * ld] = data[i];
+    }
+}
+
 inline unsigned grid_for(long long n, int maxblocks = 8192) {
     long long b = (n + BM_BLOCK - 1) / BM_BLOCK;
     if (b < 1) b = 1;
@@ -191,6 +204,14 @@ hipError_t nhot(int n, int ncols, const int* cats, int* ir, int* ic, int* jc, fl
     const long long total = (long long)n * ncols;
     const long long lim = total > (long long)ncols + 1 ? total : (long long)ncols + 1;
     hipLaunchKernelGGL(k_nhot, dim3(grid_for(lim)), dim3(BM_BLOCK), 0, s, n, ncols, cats, ir, ic, jc, data, d_maxcat);
+    return hipGetLastError();
+}
+
+hipError_t full_from_coo(int nrows, int ncols, int nnz, const int* ir, const int* ic, const float* data, float* od,
+                         int ld, hipStream_t s) {
+    if (nnz <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_full, dim3(grid_for(nnz, 16384)), dim3(BM_BLOCK), 0, s, (long long)nnz, ir, ic, data, od,
+                       nrows, ncols, (long long)ld);
     return hipGetLastError();
 }
 

@@ -126,6 +126,13 @@ JFN(jint, cscColslice)(JNIEnv*, jclass, jint col1, jint col2, jint start, jint n
                                 P(int, ojc), P(int, oir), P(int, oic), P(float, odata), nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
+// GSMat.t without the host round trip, and the launcher behind GSMat.full (CUMAT.full)
+JFN(jint, cscTranspose)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong Sdata, jlong Sir, jlong Sjc, jlong odata, jlong oir, jlong ojc) {
+    return bidmat_csc_transpose(nr, nc, nnz, P(const float, Sdata), P(const int, Sir), P(const int, Sjc), P(float, odata), P(int, oir), P(int, ojc));
+}
+JFN(jint, full)(JNIEnv*, jclass, jlong ir, jlong ic, jlong data, jlong od, jint nr, jint nc, jint nnz) {
+    return bidmat_full(P(const int, ir), P(const int, ic), P(const float, data), P(float, od), nr, nc, nnz);
+}
 JFN(jint, cscExpandCols)(JNIEnv*, jclass, jint nc, jint nnz, jlong Sjc, jlong Sic) {
     int e = bidmat_csc_expand_cols(nc, nnz, P(const int, Sjc), P(int, Sic), nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);

@@ -20,6 +20,13 @@ hipError_t csc_colslice(int nc, int start, int n, const int* jc_at_col1, const i
 // n-hot pattern from an n x ncols category matrix; *d_maxcat (device int) receives the largest category
 hipError_t nhot(int n, int ncols, const int* cats, int* ir, int* ic, int* jc, float* data, int* d_maxcat,
                 hipStream_t s);
+// transpose of a CSC matrix (csc_transpose.hip): out_jc has nrows+1 entries, out_ir holds the
+// original columns in ascending order inside every output column. Blocks until done.
+hipError_t csc_transpose(int nrows, int ncols, int nnz, const float* data, const int* ir, const int* jc,
+                         float* out_data, int* out_ir, int* out_jc, hipStream_t s);
+// od[ir[j] + ic[j]*ld] = data[j] for every nonzero (od cleared by the caller)
+hipError_t full_from_coo(int nrows, int ncols, int nnz, const int* ir, const int* ic, const float* data, float* od,
+                         int ld, hipStream_t s);
 // out[i] = v for i < n (a kernel, so that callers may record it into a HIP graph)
 hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
 hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);

@@ -17,6 +17,7 @@ enum WsSlot {
     WS_TRANS_IN,      // float[...]    transposed dense operand of S*A / S^T*A
     WS_TRANS_OUT,     // float[...]    transposed result of S*A / S^T*A
     WS_PLAN,          // bytes         temporaries of a plan build (dropped again when large)
+    WS_TRANSPOSE,     // bytes         sort buffers of the sparse transpose
     WS_NSLOTS
 };
 

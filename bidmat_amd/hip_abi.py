@@ -40,6 +40,8 @@ SIGNATURES = {
     "bidmat_csc_expand_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
     "bidmat_csc_colslice_range": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "bidmat_csc_colslice": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, vp, vp, vp]),
+    "bidmat_csc_transpose": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, vp]),
+    "bidmat_full": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]),
     "bidmat_nhot": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp, vp, C.POINTER(C.c_int)]),
     "bidmat_coo_compress_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
     "bidmat_sdtmult_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int, vp, C.c_int, vp]),

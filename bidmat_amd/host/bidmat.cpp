@@ -449,6 +449,25 @@ GSMatP GSMat::nHot(const std::vector<int>& cats, int n, int ncols, int ncats0) {
     return out;
 }
 
+GSMatP GSMat::t(GSMatP omat) {
+    GSMatP out = newOrCheckGSMat(ncols, nrows, nnz0, realnnz, omat, GUID, 0, 0, opHash("t"));
+    out->nnz0 = nnz0;
+    out->planHolder = std::make_shared<PlanHolder>();
+    int err = bidmat_csc_transpose(nrows, ncols, nnz0, pdata, pir, pjc, out->pdata, out->pir, out->pjc);
+    if (err == 0) err = bidmat_csc_expand_cols(out->ncols, nnz0, out->pjc, out->pic, nullptr);
+    if (err == 0) err = bidmat_stream_synchronize(nullptr);
+    if (err != 0) fail(std::string("HIP error in GSMat.t ") + bidmat_error_string(err));
+    return out;
+}
+
+GMatP GSMat::full(GMatP omat) {
+    GMatP out = GMat::newOrCheckGMat(nrows, ncols, omat, GUID, 0, opHash("full"));
+    out->clear();
+    int err = bidmat_full(pir, pic, pdata, out->pdata, nrows, ncols, nnz0);
+    if (err != 0) fail(std::string("HIP full kernel error ") + bidmat_error_string(err));
+    return out;
+}
+
 GSMatP GSMat::colslice(int col1, int col2, GSMatP omat) {
     if (col1 < 0 || col2 < col1 || col2 > ncols) fail("GSMat.colslice: column range outside the matrix");
     int starti = 0, newnnz = 0;

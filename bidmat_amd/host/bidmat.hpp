@@ -147,6 +147,8 @@ public:
     GMatP sum(int n, GMatP oldmat);                              // GSMat.scala:250-261
     GSMatP GSDop(const GMatP& b, GSMatP omat, int op);           // this op edge vector (GSMat.scala:315-330)
     GSMatP copy(GSMatP omat, long long key1, long long key2);    // GSMat.copy / copyTo
+    GSMatP t(GSMatP omat = nullptr);                             // transpose, on the device (GSMat.scala:218-223)
+    GMatP full(GMatP omat = nullptr);                            // dense image (GSMat.scala:206-216)
     GSMatP colslice(int col1, int col2, GSMatP omat = nullptr);  // columns [col1, col2)  (GSMat.scala:77-104)
     GMatP SDMult(const GMatP& a, GMatP omat);                    // this * a    (GSMat.scala:265-289)
     GMatP SDTMult(const GMatP& a, GMatP omat);                   // this ^* a   (GSMat.scala:291-313)

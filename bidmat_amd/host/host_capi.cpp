@@ -100,6 +100,8 @@ API void* bmh_nhot(const int* cats, int n, int ncols, int ncats) {
         return wrap(GSMat::nHot(c, n, ncols, ncats));
     });
 }
+API void* bmh_t(void* s, void* out) { return guard_ptr([&] { return wrap(S(s)->t(S(out))); }); }
+API void* bmh_full(void* s, void* out) { return guard_ptr([&] { return wrap(S(s)->full(G(out))); }); }
 API void* bmh_colslice(void* s, int col1, int col2, void* out) {
     return guard_ptr([&] { return wrap(S(s)->colslice(col1, col2, S(out))); });
 }

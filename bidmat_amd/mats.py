@@ -31,7 +31,7 @@ def _load():
         L = C.CDLL(LIB_PATH)
         for name in ("bmh_gmat_from_host", "bmh_gmat_zeros", "bmh_gsmat_from_host", "bmh_mult", "bmh_madd",
                      "bmh_multT", "bmh_maddT", "bmh_dds", "bmh_sum_sparse", "bmh_sum_dense", "bmh_reduce",
-                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop", "bmh_load_gsmat", "bmh_colslice", "bmh_nhot"):
+                     "bmh_gop", "bmh_contents", "bmh_with_values", "bmh_tile_mult", "bmh_sdmult", "bmh_gsdop", "bmh_load_gsmat", "bmh_colslice", "bmh_nhot", "bmh_full", "bmh_t"):
             getattr(L, name).restype = vp
         L.bmh_gmat_from_host.argtypes = [C.c_int, C.c_int, vp]
         L.bmh_gmat_zeros.argtypes = [C.c_int, C.c_int]
@@ -43,6 +43,8 @@ def _load():
         L.bmh_gsdop.argtypes = [vp, vp, vp, C.c_int]
         L.bmh_colslice.argtypes = [vp, C.c_int, C.c_int, vp]
         L.bmh_nhot.argtypes = [vp, C.c_int, C.c_int, C.c_int]
+        L.bmh_full.argtypes = [vp, vp]
+        L.bmh_t.argtypes = [vp, vp]
         L.bmh_load_gsmat.argtypes = [C.c_char_p]
         ip = C.POINTER(C.c_int)
         L.bmh_save_smat.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, vp, vp, vp]
@@ -246,6 +248,12 @@ class GSMat(_Handle):
 
     def contents(self):
         return GMat(_load().bmh_contents(self._h))
+
+    def t(self, out=None):                        # transpose, computed on the device
+        return GSMat(_load().bmh_t(self._h, out._h if out else None))
+
+    def full(self, out=None):                     # dense image as a GMat
+        return GMat(_load().bmh_full(self._h, out._h if out else None))
 
     def colslice(self, col1, col2, out=None):     # columns [col1, col2)
         return GSMat(_load().bmh_colslice(self._h, col1, col2, out._h if out else None))

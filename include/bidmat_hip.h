@@ -151,6 +151,19 @@ int bidmat_spsum_rows_plan(bidmat_plan *plan, const float *Sdata, float *out, in
 /* jc[ncols+1] -> ic[nnz] (per-nonzero column index).  Replaces cusparseXcsr2coo at
  * GSMat.scala:639.  Enqueues on stream. */
 int bidmat_csc_expand_cols(int ncols, int nnz, const int *Sjc, int *Sic, void *stream);
+/* Transpose of a device CSC matrix (nrows x ncols, nnz nonzeros) without leaving the device:
+ * out_jc (nrows+1), out_ir (nnz: the original columns, ascending inside every output column),
+ * out_data (nnz).  The reference's GSMat.t downloads, transposes on the host and uploads
+ * (GSMat.scala:218-223).  Row indices outside the matrix are rejected.  Blocking. */
+int bidmat_csc_transpose(int nrows, int ncols, int nnz, const float *Sdata, const int *Sir,
+                         const int *Sjc, float *out_data, int *out_ir, int *out_jc);
+
+/* Dense image of a sparse matrix, od[ir[j] + ic[j]*nrows] = data[j]; the caller clears od first
+ * (GSMat.full, GSMat.scala:206-214).  Replaces full (CopyFill.cu:1456-1475,
+ * CUMAT.java full).  Where a column stores one row twice, one of the values stays, as in the
+ * reference.  Indices outside the matrix are skipped.  Blocking. */
+int bidmat_full(const int *ir, const int *ic, const float *data, float *od, int nrows, int ncols, int nnz);
+
 /* One-hot / n-hot pattern (GSMat.oneHot / GSMat.nHot, GSMat.scala:686-720): cats is an
  * n x ncols device int matrix of categories; column j of the result holds rows cats[:, j] in
  * the given order (not sorted, repeats allowed) with value 1.  Outputs: out_ir, out_ic,

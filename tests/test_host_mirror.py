@@ -394,3 +394,26 @@ def test_onehot_and_nhot(hip):
         np.add.at(wantT.T, cats[i], b.astype(np.float64).T)
     np.testing.assert_allclose(GMat.from_numpy(b).xT(s3).numpy(), wantT, rtol=0, atol=EPS)
     np.testing.assert_allclose(s3.sum(2).numpy().ravel(), np.bincount(cats.ravel(), minlength=ncats), rtol=0, atol=EPS)
+
+
+@gpu
+def test_matrix_transpose_and_full(hip):
+    """'A GSMat should support matrix transpose' (GSMatTest.scala:46-53), computed on the device
+    here; full() is the dense image (GSMat.scala:206-216)."""
+    rng = np.random.default_rng(14)
+    for m, n, dens in [(nr, nc, 0.2), (200, 3000, 0.05), (1, 50, 0.5), (50, 1, 0.5), (30, 40, 0.0)]:
+        a = sprand(rng, m, n, dens)
+        aa = GSMat.from_csc(m, n, *a)
+        dense = full(m, n, *a)
+        ff = aa.full()
+        assert ff.mytype == "GMat" and ff.shape == (m, n)
+        assert np.array_equal(ff.numpy(), dense.astype(np.float32))
+        bb = aa.t()
+        assert bb.mytype == "GSMat" and bb.dims == (n, m, a[0].size)
+        d2, ir2, jc2 = bb.to_csc()                                # SparseMat.check passes: rows sorted
+        assert np.array_equal(full(n, m, d2, ir2, jc2), dense.T)
+        assert np.array_equal(bb.full().numpy(), dense.T.astype(np.float32))
+        if a[0].size:
+            x = rng.random((7, n)).astype(np.float32)             # x * a^T through the transposed matrix
+            np.testing.assert_allclose((GMat.from_numpy(x) * bb).numpy(), x.astype(np.float64) @ dense.T, rtol=0, atol=EPS)
+            assert np.array_equal(bb.t().to_csc()[1], a[1])       # transpose twice: the pattern is back
