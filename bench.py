@@ -397,6 +397,20 @@ def next_rows(lib, args):
     out["sdoprow"] = {"ms": round(t, 3), "GBps": round(12.0 * nnz / t / 1e6, 1)}
     t = _timed(lib, lambda: lib.bidmat_sdopcol(nrows, ncols, nnz, d_w.ptr, d_ir.ptr, d_col.ptr, nrows, 2), stream, reps, 1)
     out["sdopcol"] = {"ms": round(t, 3), "GBps": round(12.0 * nnz / t / 1e6, 1)}
+    # pattern utilities: transpose on the device, a column range as a matrix of its own, dense image skipped (too large)
+    d_tv, d_tir, d_tjc = DeviceArray(nnz, np.float32), DeviceArray(nnz, np.int32), DeviceArray(nrows + 1, np.int32)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        hip_abi.check(lib.bidmat_csc_transpose(nrows, ncols, nnz, d_v.ptr, d_ir.ptr, d_jc.ptr, d_tv.ptr, d_tir.ptr, d_tjc.ptr))
+    t = (time.perf_counter() - t0) / 3 * 1e3
+    out["GSMat.t (device)"] = {"ms": round(t, 3), "Mnnz_per_s": round(nnz / t / 1e3, 1)}
+    c1, c2 = ncols // 4, ncols // 2
+    start, cnt = C.c_int(), C.c_int()
+    hip_abi.check(lib.bidmat_csc_colslice_range(ncols, c1, c2, d_jc.ptr, C.byref(start), C.byref(cnt)))
+    d_sjc, d_sic = DeviceArray(c2 - c1 + 1, np.int32), DeviceArray(cnt.value, np.int32)
+    t = _timed(lib, lambda: lib.bidmat_csc_colslice(c1, c2, start.value, cnt.value, d_jc.ptr, d_ir.ptr, d_v.ptr, d_sjc.ptr,
+                                                    d_tir.ptr, d_sic.ptr, d_tv.ptr, stream), stream, reps, 1)
+    out["colslice (quarter of the columns)"] = {"ms": round(t, 3), "GBps": round(20.0 * cnt.value / t / 1e6, 1)}
     # file -> device (pinned, double-buffered) against host arrays -> device (pageable copies)
     with tempfile.TemporaryDirectory() as tmp:
         f = os.path.join(tmp, "pattern.smat")
