@@ -364,10 +364,12 @@ def test_spsum_large_with_plan(hip):
 @pytest.mark.parametrize("opn,initv", [(0, 0.0), (2, 1.0), (10, -3.4e38), (11, 3.4e38)])
 def test_dense_reduce(hip, shape, opn, initv):
     nrows, ncols = shape
-    if opn == 2 and nrows * ncols > 1000:
-        pytest.skip("products of long vectors leave the float range")
     rng = np.random.default_rng(60 + nrows + ncols)
-    A = (rng.random(nrows * ncols).astype(np.float32) + 0.5) if opn == 2 else rng.standard_normal(nrows * ncols).astype(np.float32)
+    if opn == 2:
+        # factors exp(N(0,1)/sqrt(n)): products of n of them stay near 1 whatever the length
+        A = np.exp(rng.standard_normal(nrows * ncols) / np.sqrt(max(nrows, ncols))).astype(np.float32)
+    else:
+        A = rng.standard_normal(nrows * ncols).astype(np.float32)
     d = Dev(A=A)
     d.zeros("c", ncols), d.zeros("r", nrows)
     hip_abi.check(hip.bidmat_reduce1op(nrows, ncols, d.A.ptr, d.c.ptr, initv, opn))
