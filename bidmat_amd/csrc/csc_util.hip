@@ -82,7 +82,14 @@ __global__ __launch_bounds__(BM_BLOCK) void k_pattern_digest(const int* __restri
         hb += __shfl_xor(hb, d, 64);
         m = max(m, __shfl_xor(m, d, 64));
     }
-    if ((threadIdx.x & 63) == 0) {
+    // one set of atomics per workgroup: thousands of them on three addresses would serialise
+    __shared__ unsigned long long sa[BM_WAVES_PER_BLOCK], sb[BM_WAVES_PER_BLOCK];
+    __shared__ int sm[BM_WAVES_PER_BLOCK];
+    if ((threadIdx.x & 63) == 0) { sa[threadIdx.x >> 6] = ha; sb[threadIdx.x >> 6] = hb; sm[threadIdx.x >> 6] = m; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < BM_WAVES_PER_BLOCK; ++w) { ha += sa[w]; hb += sb[w]; m = max(m, sm[w]); }
         atomicAdd(out, ha);
         atomicAdd(out + 1, hb);
         if (m >= 0) atomicMax(reinterpret_cast<int*>(out + 2), m);
