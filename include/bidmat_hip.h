@@ -233,7 +233,10 @@ int bidmat_host_free(void *hptr);
  * Only kernels are recorded (the library clears memory with fill kernels, never memset nodes).
  * Nothing may allocate while recording: run the same calls once on the same stream beforehand,
  * so that the stream's scratch buffers and any plan's partial-sum buffer have their size.  The
- * recorded pointers and sizes are fixed; the data they point to may change between replays. */
+ * recorded pointers and sizes are fixed; the data they point to may change between replays.
+ * A recording also holds the addresses of the stream's scratch buffers and of any plan it used:
+ * destroy it (and record again) before a larger problem is run on that stream (scratch grows by
+ * reallocation), before the plan is destroyed and before bidmat_release_caches. */
 int bidmat_graph_begin_capture(void *stream);
 int bidmat_graph_end_capture(void *stream, void **graph_exec);
 int bidmat_graph_launch(void *graph_exec, void *stream);
