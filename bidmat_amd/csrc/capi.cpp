@@ -428,6 +428,11 @@ API int bidmat_nhot(int n, int ncols, const int* cats, int* out_ir, int* out_ic,
     return finish_blocking(err);
 }
 
+API int bidmat_index_shift(int* p, long long n, int delta, void* stream) {
+    if (n < 0 || (n > 0 && !p)) return kInvalid;
+    return (int)bm::index_shift(p, n, delta, as_stream(stream));
+}
+
 API int bidmat_coo_compress_cols(int ncols, int nnz, const int* Sic, int* Sjc, void* stream) {
     if (ncols < 0 || nnz < 0) return kInvalid;
     if (!Sjc || (nnz > 0 && !Sic)) return kInvalid;

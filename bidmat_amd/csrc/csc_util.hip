@@ -157,6 +157,13 @@ __global__ __launch_bounds__(BM_BLOCK) void k_full(long long nnz, const int* __r
     }
 }
 
+// p[i] += delta (index-base conversion of uploaded / downloaded index arrays)
+__global__ __launch_bounds__(BM_BLOCK) void k_index_shift(int* __restrict__ p, long long n, int delta) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    for (; i < n; i += stride) p[i] += delta;
+}
+
 inline unsigned grid_for(long long n, int maxblocks = 8192) {
     long long b = (n + BM_BLOCK - 1) / BM_BLOCK;
     if (b < 1) b = 1;
@@ -219,6 +226,12 @@ hipError_t full_from_coo(int nrows, int ncols, int nnz, const int* ir, const int
     if (nnz <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_full, dim3(grid_for(nnz, 16384)), dim3(BM_BLOCK), 0, s, (long long)nnz, ir, ic, data, od,
                        nrows, ncols, (long long)ld);
+    return hipGetLastError();
+}
+
+hipError_t index_shift(int* p, long long n, int delta, hipStream_t s) {
+    if (n <= 0 || delta == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_index_shift, dim3(grid_for(n, 16384)), dim3(BM_BLOCK), 0, s, p, n, delta);
     return hipGetLastError();
 }
 

@@ -27,6 +27,8 @@ hipError_t csc_transpose(int nrows, int ncols, int nnz, const float* data, const
 // od[ir[j] + ic[j]*ld] = data[j] for every nonzero (od cleared by the caller)
 hipError_t full_from_coo(int nrows, int ncols, int nnz, const int* ir, const int* ic, const float* data, float* od,
                          int ld, hipStream_t s);
+// p[i] += delta
+hipError_t index_shift(int* p, long long n, int delta, hipStream_t s);
 // out[i] = v for i < n (a kernel, so that callers may record it into a HIP graph)
 hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
 hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);

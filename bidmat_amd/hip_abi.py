@@ -43,6 +43,7 @@ SIGNATURES = {
     "bidmat_csc_transpose": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, vp]),
     "bidmat_full": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]),
     "bidmat_nhot": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp, vp, C.POINTER(C.c_int)]),
+    "bidmat_index_shift": (C.c_int, [vp, C.c_longlong, C.c_int, vp]),
     "bidmat_coo_compress_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
     "bidmat_sdtmult_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int, vp, C.c_int, vp]),
     "bidmat_sdmult_plan": (C.c_int, [vp, C.c_int, vp, vp, C.c_int, vp, C.c_int, vp]),

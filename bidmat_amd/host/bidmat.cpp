@@ -353,15 +353,11 @@ GSMatP GSMat::fromSMat(const SMat& a, GSMatP b) {
     out->planHolder = std::make_shared<PlanHolder>();      // new pattern: any older plan is stale
     const int n = a.nnz();
     hipcheck(bidmat_memcpy_h2d(out->pdata, a.data.data(), (long long)sizeof(float) * n), "copy error in GSMat.fromSMat");
-    if (Mat::ioneBased == 1) {   // device indices are always 0-based (GSMat.scala:626-632)
-        std::vector<int> ir0(a.ir), jc0(a.jc);
-        for (auto& v : ir0) v -= 1;
-        for (auto& v : jc0) v -= 1;
-        hipcheck(bidmat_memcpy_h2d(out->pir, ir0.data(), (long long)sizeof(int) * n), "copy error in GSMat.fromSMat");
-        hipcheck(bidmat_memcpy_h2d(out->pjc, jc0.data(), (long long)sizeof(int) * (a.ncols + 1)), "copy error in GSMat.fromSMat");
-    } else {
-        hipcheck(bidmat_memcpy_h2d(out->pir, a.ir.data(), (long long)sizeof(int) * n), "copy error in GSMat.fromSMat");
-        hipcheck(bidmat_memcpy_h2d(out->pjc, a.jc.data(), (long long)sizeof(int) * (a.ncols + 1)), "copy error in GSMat.fromSMat");
+    hipcheck(bidmat_memcpy_h2d(out->pir, a.ir.data(), (long long)sizeof(int) * n), "copy error in GSMat.fromSMat");
+    hipcheck(bidmat_memcpy_h2d(out->pjc, a.jc.data(), (long long)sizeof(int) * (a.ncols + 1)), "copy error in GSMat.fromSMat");
+    if (Mat::ioneBased == 1) {   // device indices are always 0-based (GSMat.scala:626-632); shifted on the device
+        hipcheck(bidmat_index_shift(out->pir, n, -1, nullptr), "GSMat.fromSMat");
+        hipcheck(bidmat_index_shift(out->pjc, (long long)a.ncols + 1, -1, nullptr), "GSMat.fromSMat");
     }
     // per-nonzero column indices (the reference calls cusparseXcsr2coo here, GSMat.scala:639)
     int err = bidmat_csc_expand_cols(out->ncols, n, out->pjc, out->pic, nullptr);

@@ -185,6 +185,11 @@ int bidmat_csc_colslice(int col1, int col2, int start, int nnz, const int *Sjc, 
                         const float *Sdata, int *out_jc, int *out_ir, int *out_ic, float *out_data,
                         void *stream);
 
+/* p[i] += delta on a device int array: the index-base conversion of GSMat.fromSMat / toSMat
+ * (host SMat indices are 1-based by default, GSMat.scala:123-125,626-632) done on the device
+ * instead of in a host loop.  Enqueues on stream. */
+int bidmat_index_shift(int *p, long long n, int delta, void *stream);
+
 /* non-decreasing ic[nnz] -> jc[ncols+1].  Replaces cusparseXcoo2csr at GSMat.scala:698,716
  * and SparseMat.compressInds (SparseMat.scala:857-868). Enqueues on stream. */
 int bidmat_coo_compress_cols(int ncols, int nnz, const int *Sic, int *Sjc, void *stream);
