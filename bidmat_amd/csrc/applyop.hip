@@ -2,29 +2,11 @@
 // per element; the equal-shape case uses 128-bit accesses.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "ops.hpp"
 #include <math.h>
 
 namespace bm {
 namespace {
-
-template <int OP>
-__device__ __forceinline__ float binop(float a, float b) {
-    if constexpr (OP == 0) return a + b;
-    else if constexpr (OP == 1) return a - b;
-    else if constexpr (OP == 2) return a * b;
-    else if constexpr (OP == 3) return a / b;
-    else if constexpr (OP == 4) return (a > b) ? 1.0f : 0.0f;
-    else if constexpr (OP == 5) return (a < b) ? 1.0f : 0.0f;
-    else if constexpr (OP == 6) return (a == b) ? 1.0f : 0.0f;
-    else if constexpr (OP == 7) return (a >= b) ? 1.0f : 0.0f;
-    else if constexpr (OP == 8) return (a <= b) ? 1.0f : 0.0f;
-    else if constexpr (OP == 9) return (a != b) ? 1.0f : 0.0f;
-    else if constexpr (OP == 10) return fmaxf(a, b);
-    else if constexpr (OP == 11) return fminf(a, b);
-    else if constexpr (OP == 12) return atan2f(a, b);
-    else if constexpr (OP == 13) return powf(a, b);
-    else return (a > 0) ? b : 0.0f;
-}
 
 // Index modes: how element i (column-major, nrows x ncols) picks its operand.
 enum Mode { FULL = 0, COL = 1, ROW = 2, VAL = 3 };

@@ -47,6 +47,7 @@ inline int finish_blocking(hipError_t launch_err) {
 struct CacheEntry {
     int device;
     int ncols, nnz, nrows, k_hint;
+    const int *ir, *ic;                     // where the pattern lay when the plan was built
     unsigned long long fa, fb;
     std::shared_ptr<bidmat_plan> plan;      // callers hold a reference while they use the plan
 };
@@ -77,7 +78,7 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
         // panels are sized for k_hint: a request that names k only takes a plan built for that k
         const bool k_ok = k_hint <= 0 || (it->k_hint > 0 ? it->k_hint : 256) == k_hint;
         if (k_ok && it->device == dev && it->ncols == ncols && it->nnz == nnz && it->nrows == nrows &&
-            it->fa == h[0] && it->fb == h[1]) {
+            it->ir == ir && it->ic == ic && it->fa == h[0] && it->fb == h[1]) {
             g_cache.splice(g_cache.begin(), g_cache, it);
             *out = g_cache.front().plan;
             return hipSuccess;
@@ -89,24 +90,28 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     bidmat_plan* p = nullptr;
     if ((err = bm::plan_build(nrows, ncols, nnz, ir, jc, k_hint, &p)) != hipSuccess) return err;
     while (g_cache.size() >= kMaxCachedPlans) g_cache.pop_back();   // freed when its last user lets go
-    g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, h[0], h[1], own(p)});
+    g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, ir, ic, h[0], h[1], own(p)});
     *out = g_cache.front().plan;
     return hipSuccess;
 }
 
+// vals == nullptr: the values stored in the plan by bidmat_plan_set_values (already in plan order)
 hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* vals, float* C, int beta,
                        hipStream_t s) {
     hipError_t err;
+    if (!vals && !plan->pvals && plan->nnz > 0) return hipErrorInvalidValue;
     if ((err = bm::plan_reserve_partial(plan, k)) != hipSuccess) return err;
-    if ((err = bm::gather_segments(k, plan->nseg, plan->xcd_start, A, vals, plan->pc, plan->perm, plan->segstart,
-                                   plan->partial, s)) != hipSuccess) return err;
+    if ((err = bm::gather_segments(k, plan->nseg, plan->xcd_start, A, vals ? vals : plan->pvals, plan->pc,
+                                   vals ? plan->perm : nullptr, plan->segstart, plan->partial, s)) != hipSuccess) return err;
     return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, C, beta, s);
 }
 
 hipError_t run_spsum_rows(bidmat_plan* plan, const float* vals, float* out, int beta, hipStream_t s) {
     hipError_t err;
+    if (!vals && !plan->pvals && plan->nnz > 0) return hipErrorInvalidValue;
     if ((err = bm::plan_reserve_partial(plan, 1)) != hipSuccess) return err;
-    if ((err = bm::spsum_segments(plan->nseg, plan->xcd_start, vals, plan->perm, plan->segstart, plan->partial, s)) != hipSuccess)
+    if ((err = bm::spsum_segments(plan->nseg, plan->xcd_start, vals ? vals : plan->pvals, vals ? plan->perm : nullptr,
+                                  plan->segstart, plan->partial, s)) != hipSuccess)
         return err;
     return bm::reduce_segments(1, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, out, beta, s);
 }
@@ -122,6 +127,7 @@ bool plan_on_current_device(const bidmat_plan* p) {
 
 API int bidmat_dsmult(int nrows, int ncols, int nnz, const float* A, const float* Bdata,
                       const int* Bir, const int* Bic, float* C) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
     if (nrows == 0 || ncols == 0 || nnz == 0) return 0;           // C += 0
     if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
@@ -135,6 +141,7 @@ API int bidmat_dsmult(int nrows, int ncols, int nnz, const float* A, const float
 
 API int bidmat_dsmultT(int nrows, int ncols, int nnz, const float* A, const float* Bdata,
                        const int* Bir, const int* Bic, float* C) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
     if (nrows == 0 || ncols == 0 || nnz == 0) return 0;
     if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
@@ -146,6 +153,7 @@ API int bidmat_dsmultT(int nrows, int ncols, int nnz, const float* A, const floa
 
 API int bidmat_dsmultTile(int nr, int nc, int kk, int nnz, const float* A, int lda, const float* Bdata,
                           const int* Bir, const int* Bic, int broff, int bcoff, float* C, int ldc) {
+    auto lock = bm::device_lock();
     if (nr < 0 || nc < 0 || kk < 0 || nnz < 0 || broff < 0 || bcoff < 0 || lda < nr || ldc < nr) return kInvalid;
     if (nr == 0 || nc == 0 || kk == 0 || nnz == 0) return 0;
     if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
@@ -167,6 +175,7 @@ API int bidmat_dsmultTile(int nr, int nc, int kk, int nnz, const float* A, int l
 
 API int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float* A, int lda, const float* Bdata,
                            const int* Bir, const int* Bic, int broff, int bcoff, float* C, int ldc) {
+    auto lock = bm::device_lock();
     if (nr < 0 || nc < 0 || kk < 0 || nnz < 0 || broff < 0 || bcoff < 0 || lda < nr || ldc < nr) return kInvalid;
     if (nr == 0 || nc == 0 || kk == 0 || nnz == 0) return 0;
     if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
@@ -207,6 +216,7 @@ API int bidmat_sdopcol(int nrows, int ncols, int nnz, float* A, const int* Air, 
 
 API int bidmat_dds(int nrows, int nnz, const float* A, const float* B, const int* Cir,
                    const int* Cic, float* P) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || nnz < 0) return kInvalid;
     if (nnz == 0) return 0;
     if (!Cir || !Cic || !P || (nrows > 0 && (!A || !B))) return kInvalid;
@@ -225,6 +235,7 @@ API int bidmat_dds(int nrows, int nnz, const float* A, const float* B, const int
 
 API int bidmat_spsum(int nrows, int ncols, int nnz, const int* Air, const int* Aic, const float* P,
                      float* B, int n) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || ncols < 0 || nnz < 0) return kInvalid;
     if (nnz == 0) return 0;
     if (!Air || !Aic || !P || !B) return kInvalid;
@@ -244,6 +255,7 @@ API int bidmat_spsum(int nrows, int ncols, int nnz, const int* Air, const int* A
 }
 
 API int bidmat_reduce1op(int nrows, int ncols, const float* A, float* B, float initv, int opn) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || ncols < 0) return kInvalid;
     if (ncols == 0) return 0;
     if (!B || (nrows > 0 && !A)) return kInvalid;
@@ -251,6 +263,7 @@ API int bidmat_reduce1op(int nrows, int ncols, const float* A, float* B, float i
 }
 
 API int bidmat_reduce2op(int nrows, int ncols, const float* A, float* B, float initv, int opn) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || ncols < 0) return kInvalid;
     if (nrows == 0) return 0;
     if (!B || (ncols > 0 && !A)) return kInvalid;
@@ -270,6 +283,7 @@ API int bidmat_applyop(const float* A, int Anrows, int Ancols, const float* B, i
 
 API int bidmat_dsmult_csc(int k, int ncols, int nnz, const float* A, const float* Sdata,
                           const int* Sir, const int* Sjc, float* C, int beta, void* stream) {
+    auto lock = bm::device_lock();
     if (k < 0 || ncols < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
     if (k == 0 || ncols == 0) return 0;
     if (!Sjc || !C || (nnz > 0 && (!A || !Sdata || !Sir))) return kInvalid;
@@ -278,14 +292,41 @@ API int bidmat_dsmult_csc(int k, int ncols, int nnz, const float* A, const float
 
 API int bidmat_dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* Sir,
                        const int* Sjc, float* P, int beta, void* stream) {
+    auto lock = bm::device_lock();
     if (k < 0 || ncols < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
     if (ncols == 0 || nnz == 0) return 0;
     if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
     return (int)bm::dds_csc(k, ncols, nnz, A, B, Sir, Sjc, P, beta, as_stream(stream));
 }
 
+API int bidmat_dds_csc_op(int k, int ncols, int nnz, const float* A, const float* B, const int* Sir,
+                          const int* Sjc, const float* V, int opn, float* P, void* stream) {
+    auto lock = bm::device_lock();
+    if (k < 0 || ncols < 0 || nnz < 0 || opn < 0 || opn > 14) return kInvalid;
+    if (ncols == 0 || nnz == 0) return 0;
+    if (!Sjc || !Sir || !P || !V || (k > 0 && (!A || !B))) return kInvalid;
+    return (int)bm::dds_csc(k, ncols, nnz, A, B, Sir, Sjc, P, 0, as_stream(stream), V, opn);
+}
+
+API int bidmat_dds0(int nrows, int ncols, const float* A, const float* B, const int* Cir, const int* Cjc,
+                    float* P) {
+    auto lock = bm::device_lock();
+    if (nrows < 0 || ncols < 0) return kInvalid;
+    if (ncols == 0) return 0;
+    if (!Cjc) return kInvalid;
+    // the launcher has no nonzero count: it is the last column pointer
+    int nnz = 0;
+    hipError_t err = hipMemcpy(&nnz, Cjc + ncols, sizeof(int), hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return (int)err;
+    if (nnz < 0) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!Cir || !P || (nrows > 0 && (!A || !B))) return kInvalid;
+    return finish_blocking(bm::dds_csc(nrows, ncols, nnz, A, B, Cir, Cjc, P, 0, nullptr));
+}
+
 API int bidmat_plan_create(int nrows, int ncols, int nnz, const int* Sir, const int* Sjc, int k_hint,
                            bidmat_plan** plan) {
+    auto lock = bm::device_lock();
     if (!plan) return kInvalid;
     *plan = nullptr;
     if (nrows < 0 || ncols < 0 || nnz < 0 || k_hint < 0) return kInvalid;
@@ -300,19 +341,65 @@ API int bidmat_plan_destroy(bidmat_plan* plan) {
 
 API long long bidmat_plan_bytes(const bidmat_plan* plan) {
     if (!plan) return 0;
-    return (long long)(plan->index_bytes + plan->partial_floats * sizeof(float));
+    return (long long)(plan->index_bytes + (plan->partial_floats + plan->ovf_partial_floats) * sizeof(float) +
+                       (plan->pvals ? (size_t)plan->nnz * sizeof(float) : 0));
 }
 
 API int bidmat_plan_segments(const bidmat_plan* plan) { return plan ? plan->nseg : 0; }
 
 API int bidmat_dsmultT_plan(bidmat_plan* plan, int k, const float* A, const float* Sdata, float* C,
                             int beta, void* stream) {
+    auto lock = bm::device_lock();
     if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (k == 0 || plan->nrows == 0) return 0;
-    if (!C || (plan->nnz > 0 && (!A || !Sdata))) return kInvalid;
+    if (!C || (plan->nnz > 0 && (!A || (!Sdata && !plan->pvals)))) return kInvalid;
     return (int)run_dsmultT(plan, k, A, Sdata, C, beta, as_stream(stream));
 }
+
+namespace {
+// the plan's column table as the kernels take it
+bm::ColTable col_table(bidmat_plan* plan) {
+    return bm::ColTable{plan->col_seglen, plan->ovf, (long long)plan->novf, plan->ovf_partial};
+}
+}  // namespace
+
+API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float* Sdata, const int* Sir,
+                           const int* Sjc, float* C, int beta, void* stream) {
+    auto lock = bm::device_lock();
+    if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (k == 0 || plan->ncols == 0) return 0;
+    if (!Sjc || !C || (plan->nnz > 0 && (!A || !Sdata || !Sir))) return kInvalid;
+    if (plan->novf > 0) {
+        hipError_t err = bm::plan_reserve_ovf_partial(plan, k);
+        if (err != hipSuccess) return (int)err;
+    }
+    const bm::ColTable tab = col_table(plan);
+    return (int)bm::dsmult_csc(k, plan->ncols, plan->nnz, A, Sdata, Sir, Sjc, C, beta, as_stream(stream), &tab);
+}
+
+API int bidmat_dds_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc,
+                        const float* V, int opn, float* P, int beta, void* stream) {
+    auto lock = bm::device_lock();
+    if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (V && (beta != 0 || opn < 0 || opn > 14)) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (plan->ncols == 0 || plan->nnz == 0) return 0;
+    if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
+    const bm::ColTable tab = col_table(plan);
+    return (int)bm::dds_csc(k, plan->ncols, plan->nnz, A, B, Sir, Sjc, P, beta, as_stream(stream), V, opn, &tab);
+}
+
+API int bidmat_plan_set_values(bidmat_plan* plan, const float* Sdata, void* stream) {
+    if (!plan) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (plan->nnz == 0) return 0;
+    if (!Sdata) return kInvalid;
+    return (int)bm::plan_set_values(plan, Sdata, as_stream(stream));
+}
+
+API int bidmat_plan_overflow_segments(const bidmat_plan* plan) { return plan ? plan->novf : 0; }
 
 API int bidmat_spsum_cols(int ncols, int nnz, const float* Sdata, const int* Sjc, float* out, int beta,
                           void* stream) {
@@ -323,10 +410,11 @@ API int bidmat_spsum_cols(int ncols, int nnz, const float* Sdata, const int* Sjc
 }
 
 API int bidmat_spsum_rows_plan(bidmat_plan* plan, const float* Sdata, float* out, int beta, void* stream) {
+    auto lock = bm::device_lock();
     if (!plan || (beta != 0 && beta != 1)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (plan->nrows == 0) return 0;
-    if (!out || (plan->nnz > 0 && !Sdata)) return kInvalid;
+    if (!out || (plan->nnz > 0 && !Sdata && !plan->pvals)) return kInvalid;
     return (int)run_spsum_rows(plan, Sdata, out, beta, as_stream(stream));
 }
 
@@ -339,6 +427,7 @@ API int bidmat_transpose(int nrows, int ncols, const float* in, int ldi, float* 
 
 API int bidmat_sdtmult_csc(int nrows, int ncols, int nnz, int p, const float* Sdata, const int* Sir,
                            const int* Sjc, const float* A, int lda, float* C, int ldc, void* stream) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || ncols < 0 || nnz < 0 || p < 0 || lda < nrows || ldc < ncols) return kInvalid;
     if (ncols == 0 || p == 0) return 0;
     if (!Sjc || !C || (nnz > 0 && (!Sdata || !Sir || !A))) return kInvalid;
@@ -356,6 +445,7 @@ API int bidmat_sdtmult_csc(int nrows, int ncols, int nnz, int p, const float* Sd
 
 API int bidmat_sdmult_plan(bidmat_plan* plan, int p, const float* Sdata, const float* A, int lda, float* C,
                            int ldc, void* stream) {
+    auto lock = bm::device_lock();
     if (!plan || p < 0) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (lda < plan->ncols || ldc < plan->nrows) return kInvalid;
@@ -402,6 +492,7 @@ API int bidmat_csc_colslice(int col1, int col2, int start, int nnz, const int* S
 
 API int bidmat_csc_transpose(int nrows, int ncols, int nnz, const float* Sdata, const int* Sir, const int* Sjc,
                              float* out_data, int* out_ir, int* out_jc) {
+    auto lock = bm::device_lock();
     if (nrows < 0 || ncols < 0 || nnz < 0 || !out_jc) return kInvalid;
     if (nnz > 0 && (!Sdata || !Sir || !Sjc || !out_data || !out_ir)) return kInvalid;
     return finish_blocking(bm::csc_transpose(nrows, ncols, nnz, Sdata, Sir, Sjc, out_data, out_ir, out_jc, nullptr));
@@ -416,6 +507,7 @@ API int bidmat_full(const int* ir, const int* ic, const float* data, float* od, 
 
 API int bidmat_nhot(int n, int ncols, const int* cats, int* out_ir, int* out_ic, int* out_jc, float* out_data,
                     int* maxcat) {
+    auto lock = bm::device_lock();
     if (n < 0 || ncols < 0 || (long long)n * ncols > 0x7fffffffLL || !out_jc) return kInvalid;
     if ((long long)n * ncols > 0 && (!cats || !out_ir || !out_ic || !out_data)) return kInvalid;
     hipError_t err;
@@ -520,6 +612,7 @@ API int bidmat_stream_create(void** stream) {
     return (int)e;
 }
 API int bidmat_stream_destroy(void* stream) {
+    auto lock = bm::device_lock();
     if (!stream) return 0;
     hipError_t e = hipStreamSynchronize(as_stream(stream));
     hipError_t f = bm::ws_drop_stream(as_stream(stream));      // the stream's scratch goes with it
@@ -619,6 +712,7 @@ API long long bidmat_get_option(const char* name) {
 }
 
 API int bidmat_release_caches(void) {
+    auto lock = bm::device_lock();
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;

@@ -38,17 +38,22 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fill(T* __restrict__ out, long lon
     for (; i < n; i += stride) out[i] = v;
 }
 
-// Weight of position i in the digest: odd, and different positions get unrelated weights.
-__device__ __forceinline__ unsigned pos_weight(unsigned i) {
-    unsigned x = (i + 1u) * 0x9E3779B1u;
-    x ^= x >> 15; x *= 0x85EBCA77u;
-    x ^= x >> 13;
-    return x | 1u;
+// 64-bit finaliser (splitmix64): every input bit reaches every output bit.
+__device__ __forceinline__ unsigned long long mix64(unsigned long long x) {
+    x ^= x >> 30; x *= 0xBF58476D1CE4E5B9ULL;
+    x ^= x >> 27; x *= 0x94D049BB133111EBULL;
+    x ^= x >> 31;
+    return x;
+}
+// Contribution of (position i, value v) to a digest: a non-linear 64-bit hash of the pair, so that
+// neither moving a value to another position nor trading amounts between two positions cancels out.
+__device__ __forceinline__ unsigned long long digest_term(unsigned long long i, unsigned v, unsigned long long salt) {
+    return mix64(((i + 1ULL) << 32 | (unsigned long long)v) ^ salt);
 }
 
-// One pass over both index arrays of a pattern: digests sum_i weight(i) * (value_i + c) of ir and
-// of ic (64-bit integer sums: position-sensitive, independent of the order in which threads
-// contribute) and the largest row index. A workgroup walks tiles of 4 x 256 positions with four
+// One pass over both index arrays of a pattern: digests sum_i hash64(i, value_i) of ir and of ic
+// (64-bit integer sums: position-sensitive, independent of the order in which threads contribute)
+// and the largest row index. A workgroup walks tiles of 4 x 256 positions with four
 // loads per array in flight per thread. out: [0] digest of ir, [1] digest of ic, [2] (int) max.
 __global__ __launch_bounds__(BM_BLOCK) void k_pattern_digest(const int* __restrict__ ir, const int* __restrict__ ic,
                                                              long long n, unsigned long long* out) {
@@ -69,9 +74,8 @@ __global__ __launch_bounds__(BM_BLOCK) void k_pattern_digest(const int* __restri
         for (int u = 0; u < UN; ++u) {
             const long long j = i + u * BM_BLOCK;
             if (j < n) {
-                const unsigned long long w = pos_weight((unsigned)j);
-                ha += w * (unsigned long long)((unsigned)r[u] + 0x7F4A7C15u);
-                hb += w * (unsigned long long)((unsigned)c[u] + 0x2545F491u);
+                ha += digest_term((unsigned long long)j, (unsigned)r[u], 0x7F4A7C159E3779B9ULL);
+                hb += digest_term((unsigned long long)j, (unsigned)c[u], 0x2545F4914F6CDD1DULL);
                 m = max(m, r[u]);
             }
         }

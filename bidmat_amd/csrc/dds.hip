@@ -9,6 +9,7 @@
 // "its" nonzero, so a chunk of 64 results is written with one coalesced store.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "ops.hpp"
 #include "workspace.hpp"
 
 namespace bm {
@@ -25,6 +26,8 @@ struct DdsArgs {
     const int* jc;
     const int* ovf;
     float* P;
+    const float* V;      // epilogue operand (nullable): P[j] = op(V[j], dot_j)
+    int opn;
 };
 
 template <int V, int LPN>
@@ -33,7 +36,7 @@ struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw <
 template <int W, int V, int LPN, bool EXACT, bool FULL>
 __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, int myrow, float* o, int rem, int g,
                                           int l, const int (&eld)[V], const bool (&ev)[V],
-                                          const Vec<W> (&b)[V], bool accumulate) {
+                                          const Vec<W> (&b)[V], bool accumulate, const float* vq, int opn) {
     constexpr int NG = 64 / LPN;
     constexpr int U = Unroll<V, LPN>::U;
     const int q = l * NG + g;            // the nonzero of this chunk whose result this lane keeps
@@ -78,7 +81,11 @@ __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, in
             }
         }
     }
-    if (FULL || q < rem) *o = accumulate ? (*o + res) : res;      // o: where this lane's nonzero goes
+    if (FULL || q < rem) {                                        // o: where this lane's nonzero goes
+        if (accumulate) res += *o;
+        if (vq != nullptr) res = binop_rt(opn, *vq, res);         // only on the last pass over k
+        *o = res;
+    }
 }
 
 template <int W, int V, int LPN, bool EXACT>
@@ -132,8 +139,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
         while (rem > 0) {
             const int nrow = (q < rem - 64) ? a.ir[j0 + 64 + q] : 0;
             float* o = a.P + j0 + q;
-            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate);
-            else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate);
+            const float* vq = (a.V != nullptr && k0 + KT >= a.k) ? a.V + j0 + q : nullptr;
+            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, vq, a.opn);
+            else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, vq, a.opn);
             crow = nrow;
             j0 += 64;
             rem -= 64;
@@ -168,24 +176,36 @@ hipError_t launch_dds(const Shape& sh, bool exact, const DdsArgs& a, long long n
 }  // namespace
 
 hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
-                   const int* jc, float* P, int beta, hipStream_t s) {
+                   const int* jc, float* P, int beta, hipStream_t s, const float* V, int opn,
+                   const ColTable* tab) {
     if (ncols <= 0 || nnz <= 0) return hipSuccess;
+    if (V != nullptr && (beta != 0 || opn < 0 || opn > 14)) return hipErrorInvalidValue;
     if (k <= 0) {
-        // empty dot products: P = beta*P + 0
+        // empty dot products: P = beta*P + 0, or op(V, 0)
+        if (V != nullptr) {
+            hipError_t e = fill_f32(P, nnz, 0.f, s);
+            return e != hipSuccess ? e : applyop(V, nnz, 1, P, nnz, 1, P, opn, s);
+        }
         if (!beta) return fill_f32(P, nnz, 0.f, s);
         return hipSuccess;
     }
-    const int seglen = opt_seglen();
+    int seglen = opt_seglen();
     int* ovf = nullptr;
-    hipError_t err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
-    if (err != hipSuccess) return err;
-    long long novf_max = ovf ? nnz / seglen : 0;
+    long long novf_max = 0;
+    if (tab) {
+        seglen = tab->seglen;
+        if (tab->novf > 0) { ovf = const_cast<int*>(tab->ovf); novf_max = tab->novf; }
+    } else {
+        hipError_t err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
+        if (err != hipSuccess) return err;
+        novf_max = ovf ? nnz / seglen : 0;
+    }
     Shape sh = pick_shape(k, aligned16(A) && aligned16(B));
     if (sh.V > 4) sh.V = 4;
     const bool exact = (sh.W == 4) && (k % (sh.W * sh.V * sh.LPN) == 0);
     DdsArgs a;
     a.k = k; a.ncols = ncols; a.seglen = seglen; a.beta = beta;
-    a.A = A; a.B = B; a.ir = ir; a.jc = jc; a.ovf = ovf; a.P = P;
+    a.A = A; a.B = B; a.ir = ir; a.jc = jc; a.ovf = ovf; a.P = P; a.V = V; a.opn = opn;
     return launch_dds(sh, exact, a, (long long)ncols + novf_max, s);
 }
 

@@ -42,6 +42,10 @@ JFN(jint, sdopcol)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong A, jlong A
 JFN(jint, dds)(JNIEnv*, jclass, jint nr, jint nnz, jlong A, jlong B, jlong Cir, jlong Cic, jlong Pv) {
     return bidmat_dds(nr, nnz, P(const float, A), P(const float, B), P(const int, Cir), P(const int, Cic), P(float, Pv));
 }
+// replaces Java_edu_berkeley_bid_CUMAT_dds0 (BIDMat_CUMAT.cpp:787-798): column pointer instead of column indices
+JFN(jint, dds0)(JNIEnv*, jclass, jint nr, jint nc, jlong A, jlong B, jlong Cir, jlong Cjc, jlong Pv) {
+    return bidmat_dds0(nr, nc, P(const float, A), P(const float, B), P(const int, Cir), P(const int, Cjc), P(float, Pv));
+}
 // replaces Java_edu_berkeley_bid_CUMAT_spsum (BIDMat_CUMAT.cpp:873-882)
 JFN(jint, spsum)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong Air, jlong Aic, jlong Pv, jlong B, jint n) {
     return bidmat_spsum(nr, nc, nnz, P(const int, Air), P(const int, Aic), P(const float, Pv), P(float, B), n);
@@ -66,6 +70,12 @@ JFN(jint, ddsCsc)(JNIEnv*, jclass, jint k, jint nc, jint nnz, jlong A, jlong B, 
     int e = bidmat_dds_csc(k, nc, nnz, P(const float, A), P(const float, B), P(const int, Sir), P(const int, Sjc), P(float, Pv), beta, nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
+// DDS with the elementwise step fused in: Pv[j] = op(V[j], dot_j) (GSMat.DDS + GMat.gOp in one launch)
+JFN(jint, ddsCscOp)(JNIEnv*, jclass, jint k, jint nc, jint nnz, jlong A, jlong B, jlong Sir, jlong Sjc, jlong V, jint opn, jlong Pv) {
+    int e = bidmat_dds_csc_op(k, nc, nnz, P(const float, A), P(const float, B), P(const int, Sir), P(const int, Sjc),
+                              P(const float, V), opn, P(float, Pv), nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
 JFN(jlong, planCreate)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong Sir, jlong Sjc, jint khint) {
     bidmat_plan* p = nullptr;
     int e = bidmat_plan_create(nr, nc, nnz, P(const int, Sir), P(const int, Sjc), khint, &p);
@@ -74,6 +84,21 @@ JFN(jlong, planCreate)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jlong Sir, j
 JFN(jint, planDestroy)(JNIEnv*, jclass, jlong plan) { return bidmat_plan_destroy(P(bidmat_plan, plan)); }
 JFN(jint, dsmultTPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong Sdata, jlong C, jint beta) {
     int e = bidmat_dsmultT_plan(P(bidmat_plan, plan), k, P(const float, A), P(const float, Sdata), P(float, C), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+// A*S and DDS through a plan (one launch when no column is long), values kept in plan order
+JFN(jint, dsmultPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong Sdata, jlong Sir, jlong Sjc, jlong C, jint beta) {
+    int e = bidmat_dsmult_plan(P(bidmat_plan, plan), k, P(const float, A), P(const float, Sdata), P(const int, Sir),
+                               P(const int, Sjc), P(float, C), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jint, ddsPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong B, jlong Sir, jlong Sjc, jlong V, jint opn, jlong Pv, jint beta) {
+    int e = bidmat_dds_plan(P(bidmat_plan, plan), k, P(const float, A), P(const float, B), P(const int, Sir), P(const int, Sjc),
+                            P(const float, V), opn, P(float, Pv), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+JFN(jint, planSetValues)(JNIEnv*, jclass, jlong plan, jlong Sdata) {
+    int e = bidmat_plan_set_values(P(bidmat_plan, plan), P(const float, Sdata), nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
 // sparse sums without the per-nonzero column array (GSMat.sum, GSMat.scala:250-261)

@@ -41,20 +41,33 @@ hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned 
 // seglen-sized segments of each column), or nullptr when no column can exceed seglen.
 hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, int** d_ovf,
                                 hipStream_t s);
+// The same into caller-provided memory of overflow_table_ints(ncols) ints (no allocation).
+size_t overflow_table_ints(int ncols);
+hipError_t build_overflow_table_in(int ncols, int nnz, const int* jc, int seglen, int* buf, int** d_ovf,
+                                   hipStream_t s);
+// A column overflow table that the caller already holds (a plan builds it once per pattern):
+// seglen it was built with, table (ncols+1 ints; unused when novf == 0), number of overflow
+// segments, and for A*S a buffer of novf*k floats for their partial sums.
+struct ColTable { int seglen; const int* ovf; long long novf; float* partial; };
 
 // A window [off, off+len) on the gather index of the nonzeros (tile variants); on == 0: no filter.
 struct Window { int on, off, len; };
 
 // ---- A*S (spmm.hip)
 hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* vals, const int* ir,
-                      const int* jc, float* C, int beta, hipStream_t s);
+                      const int* jc, float* C, int beta, hipStream_t s, const ColTable* tab = nullptr);
 // tile form: A and C with their own column strides; only nonzeros with a row inside `rows`
 // take part, rebased to rows.off (jc already points at the first column of the tile).
 hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const float* A, const float* vals,
-                         const int* ir, const int* jc, float* C, int beta, Window rows, hipStream_t s);
+                         const int* ir, const int* jc, float* C, int beta, Window rows, hipStream_t s,
+                         const ColTable* tab = nullptr);
 // ---- DDS (dds.hip)
+// V != nullptr: P[j] = op(V[j], dot_j) with the BinOp code opn (beta must be 0) - the elementwise
+// step that follows DDS in an NMF update, applied before the result leaves the registers.
 hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
-                   const int* jc, float* P, int beta, hipStream_t s);
+                   const int* jc, float* P, int beta, hipStream_t s, const float* V = nullptr, int opn = 0,
+                   const ColTable* tab = nullptr);
+
 
 // ---- plan stage kernels (spmm.hip): segment s gathers columns pc[p] of A scaled by
 // vals[perm[p]] for p in [segstart[s], segstart[s+1]) into partial[s*k ..].

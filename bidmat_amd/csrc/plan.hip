@@ -169,7 +169,7 @@ inline int bits_for(unsigned long long maxval) {
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
     hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->block_nnz, p->block_seg, p->partial};
+    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals};
     for (void* b : bufs)
         if (b && (f = hipFree(b)) != hipSuccess) e = f;
     delete p;
@@ -185,9 +185,54 @@ hipError_t plan_reserve_partial(bidmat_plan* p, int k) {
         if (e != hipSuccess) return e;
     }
     hipError_t e = hipMalloc((void**)&p->partial, need * sizeof(float));
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess) { (void)hipGetLastError(); return e; }
     p->partial_floats = need;
     return hipSuccess;
+}
+
+hipError_t plan_reserve_ovf_partial(bidmat_plan* p, int k) {
+    size_t need = (size_t)p->novf * (size_t)k;
+    if (need <= p->ovf_partial_floats) return hipSuccess;
+    if (p->ovf_partial) {
+        hipError_t e = hipFree(p->ovf_partial);
+        p->ovf_partial = nullptr; p->ovf_partial_floats = 0;
+        if (e != hipSuccess) return e;
+    }
+    hipError_t e = hipMalloc((void**)&p->ovf_partial, need * sizeof(float));
+    if (e != hipSuccess) { (void)hipGetLastError(); return e; }
+    p->ovf_partial_floats = need;
+    return hipSuccess;
+}
+
+namespace {
+__global__ __launch_bounds__(BM_BLOCK) void k_permute_values(long long n, const float* __restrict__ data,
+                                                             const int* __restrict__ perm, float* __restrict__ out) {
+    // tiles of 4 x 256 positions per workgroup: four dependent gathers in flight per thread
+    constexpr int UN = 4;
+    long long i = (long long)blockIdx.x * (UN * BM_BLOCK) + threadIdx.x;
+    const long long stride = (long long)gridDim.x * (UN * BM_BLOCK);
+    for (; i < n; i += stride) {
+        int ix[UN];
+        float v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) { const long long j = i + u * BM_BLOCK; ix[u] = j < n ? perm[j] : 0; }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) v[u] = data[ix[u]];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) { const long long j = i + u * BM_BLOCK; if (j < n) out[j] = v[u]; }
+    }
+}
+}  // namespace
+
+hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s) {
+    if (p->nnz <= 0) return hipSuccess;
+    if (!p->pvals) {
+        hipError_t e = hipMalloc((void**)&p->pvals, sizeof(float) * (size_t)p->nnz);
+        if (e != hipSuccess) { (void)hipGetLastError(); p->pvals = nullptr; return e; }
+    }
+    hipLaunchKernelGGL(k_permute_values, dim3(grid_for(((long long)p->nnz + 3) / 4, 8192)), dim3(BM_BLOCK), 0, s,
+                       (long long)p->nnz, data, p->perm, p->pvals);
+    return hipGetLastError();
 }
 
 #define PB_CHECK(expr)                                          \
@@ -249,6 +294,24 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         PB_CHECK(hipStreamSynchronize(s));
         *out = plan;
         return hipSuccess;
+    }
+
+    // column side: the overflow-segment table of the columns, kept only when a column is longer
+    // than seglen
+    plan->col_seglen = opt_seglen();
+    {
+        int* tbl = nullptr;
+        PB_CHECK(build_overflow_table(ncols, nnz, jc, plan->col_seglen, &tbl, s));
+        if (tbl) {
+            int n = 0;
+            PB_CHECK(hipMemcpy(&n, tbl + ncols, sizeof(int), hipMemcpyDeviceToHost));
+            if (n > 0) {
+                PB_CHECK(hipMalloc((void**)&plan->ovf, sizeof(int) * ((size_t)ncols + 1)));
+                PB_CHECK(hipMemcpy(plan->ovf, tbl, sizeof(int) * ((size_t)ncols + 1), hipMemcpyDeviceToDevice));
+                plan->novf = n;
+                plan->index_bytes += sizeof(int) * ((size_t)ncols + 1);
+            }
+        }
     }
 
     // temporaries: one arena out of the library's workspace

@@ -34,6 +34,16 @@ struct bidmat_plan {
     float* partial = nullptr;
     size_t partial_floats = 0;
     size_t index_bytes = 0;
+    // Column side (A*S and DDS through the plan): the overflow-segment table of the columns is a
+    // function of jc and seglen only, so it is built once here instead of on every call.
+    int col_seglen = 0;          // seglen in force when the plan was built
+    int novf = 0;                // overflow segments of all columns (0: no column is longer than col_seglen)
+    int* ovf = nullptr;          // [ncols+1] exclusive scan of extra segments per column (only when novf > 0)
+    float* ovf_partial = nullptr;        // A*S: partial sums of the overflow segments (novf*k floats)
+    size_t ovf_partial_floats = 0;
+    // Values in plan order (optional, bidmat_plan_set_values): pvals[p] = data[perm[p]], so that
+    // A*^S and row sums stream their values instead of fetching each one through perm.
+    float* pvals = nullptr;
 };
 
 namespace bm {
@@ -42,4 +52,8 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
 hipError_t plan_free(bidmat_plan* p);
 // Makes sure the plan's partial buffer holds nseg*k floats.
 hipError_t plan_reserve_partial(bidmat_plan* p, int k);
+// Makes sure the buffer for the overflow partials of A*S holds novf*k floats.
+hipError_t plan_reserve_ovf_partial(bidmat_plan* p, int k);
+// pvals[p] = data[perm[p]] (allocates pvals on first use).
+hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s);
 }  // namespace bm

@@ -36,7 +36,7 @@ struct GatherArgs {
     const float* A;
     const float* vals;
     const int* idx;      // ir (CSC mode) / pc (plan mode): which column of A to gather
-    const int* perm;     // plan mode: position of the value in the original CSC order
+    const int* perm;     // plan mode: position of the value in the original CSC order (nullptr: vals is in plan order)
     const int* ptr;      // jc (CSC mode) / segstart (plan mode)
     const int* ovf;      // CSC mode: overflow table (nullable)
     float* out;          // C (CSC mode) / partial (plan mode)
@@ -57,7 +57,7 @@ __device__ __forceinline__ void load_chunk(const GatherArgs& a, int j0, int ahea
     if (q < rem) {
         const int p = j0 + ahead + q;
         myrow = a.idx[p];
-        myval = PLAN ? a.vals[a.perm[p]] : a.vals[p];
+        myval = (PLAN && a.perm != nullptr) ? a.vals[a.perm[p]] : a.vals[p];     // perm == nullptr: values already in plan order
     }
 }
 
@@ -355,12 +355,15 @@ static Shape clamp_shape(Shape sh) {
     return sh;
 }
 
-hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, int** d_ovf, hipStream_t s) {
+size_t overflow_table_ints(int ncols) {
+    // table area (2*ncols + 2 ints, rounded to 64) followed by the scan's block sums
+    const size_t area = ((2 * (size_t)ncols + 2) + 63) & ~size_t(63);
+    return area + scan_tmp_ints(ncols);
+}
+
+hipError_t build_overflow_table_in(int ncols, int nnz, const int* jc, int seglen, int* buf, int** d_ovf, hipStream_t s) {
     *d_ovf = nullptr;
     if (nnz <= seglen || ncols <= 0) return hipSuccess;
-    hipError_t err;
-    int* buf = (int*)ws_get(WS_OVF, sizeof(int) * (2 * (size_t)ncols + 2), &err, s);
-    if (!buf) return err;
     unsigned nblk = (unsigned)(((long long)ncols + BM_BLOCK - 1) / BM_BLOCK);
     if (nblk <= (unsigned)OVF2_MAX_BLOCKS) {
         int* bsum = buf + ncols + 1;
@@ -369,15 +372,23 @@ hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, i
         *d_ovf = buf;
         return hipGetLastError();
     }
-    int* tmp = (int*)ws_get(WS_SCAN, sizeof(int) * scan_tmp_ints(ncols), &err, s);
-    if (!tmp) return err;
+    int* tmp = buf + (((2 * (size_t)ncols + 2) + 63) & ~size_t(63));
     int* extra = buf;
     int* ovf = buf + ncols + 1;
     hipLaunchKernelGGL(k_extra_segments, dim3(nblk), dim3(BM_BLOCK), 0, s, ncols, jc, seglen, extra);
-    err = scan_exclusive_i32(extra, ovf, ncols, tmp, s);
+    hipError_t err = scan_exclusive_i32(extra, ovf, ncols, tmp, s);
     if (err != hipSuccess) return err;
     *d_ovf = ovf;
     return hipGetLastError();
+}
+
+hipError_t build_overflow_table(int ncols, int nnz, const int* jc, int seglen, int** d_ovf, hipStream_t s) {
+    *d_ovf = nullptr;
+    if (nnz <= seglen || ncols <= 0) return hipSuccess;
+    hipError_t err;
+    int* buf = (int*)ws_get(WS_OVF, sizeof(int) * overflow_table_ints(ncols), &err, s);
+    if (!buf) return err;
+    return build_overflow_table_in(ncols, nnz, jc, seglen, buf, d_ovf, s);
 }
 
 namespace {
@@ -389,23 +400,31 @@ void init_args(GatherArgs& a) {
 }  // namespace
 
 hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* vals, const int* ir,
-                      const int* jc, float* C, int beta, hipStream_t s) {
-    return dsmult_csc_ex(k, k, k, ncols, nnz, A, vals, ir, jc, C, beta, Window{0, 0, 0}, s);
+                      const int* jc, float* C, int beta, hipStream_t s, const ColTable* tab) {
+    return dsmult_csc_ex(k, k, k, ncols, nnz, A, vals, ir, jc, C, beta, Window{0, 0, 0}, s, tab);
 }
 
 hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const float* A, const float* vals,
-                         const int* ir, const int* jc, float* C, int beta, Window rows, hipStream_t s) {
+                         const int* ir, const int* jc, float* C, int beta, Window rows, hipStream_t s,
+                         const ColTable* tab) {
     if (k <= 0 || ncols <= 0) return hipSuccess;
-    const int seglen = opt_seglen();
+    int seglen = opt_seglen();
     int* ovf = nullptr;
-    hipError_t err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
-    if (err != hipSuccess) return err;
     float* partial = nullptr;
     long long novf_max = 0;
-    if (ovf) {
-        novf_max = nnz / seglen;
-        partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err, s);
-        if (!partial) return err;
+    hipError_t err;
+    if (tab) {
+        // the caller knows the pattern's overflow segments: nothing to build, nothing to allocate
+        seglen = tab->seglen;
+        if (tab->novf > 0) { ovf = const_cast<int*>(tab->ovf); novf_max = tab->novf; partial = tab->partial; }
+    } else {
+        err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
+        if (err != hipSuccess) return err;
+        if (ovf) {
+            novf_max = nnz / seglen;
+            partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err, s);
+            if (!partial) return err;
+        }
     }
     const bool al = aligned16(A) && aligned16(C) && aligned16(partial) && lda % 4 == 0 && ldc % 4 == 0;
     Shape sh = clamp_shape(pick_shape(k, al));

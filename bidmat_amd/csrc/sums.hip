@@ -52,11 +52,19 @@ __global__ __launch_bounds__(BM_BLOCK) void k_spsum_plan(int nseg, XcdStarts xs,
         const int s = segstart[seg], e = segstart[seg + 1];
         float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
         int j = s + l;
-        for (; j + 48 < e; j += 64) {
-            const int p0 = perm[j], p1 = perm[j + 16], p2 = perm[j + 32], p3 = perm[j + 48];
-            a0 += vals[p0]; a1 += vals[p1]; a2 += vals[p2]; a3 += vals[p3];
+        if (perm != nullptr) {
+            for (; j + 48 < e; j += 64) {
+                const int p0 = perm[j], p1 = perm[j + 16], p2 = perm[j + 32], p3 = perm[j + 48];
+                a0 += vals[p0]; a1 += vals[p1]; a2 += vals[p2]; a3 += vals[p3];
+            }
+            for (; j < e; j += 16) a0 += vals[perm[j]];
+        } else {                                        // values already in plan order
+            for (; j + 48 < e; j += 64) {
+                const float v0 = vals[j], v1 = vals[j + 16], v2 = vals[j + 32], v3 = vals[j + 48];
+                a0 += v0; a1 += v1; a2 += v2; a3 += v3;
+            }
+            for (; j < e; j += 16) a0 += vals[j];
         }
-        for (; j < e; j += 16) a0 += vals[perm[j]];
         acc = (a0 + a1) + (a2 + a3);
     }
     acc = group_allsum<16>(acc);

@@ -13,6 +13,7 @@ struct Slot { void* ptr = nullptr; size_t bytes = 0; };
 using SlotSet = std::array<Slot, WS_NSLOTS>;
 std::map<std::pair<int, hipStream_t>, SlotSet> g_sets;      // (device, stream) -> slots
 std::mutex g_mu;
+std::map<int, std::recursive_mutex> g_device_mu;            // nodes of a std::map never move
 
 bool debug_mem() {
     static int v = -1;
@@ -52,9 +53,10 @@ void* ws_get(WsSlot slot, size_t bytes, hipError_t* err, hipStream_t stream) {
     want = (want + 255) & ~size_t(255);
     *err = hipMalloc(&s.ptr, want);
     if (*err != hipSuccess) {
+        (void)hipGetLastError();            // handled here: do not leave it for the next launch check
         *err = hipMalloc(&s.ptr, bytes);
         want = bytes;
-        if (*err != hipSuccess) { s.ptr = nullptr; return nullptr; }
+        if (*err != hipSuccess) { (void)hipGetLastError(); s.ptr = nullptr; return nullptr; }
     }
     s.bytes = want;
     if (debug_mem())
@@ -104,6 +106,17 @@ hipError_t ws_release() {
         }
     }
     return e;
+}
+
+std::unique_lock<std::recursive_mutex> device_lock() {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    std::recursive_mutex* m;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        m = &g_device_mu[dev];
+    }
+    return std::unique_lock<std::recursive_mutex>(*m);
 }
 
 size_t ws_bytes() {

@@ -4,6 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stddef.h>
+#include <mutex>
 
 namespace bm {
 
@@ -33,5 +34,12 @@ hipError_t ws_drop_stream(hipStream_t stream);
 hipError_t ws_release();
 // Total bytes currently held on the current device.
 size_t ws_bytes();
+
+// Host threads that share a device also share its scratch buffers and cached plans. Every entry
+// point that takes scratch or a cached plan holds this lock of the current device from its first
+// ws_get to its last launch (the blocking entries: until their synchronisation), so that another
+// thread can neither refill a buffer between "table built" and "kernel that reads it enqueued" nor
+// grow (free) a buffer whose address was just handed out. Recursive: entries may nest.
+std::unique_lock<std::recursive_mutex> device_lock();
 
 }  // namespace bm

@@ -23,6 +23,7 @@ SIGNATURES = {
     "bidmat_sdoprow": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, C.c_int, C.c_int]),
     "bidmat_sdopcol": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, C.c_int, C.c_int]),
     "bidmat_dds": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp, vp]),
+    "bidmat_dds0": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp, vp]),
     "bidmat_spsum": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int]),
     "bidmat_reduce1op": (C.c_int, [C.c_int, C.c_int, vp, vp, C.c_float, C.c_int]),
     "bidmat_reduce2op": (C.c_int, [C.c_int, C.c_int, vp, vp, C.c_float, C.c_int]),
@@ -30,6 +31,11 @@ SIGNATURES = {
     # native entries
     "bidmat_dsmult_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),
     "bidmat_dds_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),
+    "bidmat_dds_csc_op": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp, vp]),
+    "bidmat_plan_set_values": (C.c_int, [vp, vp, vp]),
+    "bidmat_dsmult_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),
+    "bidmat_dds_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp, C.c_int, vp]),
+    "bidmat_plan_overflow_segments": (C.c_int, [vp]),
     "bidmat_plan_create": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, C.POINTER(vp)]),
     "bidmat_plan_destroy": (C.c_int, [vp]),
     "bidmat_plan_bytes": (C.c_longlong, [vp]),

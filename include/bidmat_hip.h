@@ -21,6 +21,13 @@
  *     different streams may overlap; calls that use the same plan handle share its
  *     partial-sum buffer and must be ordered with each other.
  *   - results are deterministic: no floating-point atomics anywhere.
+ *   - threads: every entry point may be called from any host thread. Calls that take library
+ *     scratch or a cached plan (all product, sum and reduction entries) hold a per-device lock
+ *     while they look up / build their scratch and enqueue their kernels (the blocking entries:
+ *     until their result is complete), so two threads that drive one device through the blocking
+ *     entries or share a stream never see each other's scratch. What stays with the caller:
+ *     one plan handle must not be used by two calls at the same time (its partial-sum buffer
+ *     is one), and option changes (bidmat_set_option) are process-wide.
  */
 #ifndef BIDMAT_HIP_H
 #define BIDMAT_HIP_H
@@ -81,6 +88,14 @@ int bidmat_sdopcol(int nrows, int ncols, int nnz, float *A, const int *Air, cons
 int bidmat_dds(int nrows, int nnz, const float *A, const float *B, const int *Cir,
                const int *Cic, float *P);
 
+/* P[j] = dot(A[:,Cir[j]], B[:,c]) for every nonzero j of column c, with the column POINTER Cjc
+ * (ncols+1 entries) instead of the per-nonzero column array; overwrites P.  Replaces `int dds0(int nrows,
+ * int ncols,float*A,float*B,int*Cir,int*Cjc,float*P)` (MatKernel.hpp:156, Arith.cu:312-347,391-397;
+ * CUMAT.java:213; caller GSMat.DDS0, GSMat.scala:669-684).  The reference kernel assumes nrows == 1024
+ * (Arith.cu:316-324); any nrows works here.  Blocking. */
+int bidmat_dds0(int nrows, int ncols, const float *A, const float *B, const int *Cir, const int *Cjc,
+                float *P);
+
 /* Sparse sums: n == 1: B[Aic[i]] += P[i] (column sums, B has ncols entries); otherwise
  * B[Air[i]] += P[i] (row sums, B has nrows entries).  Replaces `int spsum(...)`
  * (Arith.cu:266-277; CUMAT.java:209; caller GSMat.scala:255). */
@@ -120,6 +135,14 @@ int bidmat_dsmult_csc(int k, int ncols, int nnz, const float *A, const float *Sd
 int bidmat_dds_csc(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir,
                    const int *Sjc, float *P, int beta, void *stream);
 
+/* DDS with the elementwise step that follows it in an NMF / LDA update fused into the kernel:
+ * P[j] = op(V[j], dot_j) with a BinOp code opn (3 = V ./ DDS).  One launch instead of
+ * GSMat.DDS + GMat.gOp on the value arrays (GSMat.scala:649-667, GMat.scala:1119-1128,
+ * Operators.cu:455-461); bit-identical to bidmat_dds_csc followed by bidmat_applyop_flat.
+ * V and P must not overlap (wide k is walked in several passes that keep their running sums in P). */
+int bidmat_dds_csc_op(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir,
+                      const int *Sjc, const float *V, int opn, float *P, void *stream);
+
 /* Row-binned execution plan of one sparsity pattern, needed by A*^S and by sparse row sums.
  * The plan keeps its own device copies of what it needs; the pattern arrays may be freed
  * afterwards.  The values array is NOT captured: pass the current values to each call.
@@ -140,6 +163,24 @@ int bidmat_plan_segments(const bidmat_plan *plan);
  * rows of S). */
 int bidmat_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *Sdata, float *C,
                         int beta, void *stream);
+
+/* The values of the pattern in plan order, stored in the plan (nnz floats): afterwards
+ * bidmat_dsmultT_plan, bidmat_sdmult_plan and bidmat_spsum_rows_plan accept Sdata == NULL and stream
+ * the stored values instead of fetching every value through the plan's permutation.  For callers
+ * whose values stay the same over several calls (a data minibatch); call it again when they change. */
+int bidmat_plan_set_values(bidmat_plan *plan, const float *Sdata, void *stream);
+
+/* A*S and DDS through a plan: the plan holds what is a function of the pattern alone (whether any
+ * column is longer than a wave segment, and the table of the extra segments if so), so a call is
+ * one launch when no column is long, and never builds or allocates per call.  Same results, bit for
+ * bit, as bidmat_dsmult_csc / bidmat_dds_csc / bidmat_dds_csc_op.  Sir / Sjc: the pattern the plan
+ * was made from.  bidmat_dds_plan: V == NULL gives P = beta*P + DDS, otherwise P = op(V, DDS). */
+int bidmat_dsmult_plan(bidmat_plan *plan, int k, const float *A, const float *Sdata, const int *Sir,
+                       const int *Sjc, float *C, int beta, void *stream);
+int bidmat_dds_plan(bidmat_plan *plan, int k, const float *A, const float *B, const int *Sir,
+                    const int *Sjc, const float *V, int opn, float *P, int beta, void *stream);
+/* Number of extra wave segments of the plan's long columns (0: every column fits one segment). */
+int bidmat_plan_overflow_segments(const bidmat_plan *plan);
 
 /* Sparse sums with jc / a plan: out = beta*out + sums.  Column sums need only jc;
  * row sums need a plan. */
