@@ -299,6 +299,17 @@ API int bidmat_dds_csc(int k, int ncols, int nnz, const float* A, const float* B
     return (int)bm::dds_csc(k, ncols, nnz, A, B, Sir, Sjc, P, beta, as_stream(stream));
 }
 
+API int bidmat_dds_csc_static(int k, int ncols, int nnz, const float* A, const float* B, const int* Sir,
+                              const int* Sjc, float* P, int beta, void* stream) {
+    if (k < 0 || ncols < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (ncols > bm::dds_static_max_cols()) return kInvalid;      // beyond the fixed scratch array
+    if (ncols == 0 || nnz == 0) return 0;
+    if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
+    return (int)bm::dds_csc_static(k, ncols, nnz, A, B, Sir, Sjc, P, beta, as_stream(stream));
+}
+
+API int bidmat_dds_static_max_cols(void) { return bm::dds_static_max_cols(); }
+
 API int bidmat_dds_csc_op(int k, int ncols, int nnz, const float* A, const float* B, const int* Sir,
                           const int* Sjc, const float* V, int opn, float* P, void* stream) {
     auto lock = bm::device_lock();

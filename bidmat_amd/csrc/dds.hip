@@ -11,6 +11,7 @@
 #include "kernels.hpp"
 #include "ops.hpp"
 #include "workspace.hpp"
+#include <mutex>
 
 namespace bm {
 namespace {
@@ -207,6 +208,58 @@ hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, co
     a.k = k; a.ncols = ncols; a.seglen = seglen; a.beta = beta;
     a.A = A; a.B = B; a.ir = ir; a.jc = jc; a.ovf = ovf; a.P = P; a.V = V; a.opn = opn;
     return launch_dds(sh, exact, a, (long long)ncols + novf_max, s);
+}
+
+// ---------------------------------------------------------------- DDS that allocates nothing
+// The only device memory dds_csc needs beyond its arguments is the overflow-segment table of the
+// columns. Here it lives in a fixed array inside the library's code object (every device that
+// loads the library holds its own copy until the process ends), so the call allocates nothing.
+// All calls on one device share the array: calls that overlap on a device race on it.
+namespace {
+constexpr int STATIC_MAX_COLS = 1 << 21;
+// table area (2*ncols + 2 ints, rounded up to 64) + block sums of the scan (one per 2048 columns)
+constexpr size_t STATIC_SCRATCH_INTS = (((2 * (size_t)STATIC_MAX_COLS + 2) + 63) & ~size_t(63)) + STATIC_MAX_COLS / 2048 + 64;
+static __device__ __align__(256) int scratch[STATIC_SCRATCH_INTS];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_static_mu;
+int* g_static_ptr[STATIC_MAX_DEVICES] = {nullptr};
+
+// Device address of this device's copy of `scratch` (the array's name is only a host-side handle).
+hipError_t static_scratch(int** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    if (!g_static_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        g_static_ptr[dev] = static_cast<int*>(p);
+    }
+    *out = g_static_ptr[dev];
+    return hipSuccess;
+}
+}  // namespace
+
+int dds_static_max_cols() { return STATIC_MAX_COLS; }
+
+hipError_t dds_csc_static(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
+                          const int* jc, float* P, int beta, hipStream_t s) {
+    if (ncols <= 0 || nnz <= 0) return hipSuccess;
+    if (ncols > STATIC_MAX_COLS || overflow_table_ints(ncols) > STATIC_SCRATCH_INTS) return hipErrorInvalidValue;
+    if (k <= 0) return beta ? hipSuccess : fill_f32(P, nnz, 0.f, s);
+    int* buf = nullptr;
+    hipError_t err = static_scratch(&buf);
+    if (err != hipSuccess) return err;
+    const int seglen = opt_seglen();
+    int* ovf = nullptr;
+    // every entry of the table that the kernels read is written by this build: nothing to clear
+    err = build_overflow_table_in(ncols, nnz, jc, seglen, buf, &ovf, s);
+    if (err != hipSuccess) return err;
+    const ColTable tab{seglen, ovf, ovf ? (long long)(nnz / seglen) : 0, nullptr};
+    return dds_csc(k, ncols, nnz, A, B, ir, jc, P, beta, s, nullptr, 0, &tab);
 }
 
 }  // namespace bm

@@ -67,7 +67,11 @@ hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const floa
 hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
                    const int* jc, float* P, int beta, hipStream_t s, const float* V = nullptr, int opn = 0,
                    const ColTable* tab = nullptr);
-
+// The same with no allocation at all: the overflow table lives in a fixed device array of the
+// library (one copy per device). ncols may not exceed dds_static_max_cols().
+int dds_static_max_cols();
+hipError_t dds_csc_static(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
+                          const int* jc, float* P, int beta, hipStream_t s);
 
 // ---- plan stage kernels (spmm.hip): segment s gathers columns pc[p] of A scaled by
 // vals[perm[p]] for p in [segstart[s], segstart[s+1]) into partial[s*k ..].

@@ -31,6 +31,8 @@ SIGNATURES = {
     # native entries
     "bidmat_dsmult_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),
     "bidmat_dds_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),
+    "bidmat_dds_csc_static": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),
+    "bidmat_dds_static_max_cols": (C.c_int, []),
     "bidmat_dds_csc_op": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp, vp]),
     "bidmat_plan_set_values": (C.c_int, [vp, vp, vp]),
     "bidmat_dsmult_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),

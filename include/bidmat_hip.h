@@ -135,6 +135,18 @@ int bidmat_dsmult_csc(int k, int ncols, int nnz, const float *A, const float *Sd
 int bidmat_dds_csc(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir,
                    const int *Sjc, float *P, int beta, void *stream);
 
+/* bidmat_dds_csc for callers that must not allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results, bit for bit, as bidmat_dds_csc; the one scratch buffer that call
+ * takes from the library's workspace (the table of extra wave segments of long columns) lives here
+ * in a fixed 16 MiB array inside the library, one copy per device, which limits
+ * ncols <= bidmat_dds_static_max_cols() (2 097 152); more columns return hipErrorInvalidValue.
+ * No hipMalloc / hipFree or allocating routine is called.  Every call on a device uses that
+ * device's one array: calls that overlap on a device (two streams, two threads) race on it. */
+int bidmat_dds_csc_static(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir,
+                          const int *Sjc, float *P, int beta, void *stream);
+int bidmat_dds_static_max_cols(void);
+
 /* DDS with the elementwise step that follows it in an NMF / LDA update fused into the kernel:
  * P[j] = op(V[j], dot_j) with a BinOp code opn (3 = V ./ DDS).  One launch instead of
  * GSMat.DDS + GMat.gOp on the value arrays (GSMat.scala:649-667, GMat.scala:1119-1128,
