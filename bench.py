@@ -6,8 +6,11 @@ P = DDS(A,B,S), C = A*S and G = A_T *^ S at k=256 on the Zipf(1.1) 100000 x 5000
 ~100 M nonzeros (BASELINE.json configs[1] and configs[2] plus A*S on the same pattern, which
 the metric names). Inputs are synthetic, seeded, and resident in HBM before the timed region.
 
-Prints ONE JSON line. `value` is the algorithmic GB/s of the whole step; per-op figures, the
-roofline object of the DDS kernel and the CPU baseline ride along.
+Prints ONE JSON line. `value` is the algorithmic GB/s of the whole step (the gathered dense operand
+charged once per nonzero, so caches can push it above the HBM peak); per-op figures, the roofline
+object of the DDS kernel (with a bound that cannot exceed 1: compulsory bytes at the HBM peak, or
+the same kernel's rate on an L2-resident operand, measured live), the CPU baseline and the check of
+every timed output against the CPU oracle ride along.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload headline|C1|C4|C5]
                   [--scale S] [--no-cpu] [--calibrate]
@@ -31,20 +34,39 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM-side bytes per launch of the roofline kernel at full scale: rocprofv3 FETCH_SIZE x 2.0 plus
-# WRITE_SIZE x 1.0 (KiB per dispatch; the factors are what the same counters read for the streaming
-# kernel of --calibrate, which moves a known 2 GiB + 1 GiB). The counter runs and their tables are
-# kept in profiles/headline_kernel_trace_and_hbm_counters.txt; a profiler cannot run inside this
-# script, so the figure is reported only for the exact workload it was measured on.
-MEASURED_TRAFFIC_BYTES = {("headline", "dds", 100003320): 41.8e9,
-                          ("C4", "dsmult", 38900534): 163.1e9}   # profiles/other_workloads_kernel_trace_and_hbm_counters.txt
+# L2-miss bytes per launch of the roofline kernel at full scale (fabric side of L2: Infinity Cache
+# and HBM together), from rocprofv3 FETCH_SIZE x 2.0 plus WRITE_SIZE x 1.0 (KiB per dispatch; the
+# factors are what the same counters read for the streaming kernel of --calibrate, which moves a
+# known 2 GiB + 1 GiB). A profiler cannot run inside this script, so each figure names the summary
+# under profiles/ it was taken from and the sha256 (first 16 hex digits) of the kernel source it
+# was taken on; it is reported only for that exact workload and dropped (null) as soon as the
+# kernel source differs.
+MEASURED_TRAFFIC = {
+    ("headline", "dds", 100003320): (41.8e9, "bidmat_amd/csrc/dds.hip", "@DDS_SHA@",
+                                     "profiles/headline_kernel_trace_and_hbm_counters.txt"),
+    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "@SPMM_SHA@",
+                                 "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
+}
+
+
+def measured_traffic(workload, op, nnz):
+    import hashlib
+    rec = MEASURED_TRAFFIC.get((workload, op, nnz))
+    if rec is None:
+        return None, None
+    nbytes, src, sha, where = rec
+    try:
+        cur = hashlib.sha256(open(os.path.join(ROOT, src), "rb").read()).hexdigest()[:16]
+    except OSError:
+        return None, None
+    return (nbytes, where) if cur == sha else (None, None)
 
 
 def alg_bytes(op, k, nnz, nrows, ncols):
     """Algorithmic bytes of one call: the gathered dense operand is charged once per nonzero,
     the streamed side once per column (row for A*^S), indices/values once."""
-    if op in ("dds", "dsmult"):
-        return nnz * (4 * k + 8) + ncols * (4 * k + 4) + 4
+    if op in ("dds", "dsmult", "dds_op"):
+        return nnz * (4 * k + 8) + ncols * (4 * k + 4) + 4 + (4 * nnz if op == "dds_op" else 0)
     if op == "dsmultT":
         return nnz * (4 * k + 8) + nrows * (4 * k + 4) + 4
     if op == "ewise":              # elementwise on the nonzero values: two reads, one write
@@ -54,11 +76,22 @@ def alg_bytes(op, k, nnz, nrows, ncols):
     raise ValueError(op)
 
 
+def compulsory_bytes(op, k, nnz, nrows, ncols):
+    """Every array of the call read or written exactly once (what an infinite cache would leave)."""
+    if op in ("dds", "dds_op"):    # A, B, ir, jc, P (+ V)
+        return 4 * k * (nrows + ncols) + 8 * nnz + 4 * (ncols + 1) + (4 * nnz if op == "dds_op" else 0)
+    if op == "dsmult":             # A, values, ir, jc, C
+        return 4 * k * (nrows + ncols) + 8 * nnz + 4 * (ncols + 1)
+    if op == "dsmultT":            # A, values, column of each nonzero, row pointer, C
+        return 4 * k * (nrows + ncols) + 8 * nnz + 4 * (nrows + 1)
+    return alg_bytes(op, k, nnz, nrows, ncols)
+
+
 def flops(op, k, nnz, ncols):
     """The reference's own accounting (GMat.scala:1057,1092; GSMat.scala:665; length for the
     elementwise op and the reduction)."""
-    if op in ("dds", "dsmult", "dsmultT"):
-        return 2.0 * k * nnz
+    if op in ("dds", "dsmult", "dsmultT", "dds_op"):
+        return 2.0 * k * nnz + (nnz if op == "dds_op" else 0)
     if op == "ewise":
         return float(nnz)
     return float(k) * ncols
@@ -71,7 +104,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="headline", choices=["headline", "C1", "C4", "C5", "next", "footprint"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows/columns of the pattern (testing)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs (baseline timing and verification)")
     ap.add_argument("--cpu-sample", type=float, default=1.0,
                     help="fraction of the columns timed on the CPU (1.0 = the whole workload)")
     ap.add_argument("--calibrate", action="store_true",
@@ -138,42 +171,45 @@ def main():
             hip_abi.check(lib.bidmat_synchronize())
             t_plan[i] = time.time() - t
 
-    # ---- the ops of one step: (name, kind, launcher)
+    # ---- the ops of one step: (name, kind, launcher). Every workload goes through a plan: the plan
+    # holds what depends on the pattern alone, so no call builds or allocates anything.
+    build_plan()
+    outputs = {}
     if args.workload == "headline":
         d_A, d_B, d_AT = (up(cfg[x]) for x in ("A", "B", "A_T"))
         d_P, d_C, d_G = DeviceArray(nnz, np.float32), DeviceArray(k * ncols, np.float32), DeviceArray(k * nrows, np.float32)
         keep += [d_A, d_B, d_AT, d_P, d_C, d_G]
-        build_plan()
+        outputs = {"dds": d_P, "dsmult": d_C, "dsmultT": d_G}
         ops = [
-            ("dds", "dds", lambda: lib.bidmat_dds_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_P.ptr, 0, stream)),
-            ("dsmult", "dsmult", lambda: lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream)),
+            ("dds", "dds", lambda: lib.bidmat_dds_plan(plan, k, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, None, 0, d_P.ptr, 0, stream)),
+            ("dsmult", "dsmult", lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream)),
             ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_AT.ptr, d_v.ptr, d_G.ptr, 0, stream)),
         ]
         workload = "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), step = DDS, A*S, A*^S"
-        metric = "achieved HBM GB/s (algorithmic bytes) for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
+        metric = "algorithmic GB/s (gathered operand charged once per nonzero) and nnz/s for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
         roof_op, roof_kernel = "dds", "k_dds<W=4,V=1,LPN=64> (one launch = DDS over the whole pattern)"
     elif args.workload in ("C1", "C4"):
         d_A = up(cfg["A"])
         d_C = DeviceArray(k * ncols, np.float32)
         keep += [d_A, d_C]
-        ops = [("dsmult", "dsmult", lambda: lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream))]
+        outputs = {"dsmult": d_C}
+        ops = [("dsmult", "dsmult", lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream))]
         workload = "configs[0]: A*S, k=32, 50 nnz per column" if args.workload == "C1" else \
             "configs[3]: A*S, k=1024, Pareto(1.5) column lengths in [1,50000]"
-        metric = "achieved HBM GB/s (algorithmic bytes) for A*S (%s)" % args.workload
+        metric = "algorithmic GB/s (gathered operand charged once per nonzero) for A*S (%s)" % args.workload
         roof_op = "dsmult"
         roof_kernel = "k_gather_axpy<W=4,V=1,LPN=8>" if args.workload == "C1" else "k_gather_axpy<W=4,V=4,LPN=64>"
-    else:  # C5: R = DDS(W,H,V); Q = V./R; G = H *^ Q; rs = sum(H,2)
+    else:  # C5: Q = V ./ DDS(W,H,V) in one launch; G = H *^ Q; rs = sum(H,2)
         d_W, d_H = up(cfg["W"]), up(cfg["H"])
-        d_R, d_G, d_rs = DeviceArray(nnz, np.float32), DeviceArray(k * nrows, np.float32), DeviceArray(k, np.float32)
-        keep += [d_W, d_H, d_R, d_G, d_rs]
-        build_plan()
+        d_Q, d_G, d_rs = DeviceArray(nnz, np.float32), DeviceArray(k * nrows, np.float32), DeviceArray(k, np.float32)
+        keep += [d_W, d_H, d_Q, d_G, d_rs]
+        outputs = {"dds_op": d_Q, "dsmultT": d_G}
         ops = [
-            ("dds", "dds", lambda: lib.bidmat_dds_csc(k, ncols, nnz, d_W.ptr, d_H.ptr, d_ir.ptr, d_jc.ptr, d_R.ptr, 0, stream)),
-            ("ewise", "ewise", lambda: lib.bidmat_applyop_flat(d_v.ptr, d_R.ptr, d_R.ptr, nnz, 3, stream)),
-            ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_H.ptr, d_R.ptr, d_G.ptr, 0, stream)),
+            ("dds_op", "dds_op", lambda: lib.bidmat_dds_plan(plan, k, d_W.ptr, d_H.ptr, d_ir.ptr, d_jc.ptr, d_v.ptr, 3, d_Q.ptr, 0, stream)),
+            ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_H.ptr, d_Q.ptr, d_G.ptr, 0, stream)),
         ]
-        workload = "configs[4]: NMF update chain R=DDS(W,H,V), Q=V./R, G=H*^Q (dense row sums timed apart)"
-        metric = "achieved HBM GB/s (algorithmic bytes) for the NMF update chain at k=128, ~400M nnz"
+        workload = "configs[4]: NMF update chain Q = V ./ DDS(W,H,V) (one fused launch), G = H *^ Q (dense row sums timed apart)"
+        metric = "algorithmic GB/s (gathered operand charged once per nonzero) for the NMF update chain at k=128, ~400M nnz"
         roof_op, roof_kernel = "dsmultT", "k_gather_axpy<W=4,V=1,LPN=32,plan>"
 
     def ev():
@@ -228,25 +264,38 @@ def main():
         avg = float(np.mean(t))
         per_op[name] = {
             "ms_avg": round(avg, 4), "ms_median": round(float(np.median(t)), 4), "ms_min": round(float(np.min(t)), 4),
-            "alg_GB": round(b / 1e9, 3),
-            "GBps": round(b / avg / 1e6, 1), "nnz_per_s": round(nnz / avg * 1e3, 1),
+            "alg_GB": round(b / 1e9, 3), "compulsory_GB": round(compulsory_bytes(kind, k, nnz, nrows, ncols) / 1e9, 3),
+            "alg_GBps": round(b / avg / 1e6, 1), "nnz_per_s": round(nnz / avg * 1e3, 1),
             "GFLOPs": round(flops(kind, k, nnz, ncols) / avg / 1e6, 1),
-            "frac_of_hbm_peak": round(b / avg / 1e6 / HBM_PEAK_GBS, 4),
+            "alg_frac_of_hbm_peak": round(b / avg / 1e6 / HBM_PEAK_GBS, 4),
         }
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
+    # ---- what bounds the roofline kernel, measured on this device in this run: the rate of the
+    # same gather kernel when the gathered rows fit in L2 (the ceiling of a kernel whose every gather
+    # is served by L2), and the plain streaming rate of the device.
+    live = live_rates(lib, stream, k, "dds" if roof_op in ("dds", "dds_op") else "dsmult")
     r_avg, r_bytes = per_op[roof_op]["ms_avg"], alg_bytes(roof_op, k, nnz, nrows, ncols)
+    r_comp = compulsory_bytes(roof_op, k, nnz, nrows, ncols)
+    gathered = nnz * 4 * k
+    bound_ms = max(r_comp / (HBM_PEAK_GBS * 1e9), gathered / (live["l2_resident_gather_GBps"] * 1e9)) * 1e3
+    traffic, traffic_src = measured_traffic(args.workload, roof_op, nnz)
     roofline = {
         "kernel": roof_kernel, "bound": "hbm", "achieved": round(r_bytes / r_avg / 1e6, 1), "peak": HBM_PEAK_GBS,
         "unit": "GB/s", "frac": round(r_bytes / r_avg / 1e6 / HBM_PEAK_GBS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, roof_op, nnz)),
+        "frac_basis": "ALGORITHMIC bytes / time / 8 TB/s: every gathered row is charged per nonzero although L1/L2 serve "
+                      "most of them, so this can exceed 1; the bounded utilisation figure is frac_of_bound",
+        "traffic": traffic, "traffic_source": traffic_src,
         "bytes_per_launch": r_bytes, "avg_launch_ms": round(r_avg, 4),
+        "compulsory_bytes": r_comp, "gathered_bytes": gathered,
+        "l2_resident_gather_GBps": live["l2_resident_gather_GBps"], "l2_resident_probe": live["probe"],
+        "stream_GBps": live["stream_GBps"],
+        "bound_ms": round(bound_ms, 4), "frac_of_bound": round(bound_ms / r_avg, 4),
+        "bound_basis": "max(compulsory bytes / 8 TB/s, gathered bytes / rate of the same kernel with an L2-resident operand)",
     }
-
-    if roofline["traffic"]:
-        # the kernel's measured HBM-side rate: the utilisation figure that cannot exceed 1
-        roofline["traffic_GBps"] = round(roofline["traffic"] / r_avg / 1e6, 1)
-        roofline["traffic_frac"] = round(roofline["traffic"] / r_avg / 1e6 / HBM_PEAK_GBS, 4)
+    if traffic:
+        # L2-miss (fabric-side) bytes over time: Infinity Cache and HBM together, not an HBM fraction
+        roofline["l2_miss_GBps"] = round(traffic / r_avg / 1e6, 1)
 
     out = {
         "metric": metric, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -255,7 +304,7 @@ def main():
         "config": {"workload": workload, "k": k, "nrows": nrows, "ncols": ncols, "nnz": nnz, "scale": args.scale},
         "nnz_per_s": round(len([o for o in ops if o[1] != "ewise"]) * nnz / (ms_per_step * 1e-3), 1),
         "GFLOPs": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),
-        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "alg_frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "ops": per_op, "roofline": roofline,
         "device": {"arch": arch.value.decode(), "compute_units": cus.value, "mem_GiB": round(mem.value / 2**30, 1)},
         "gen_s": round(t_gen, 2),
@@ -264,9 +313,12 @@ def main():
                 "GBps": round(h2d["bytes"] / h2d["s"] / 1e9, 2),
                 "step_GBps_incl_h2d": round(total_bytes / (ms_per_step * 1e-3 + h2d["s"]) / 1e9, 1)},
     }
-    if t_plan[0] is not None:
-        out["plan"] = {"first_build_ms": round(t_plan[0] * 1e3, 2), "build_ms": round(t_plan[1] * 1e3, 2), "segments": lib.bidmat_plan_segments(plan),
-                       "bytes": lib.bidmat_plan_bytes(plan)}
+    out["plan"] = {"first_build_ms": round(t_plan[0] * 1e3, 2), "build_ms": round(t_plan[1] * 1e3, 2),
+                   "segments": lib.bidmat_plan_segments(plan), "bytes": lib.bidmat_plan_bytes(plan),
+                   "column_overflow_segments": lib.bidmat_plan_overflow_segments(plan)}
+    if "dsmultT" in per_op:
+        # what a caller with a fresh pattern on every call (a BIDMach minibatch) pays for A*^S
+        per_op["dsmultT_incl_plan_ms"] = round(per_op["dsmultT"]["ms_avg"] + t_plan[1] * 1e3, 4)
     if args.workload == "C5":      # the dense row sums of H, timed apart from the chain
         e0, e1 = ev(), ev()
         hip_abi.check(lib.bidmat_reduce2op(k, ncols, d_H.ptr, d_rs.ptr, 0.0, 0))
@@ -279,6 +331,9 @@ def main():
         b = alg_bytes("rowsum", k, nnz, nrows, ncols)
         out["rowsum"] = {"ms_avg": round(t, 4), "GBps": round(b / t / 1e6, 1),
                          "frac_of_hbm_peak": round(b / t / 1e6 / HBM_PEAK_GBS, 4)}
+
+    # the outputs of the timed steps, checked below
+    results = {name: d.numpy() for name, d in outputs.items()} if not args.no_cpu else {}
 
     if args.workload == "headline":
         # What unchanged call sites get: the blocking entries with the reference's argument lists
@@ -323,8 +378,50 @@ def main():
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_sample)
+        checks = verify_outputs(args.workload, cfg, results)
+        for name, c in checks.items():
+            per_op[name].update(c)
+        out["verified"] = bool(checks) and all(c["max_err_measure"] <= 1e-4 for c in checks.values())
 
     print(json.dumps(out))
+    if not args.no_cpu and not out["verified"]:
+        print("bench.py: the timed outputs differ from the CPU oracle beyond 1e-4", file=sys.stderr)
+        sys.exit(1)
+
+
+def live_rates(lib, stream, k, op):
+    """Two reference rates of this device, measured with the library's own kernels:
+    the DDS / A*S kernel on 100 000 columns x 200 nonzeros whose rows are uniform over 2 MiB of the
+    gathered operand (half of one XCD's L2: every gather is an L2 hit, or an L1 hit), as algorithmic
+    gather bytes per second, and a streaming add over 3 x 256 MiB."""
+    from bidmat_amd import hip_abi
+    from bidmat_amd.device import DeviceArray
+    ncols, L = 100000, 200
+    R = max(16, (2 << 20) // (4 * k))
+    nnz = ncols * L
+    rng = np.random.default_rng(0)
+    d_A = DeviceArray.from_numpy(rng.random(k * R, dtype=np.float32))
+    d_B = DeviceArray.from_numpy(rng.random(k * ncols, dtype=np.float32))
+    d_v = DeviceArray.from_numpy(rng.random(nnz, dtype=np.float32))
+    d_jc = DeviceArray.from_numpy((np.arange(ncols + 1) * L).astype(np.int32))
+    d_ir = DeviceArray.from_numpy(rng.integers(0, R, size=nnz).astype(np.int32))
+    if op == "dds":
+        d_o = DeviceArray(nnz, np.float32)
+        fn = lambda: lib.bidmat_dds_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_o.ptr, 0, stream)
+    else:
+        d_o = DeviceArray(k * ncols, np.float32)
+        fn = lambda: lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_o.ptr, 0, stream)
+    t = _timed(lib, fn, stream, 5)
+    gather = nnz * 4.0 * k / t / 1e6
+    n = 1 << 26
+    s = [DeviceArray(n, np.float32) for _ in range(3)]
+    for x in s:
+        hip_abi.check(lib.bidmat_memset(x.ptr, 0, x.nbytes))
+    t2 = _timed(lib, lambda: lib.bidmat_applyop_flat(s[0].ptr, s[1].ptr, s[2].ptr, n, 0, stream), stream, 5)
+    for x in [d_A, d_B, d_v, d_jc, d_ir, d_o] + s:
+        x.free()
+    return {"l2_resident_gather_GBps": round(gather, 1), "stream_GBps": round(12.0 * n / t2 / 1e6, 1),
+            "probe": "%s kernel, k=%d, %d columns x %d nonzeros, rows uniform over %d rows (2 MiB), %.3f ms" % (op, k, ncols, L, R, t)}
 
 
 def _timed(lib, fn, stream, reps, warm=2):
@@ -502,6 +599,84 @@ def cpu_baseline(workload, cfg, frac):
         "seconds": {op: round(s, 3) for op, s in t.items()},
         "nnz_per_s": round(len([o for o in t if o != "ewise"]) * nnz / total_s, 1),
     }
+
+
+def _error_fields(x, ref64, sumabs):
+    """Pure relative error and the path's error measure min(|x-ref|/|ref|, |x-ref|/sum|terms|) of a
+    result against the fp64-accumulated CPU result, as maxima over all values."""
+    x = np.asarray(x, dtype=np.float64)
+    err = np.abs(x - ref64)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        rel = np.where(err == 0, 0.0, err / np.abs(ref64))
+        scaled = np.where(err == 0, 0.0, err / sumabs)
+    rel = np.where(np.isnan(rel), np.inf, rel)
+    measure = np.minimum(rel, np.where(np.isnan(scaled), np.inf, scaled))
+    return {"max_rel_err": float(rel.max(initial=0.0)), "max_err_measure": float(measure.max(initial=0.0)),
+            "checked_values": int(x.size)}
+
+
+def _sub_csc(ir, jc, vals, cols):
+    lens = jc[cols + 1] - jc[cols]
+    sjc = np.zeros(cols.size + 1, dtype=np.int32)
+    sjc[1:] = np.cumsum(lens)
+    idx = np.concatenate([np.arange(jc[c], jc[c + 1]) for c in cols]) if cols.size else np.zeros(0, np.int64)
+    return (vals[idx] if vals is not None else None), ir[idx], sjc, idx
+
+
+def _rows_sub_csc(ir, jc, vals, rows, nrows):
+    pos = np.full(nrows, -1, dtype=np.int64)
+    pos[rows] = np.arange(rows.size)
+    keep = np.flatnonzero(pos[ir] >= 0)
+    ic = np.searchsorted(jc, keep, side="right") - 1
+    sjc = np.zeros(jc.size, dtype=np.int32)
+    sjc[1:] = np.cumsum(np.bincount(ic, minlength=jc.size - 1))
+    return vals[keep], pos[ir[keep]].astype(np.int32), sjc
+
+
+def verify_outputs(workload, cfg, results):
+    """The outputs the timed steps left on the device against the CPU oracle's fp64-accumulated
+    results: every value for the headline workload and configs[0]; for the 40 M / 400 M-nonzero
+    workloads, whose full CPU results take minutes, all values of a random sample of columns (rows
+    for A*^S). Returns per op: max_rel_err, max_err_measure, checked_values."""
+    import oracle
+    k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
+    ir, jc, vals = cfg["ir"], cfg["jc"], cfg["vals"]
+    th = oracle.max_threads()
+    out = {}
+    rng = np.random.default_rng(0)
+    if workload == "headline":
+        ref, sa = oracle.dds_f64(cfg["A"], cfg["B"], k, ir, jc, nthreads=th)
+        out["dds"] = _error_fields(results["dds"], ref, sa)
+        ref, sa = oracle.fsmult_f64(cfg["A"], k, vals, ir, jc, nthreads=th)
+        out["dsmult"] = _error_fields(results["dsmult"], ref, sa)
+        ref, sa = oracle.fsmultT_f64(cfg["A_T"], k, nrows, vals, ir, jc, nthreads=th)
+        out["dsmultT"] = _error_fields(results["dsmultT"], ref, sa)
+    elif workload == "C1":
+        ref, sa = oracle.fsmult_f64(cfg["A"], k, vals, ir, jc, nthreads=th)
+        out["dsmult"] = _error_fields(results["dsmult"], ref, sa)
+    elif workload == "C4":
+        lens = np.diff(jc)
+        cols = np.unique(np.concatenate([rng.integers(0, ncols, 2000), np.argsort(lens)[-5:], [0, ncols - 1]]))
+        sv, sir, sjc, _ = _sub_csc(ir, jc, vals, cols)
+        ref, sa = oracle.fsmult_f64(cfg["A"], k, sv, sir, sjc, nthreads=th)
+        out["dsmult"] = _error_fields(results["dsmult"].reshape(ncols, k)[cols].ravel(), ref, sa)
+        out["dsmult"]["checked"] = "%d sampled columns incl. the 5 longest" % cols.size
+    else:   # C5: Q = V ./ DDS(W,H,V), G = H *^ Q
+        W, H = cfg["W"], cfg["H"]
+        Q, G = results["dds_op"], results["dsmultT"]
+        cols = np.unique(rng.integers(0, ncols, 2000))
+        sv, sir, sjc, idx = _sub_csc(ir, jc, vals, cols)
+        r64, sa = oracle.dds_f64(W, H.reshape(ncols, k)[cols].ravel(), k, sir, sjc, nthreads=th)
+        # all terms of R are positive: the error of Q = V/R relative to Q is the error of R relative to R
+        want = sv.astype(np.float64) / r64
+        out["dds_op"] = _error_fields(Q[idx], want, np.abs(want))
+        out["dds_op"]["checked"] = "%d sampled columns" % cols.size
+        rows = np.unique(np.concatenate([rng.integers(0, nrows, 500), [0, 1, nrows - 1]]))
+        rv, rir, rjc = _rows_sub_csc(ir, jc, Q, rows, nrows)
+        ref, sa = oracle.fsmultT_f64(H, k, rows.size, rv, rir, rjc, nthreads=th)
+        out["dsmultT"] = _error_fields(G.reshape(nrows, k)[rows].ravel(), ref, sa)
+        out["dsmultT"]["checked"] = "%d sampled rows, fed with the device's own Q" % rows.size
+    return out
 
 
 if __name__ == "__main__":
