@@ -481,6 +481,30 @@ API int bidmat_csc_expand_cols(int ncols, int nnz, const int* Sjc, int* Sic, voi
     return (int)bm::csc_expand_cols(ncols, nnz, Sjc, Sic, as_stream(stream));
 }
 
+API int bidmat_csc_implicit_rows(int ncols, int nnz, const int* Sjc, int* Sir, void* stream) {
+    if (ncols < 0 || nnz < 0) return kInvalid;
+    if (nnz == 0) return 0;
+    if (!Sjc || !Sir) return kInvalid;
+    return (int)bm::csc_implicit_rows(ncols, nnz, Sjc, Sir, as_stream(stream));
+}
+
+API int bidmat_csc_validate(int nrows, int ncols, int nnz, const int* Sir, const int* Sjc, int* rule) {
+    auto lock = bm::device_lock();
+    if (!rule) return kInvalid;
+    *rule = 0;
+    if (nrows < 0 || ncols < 0 || nnz < 0 || !Sjc) return kInvalid;
+    hipError_t err;
+    int* d_flags = (int*)bm::ws_get(bm::WS_MISC, 64, &err);
+    if (!d_flags) return (int)err;
+    err = bm::csc_validate(nrows, ncols, nnz, Sir, Sjc, d_flags, nullptr);
+    int flags = 0;
+    if (err == hipSuccess) err = hipMemcpy(&flags, d_flags, sizeof(int), hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return (int)err;
+    for (int r = 1; r <= 6; ++r)
+        if (flags & (1 << r)) { *rule = r; break; }
+    return 0;
+}
+
 API int bidmat_csc_colslice_range(int ncols, int col1, int col2, const int* Sjc, int* start, int* nnz) {
     if (ncols < 0 || col1 < 0 || col2 < col1 || col2 > ncols || !Sjc || !start || !nnz) return kInvalid;
     int lo = 0, hi = 0;

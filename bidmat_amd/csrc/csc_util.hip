@@ -6,15 +6,43 @@
 namespace bm {
 namespace {
 
-// 16 lanes per column: lane l writes ic[jc[c] + l], + 16, ...
-__global__ __launch_bounds__(BM_BLOCK) void k_expand_cols(int ncols, const int* __restrict__ jc,
-                                                          int* __restrict__ ic) {
+// 16 lanes per column: lane l writes ic[jc[c] + l], + 16, ... Positions outside [0, nnz) are never
+// written, whatever a malformed jc says. ROWS: instead of the column index, the position inside the
+// column (the implied row of a sparse matrix stored without row indices).
+template <bool ROWS>
+__global__ __launch_bounds__(BM_BLOCK) void k_expand_cols(int ncols, int nnz, const int* __restrict__ jc,
+                                                          int* __restrict__ out) {
     const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long c = t >> 4;
     const int l = (int)(t & 15);
     if (c >= ncols) return;
-    const int s = jc[c], e = jc[c + 1];
-    for (int j = s + l; j < e; j += 16) ic[j] = (int)c;
+    int s = jc[c], e = jc[c + 1];
+    if (s < 0) s = 0;
+    if (e > nnz) e = nnz;
+    for (long long j = (long long)s + l; j < e; j += 16) out[j] = ROWS ? (int)(j - s) : (int)c;
+}
+
+// What the kernels rely on: jc[0] == 0, jc non-decreasing inside [0, nnz], jc[ncols] == nnz,
+// 0 <= ir < nrows. Sets bit r of *flags for every violated rule r (numbered like the branches of
+// SparseMat.check: 1 first pointer, 2 pointer order, 5 row out of range, 6 last pointer).
+__global__ __launch_bounds__(BM_BLOCK) void k_csc_validate(int nrows, int ncols, int nnz, const int* __restrict__ ir,
+                                                           const int* __restrict__ jc, int* __restrict__ flags) {
+    long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    const long long lim = nnz > ncols + 1 ? nnz : (long long)ncols + 1;
+    int bad = 0;
+    for (; i < lim; i += stride) {
+        if (i <= ncols) {
+            const int v = jc[i];
+            if (i == 0 && v != 0) bad |= 1 << 1;
+            if (v < 0 || v > nnz || (i < ncols && v > jc[i + 1])) bad |= 1 << 2;
+            if (i == ncols && v != nnz) bad |= 1 << 6;
+        }
+        if (i < nnz && ir != nullptr) {
+            if ((unsigned)ir[i] >= (unsigned)nrows) bad |= 1 << 5;
+        }
+    }
+    if (bad) atomicOr(flags, bad);
 }
 
 // Thread j fills jc for every column that starts at position j:
@@ -182,7 +210,23 @@ hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream
     long long threads = (long long)ncols * 16;
     long long nblk = (threads + BM_BLOCK - 1) / BM_BLOCK;
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(k_expand_cols, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, jc, ic);
+    hipLaunchKernelGGL(k_expand_cols<false>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nnz, jc, ic);
+    return hipGetLastError();
+}
+
+hipError_t csc_implicit_rows(int ncols, int nnz, const int* jc, int* ir, hipStream_t s) {
+    if (ncols <= 0 || nnz <= 0) return hipSuccess;
+    long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_expand_cols<true>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nnz, jc, ir);
+    return hipGetLastError();
+}
+
+hipError_t csc_validate(int nrows, int ncols, int nnz, const int* ir, const int* jc, int* d_flags, hipStream_t s) {
+    hipError_t e = fill_i32(d_flags, 1, 0, s);
+    if (e != hipSuccess) return e;
+    const long long lim = nnz > ncols + 1 ? nnz : (long long)ncols + 1;
+    hipLaunchKernelGGL(k_csc_validate, dim3(grid_for(lim, 4096)), dim3(BM_BLOCK), 0, s, nrows, ncols, nnz, ir, jc, d_flags);
     return hipGetLastError();
 }
 

@@ -13,6 +13,11 @@ int opt_heavy_min();   // a row is cut by panels when it averages at least this 
 // ---- CSC utilities (csc_util.hip)
 hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);
 hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStream_t s);
+// ir[j] = j - jc[c]: the implied rows of a sparse matrix stored without row indices
+hipError_t csc_implicit_rows(int ncols, int nnz, const int* jc, int* ir, hipStream_t s);
+// *d_flags (device int) = bit set of violated rules: 1 jc[0] != 0, 2 jc decreasing or outside
+// [0, nnz], 5 a row index outside [0, nrows), 6 jc[ncols] != nnz. ir may be nullptr (rows not checked).
+hipError_t csc_validate(int nrows, int ncols, int nnz, const int* ir, const int* jc, int* d_flags, hipStream_t s);
 // columns [col1, col1+nc) with n nonzeros starting at position `start`: out_jc (nc+1, rebased),
 // out_ir / out_data (n), out_ic (n, nullable)
 hipError_t csc_colslice(int nc, int start, int n, const int* jc_at_col1, const int* ir, const float* data,

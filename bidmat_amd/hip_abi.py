@@ -46,6 +46,8 @@ SIGNATURES = {
     "bidmat_spsum_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, C.c_int, vp]),
     "bidmat_spsum_rows_plan": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "bidmat_csc_expand_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
+    "bidmat_csc_implicit_rows": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
+    "bidmat_csc_validate": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, C.POINTER(C.c_int)]),
     "bidmat_csc_colslice_range": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "bidmat_csc_colslice": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, vp, vp, vp]),
     "bidmat_csc_transpose": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, vp]),

@@ -281,6 +281,91 @@ GMatP GMat::reduceOp(GMatP oldmat, int dir, float initval, int op) {
     fail("dimension must be 1 or 2");
 }
 
+// ------------------------------------------------------------------ pinned staging
+Staging::Staging(size_t chunk_bytes) : chunk_(chunk_bytes) {
+    int err = bidmat_stream_create(&stream_);
+    for (int i = 0; i < 2 && err == 0; ++i) {
+        err = bidmat_host_alloc(&stage_[i], (long long)chunk_);
+        if (err == 0) err = bidmat_event_create(&ev_[i]);
+    }
+    if (err != 0) {
+        const std::string msg = std::string("HIP error creating staging buffers ") + bidmat_error_string(err);
+        this->~Staging();
+        fail(msg);
+    }
+}
+
+Staging::~Staging() {
+    if (stream_) bidmat_stream_synchronize(stream_);
+    for (int i = 0; i < 2; ++i) {
+        if (stage_[i]) bidmat_host_free(stage_[i]);
+        if (ev_[i]) bidmat_event_destroy(ev_[i]);
+        stage_[i] = ev_[i] = nullptr;
+    }
+    if (stream_) bidmat_stream_destroy(stream_);
+    stream_ = nullptr;
+}
+
+void Staging::upload(void* dst, size_t bytes, const std::function<void(void*, size_t)>& fill) {
+    char* d = static_cast<char*>(dst);
+    while (bytes > 0) {
+        const size_t n = bytes < chunk_ ? bytes : chunk_;
+        if (busy_[which_]) hipcheck(bidmat_event_synchronize(ev_[which_]), "staging wait");
+        fill(stage_[which_], n);
+        hipcheck(bidmat_memcpy_h2d_async(d, stage_[which_], (long long)n, stream_), "staged upload");
+        hipcheck(bidmat_event_record(ev_[which_], stream_), "staging event");
+        busy_[which_] = true;
+        which_ ^= 1;
+        d += n;
+        bytes -= n;
+    }
+}
+
+void Staging::upload(void* dst, const void* src, size_t bytes) {
+    const char* p = static_cast<const char*>(src);
+    upload(dst, bytes, [&p](void* buf, size_t n) { memcpy(buf, p, n); p += n; });
+}
+
+void Staging::download(void* dst, const void* src, size_t bytes, int add) {
+    // the copy into buffer b is enqueued one step ahead of the host draining buffer b^1
+    char* out = static_cast<char*>(dst);
+    const char* s = static_cast<const char*>(src);
+    wait();
+    size_t pending[2] = {0, 0};
+    char* where[2] = {nullptr, nullptr};
+    auto drain = [&](int b) {
+        if (!pending[b]) return;
+        hipcheck(bidmat_event_synchronize(ev_[b]), "staging wait");
+        if (add == 0) {
+            memcpy(where[b], stage_[b], pending[b]);
+        } else {
+            const int* in = static_cast<const int*>(stage_[b]);
+            int* o = reinterpret_cast<int*>(where[b]);
+            for (size_t i = 0; i < pending[b] / sizeof(int); ++i) o[i] = in[i] + add;
+        }
+        pending[b] = 0;
+    };
+    int b = 0;
+    while (bytes > 0) {
+        const size_t n = bytes < chunk_ ? bytes : chunk_;
+        drain(b);
+        hipcheck(bidmat_memcpy_d2h_async(stage_[b], s, (long long)n, stream_), "staged download");
+        hipcheck(bidmat_event_record(ev_[b], stream_), "staging event");
+        pending[b] = n;
+        where[b] = out;
+        out += n; s += n; bytes -= n;
+        b ^= 1;
+    }
+    drain(b);
+    drain(b ^ 1);
+    busy_[0] = busy_[1] = false;
+}
+
+void Staging::wait() {
+    hipcheck(bidmat_stream_synchronize(stream_), "staging sync");
+    busy_[0] = busy_[1] = false;
+}
+
 // ------------------------------------------------------------------ GSMat
 PlanHolder::~PlanHolder() {
     if (plan) bidmat_plan_destroy(plan);
@@ -348,44 +433,55 @@ GSMatP GSMat::newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP outma
 }
 
 GSMatP GSMat::fromSMat(const SMat& a, GSMatP b) {
-    GSMatP out = newOrCheckGSMat(a.nrows, a.ncols, a.nnz(), a.nnz(), b, a.GUID, 0, 0, opHash("fromSMat"));
-    out->nnz0 = a.nnz();
+    return fromHost(a.nrows, a.ncols, a.nnz(), a.data.data(), a.ir.data(), a.jc.data(), Mat::ioneBased, b, a.GUID);
+}
+
+// Upload of a host CSC matrix (GSMat.scala:620-647). The three arrays cross PCIe through pinned
+// staging buffers with asynchronous copies; the index base is converted and the per-nonzero column
+// indices are made on the device (the reference shifts in host loops and calls cusparseXcsr2coo,
+// GSMat.scala:626-639); the pattern is checked on the device before any kernel trusts it.
+GSMatP GSMat::fromHost(int nr, int nc, int n, const float* data, const int* ir, const int* jc, int ioff, GSMatP b,
+                       long long guid) {
+    if (guid == 0) guid = Mat::newGUID();                  // bare arrays: never share a cached output
+    GSMatP out = newOrCheckGSMat(nr, nc, n, n, b, guid, 0, 0, opHash("fromSMat"));
+    out->nnz0 = n;
     out->planHolder = std::make_shared<PlanHolder>();      // new pattern: any older plan is stale
-    const int n = a.nnz();
-    hipcheck(bidmat_memcpy_h2d(out->pdata, a.data.data(), (long long)sizeof(float) * n), "copy error in GSMat.fromSMat");
-    hipcheck(bidmat_memcpy_h2d(out->pir, a.ir.data(), (long long)sizeof(int) * n), "copy error in GSMat.fromSMat");
-    hipcheck(bidmat_memcpy_h2d(out->pjc, a.jc.data(), (long long)sizeof(int) * (a.ncols + 1)), "copy error in GSMat.fromSMat");
-    if (Mat::ioneBased == 1) {   // device indices are always 0-based (GSMat.scala:626-632); shifted on the device
-        hipcheck(bidmat_index_shift(out->pir, n, -1, nullptr), "GSMat.fromSMat");
-        hipcheck(bidmat_index_shift(out->pjc, (long long)a.ncols + 1, -1, nullptr), "GSMat.fromSMat");
+    Staging st;
+    st.upload(out->pjc, jc, sizeof(int) * ((size_t)nc + 1));
+    st.upload(out->pir, ir, sizeof(int) * (size_t)n);
+    st.upload(out->pdata, data, sizeof(float) * (size_t)n);
+    if (ioff != 0) {             // device indices are always 0-based (GSMat.scala:626-632)
+        hipcheck(bidmat_index_shift(out->pir, n, -ioff, st.stream()), "GSMat.fromSMat");
+        hipcheck(bidmat_index_shift(out->pjc, (long long)nc + 1, -ioff, st.stream()), "GSMat.fromSMat");
     }
-    // per-nonzero column indices (the reference calls cusparseXcsr2coo here, GSMat.scala:639)
-    int err = bidmat_csc_expand_cols(out->ncols, n, out->pjc, out->pic, nullptr);
+    st.wait();
+    int rule = 0;
+    hipcheck(bidmat_csc_validate(nr, nc, n, out->pir, out->pjc, &rule), "GSMat.fromSMat");
+    if (rule != 0) fail(fmt("GSMat.fromSMat: malformed sparse matrix (SparseMat.check rule %d)", rule));
+    int err = bidmat_csc_expand_cols(nc, n, out->pjc, out->pic, nullptr);
     if (err == 0) err = bidmat_stream_synchronize(nullptr);
     if (err != 0) fail(std::string("HIP error in GSMat.fromSMat ") + bidmat_error_string(err));
     return out;
 }
 
+// Download (GSMat.scala:108-127). The reference downloads the per-nonzero column indices and
+// compresses them on the host; the device already holds the column pointer, which is 200 times
+// smaller, so that is what crosses PCIe. The index base is added while the staging buffers are drained.
 SMat GSMat::toSMat() const {
     SMat out(nrows, ncols, nnz0);
-    std::vector<int> tmpcols((size_t)nnz0);
-    hipcheck(bidmat_memcpy_d2h(out.ir.data(), pir, (long long)sizeof(int) * nnz0), "HIP error in GSMat.toSMat");
-    hipcheck(bidmat_memcpy_d2h(out.data.data(), pdata, (long long)sizeof(float) * nnz0), "HIP error in GSMat.toSMat");
-    hipcheck(bidmat_memcpy_d2h(tmpcols.data(), pic, (long long)sizeof(int) * nnz0), "HIP error in GSMat.toSMat");
-    // SparseMat.compressInds (SparseMat.scala:857-868)
     const int ioff = Mat::ioneBased;
-    out.jc[0] = ioff;
-    int j = 0;
-    for (int i = 0; i < ncols; ++i) {
-        while (j < nnz0 && tmpcols[j] <= i) ++j;
-        out.jc[i + 1] = j + ioff;
-    }
-    if (ioff == 1) for (auto& v : out.ir) v += 1;
+    Staging st;
+    st.download(out.jc.data(), pjc, sizeof(int) * ((size_t)ncols + 1), ioff);
+    st.download(out.ir.data(), pir, sizeof(int) * (size_t)nnz0, ioff);
+    st.download(out.data.data(), pdata, sizeof(float) * (size_t)nnz0);
     return out;
 }
 
 GMatP GSMat::contents() {
     auto out = std::make_shared<GMat>(nnz0, 1, pdata, realnnz, false);
+    // the view does not own pdata: it keeps this matrix alive for as long as it exists
+    // (matrices made with GSMat::make are always held by a shared_ptr)
+    out->keepalive = weak_from_this().lock();
     return out;
 }
 

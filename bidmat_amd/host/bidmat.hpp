@@ -12,6 +12,7 @@
 #pragma once
 #include <atomic>
 #include <map>
+#include <functional>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -62,6 +63,32 @@ public:
     void check() const;
     FMat full() const;
     std::string mytype() const { return "SMat"; }
+};
+
+// Transfers between pageable host memory and the device through two pinned staging buffers and
+// asynchronous copies on a stream of their own: while one buffer crosses PCIe the other is being
+// filled (upload) or emptied (download). Used by GSMat.fromSMat / toSMat and HMat.loadGSMat.
+class Staging {
+public:
+    explicit Staging(size_t chunk_bytes = size_t(8) << 20);
+    ~Staging();
+    Staging(const Staging&) = delete;
+    Staging& operator=(const Staging&) = delete;
+    // dst (device) <- bytes produced by fill(staging_buffer, n) in chunks
+    void upload(void* dst, size_t bytes, const std::function<void(void*, size_t)>& fill);
+    // dst (device) <- src (host)
+    void upload(void* dst, const void* src, size_t bytes);
+    // dst (host) <- src (device); add != 0: the data are int32 and `add` is added on the way
+    void download(void* dst, const void* src, size_t bytes, int add = 0);
+    void* stream() const { return stream_; }
+    void wait();                      // until everything enqueued so far is complete
+private:
+    size_t chunk_;
+    void* stage_[2] = {nullptr, nullptr};
+    void* ev_[2] = {nullptr, nullptr};
+    bool busy_[2] = {false, false};
+    int which_ = 0;
+    void* stream_ = nullptr;
 };
 
 class GSMat;
@@ -118,7 +145,7 @@ struct PlanHolder {
 };
 
 // ---- device sparse (GSMat): pir/pic/pjc/pdata, all 0-based on the device
-class GSMat {
+class GSMat : public std::enable_shared_from_this<GSMat> {
 public:
     int nrows, ncols;
     int nnz0;
@@ -137,6 +164,9 @@ public:
     std::string mytype() const { return "GSMat"; }
     static GSMatP make(int nr, int nc, int nnz, int realnnz);
     static GSMatP fromSMat(const SMat& a, GSMatP b = nullptr);   // GSMat.scala:620-647
+    // the same from bare host arrays in index base ioff (what fromSMat does with a.data / a.ir / a.jc)
+    static GSMatP fromHost(int nr, int nc, int nnz, const float* data, const int* ir, const int* jc, int ioff,
+                           GSMatP b = nullptr, long long guid = 0);
     // oneHot (n = 1) / nHot: cats is an n x ncols category matrix (column-major, 0-based);
     // ncats0 == 0: rows = largest category + 1  (GSMat.scala:686-720)
     static GSMatP nHot(const std::vector<int>& cats, int n, int ncols, int ncats0);
@@ -176,15 +206,19 @@ GMatP sum(const GMatP& a, int n = 0, GMatP omat = nullptr);       // GFunctions.
 
 // ---- matrix files (HMat.scala): little-endian int32 header [type, nrows, ncols, nnz], then
 // for a sparse float matrix (type 231) jc[ncols+1], ir[nnz], data[nnz] with 0-based indices on
-// disk (HMat.scala:1232-1266, 1444-1480); for a dense float matrix (type 130) the column-major
+// disk (HMat.scala:1232-1266, 1444-1480); type 331 is the same without ir (HMat.scala:1246-1258):
+// the j-th stored element of a column sits in row j (SparseMat.explicitInds, SparseMat.scala:79-93),
+// and the loaders make those rows explicit; for a dense float matrix (type 130) the column-major
 // floats (HMat.scala:337-399, 876-891). Names ending in .gz are gzip streams; .lz4 is refused.
 namespace HMat {
 SMat loadSMat(const std::string& fname);
 void saveSMat(const std::string& fname, const SMat& m);
 FMat loadFMat(const std::string& fname);
 void saveFMat(const std::string& fname, const FMat& m);
-// Reads a type-231 file straight into a GSMat: chunks go through two pinned staging buffers and
-// asynchronous copies, so reading the file and crossing PCIe overlap.
+// Reads a type-231 / 331 file straight into a GSMat: chunks go through two pinned staging buffers
+// and asynchronous copies, so reading the file and crossing PCIe overlap. The pattern is checked on
+// the device (column pointers in order and inside the file's nnz, rows inside the matrix) before
+// any kernel trusts it; a malformed file throws.
 GSMatP loadGSMat(const std::string& fname);
 }  // namespace HMat
 

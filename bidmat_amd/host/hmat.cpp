@@ -64,13 +64,22 @@ struct Writer {
     }
 };
 
-void read_sparse_header(Reader& r, int& nrows, int& ncols, int& nnz) {
+// norows: type 331, the file holds no row indices (HMat.scala:1246-1258)
+void read_sparse_header(Reader& r, int& nrows, int& ncols, int& nnz, bool& norows) {
     int h[4];
     r.read(h, sizeof h, "header");
-    if (h[0] == 331) fail("loadSMat: type 331 (sparse without row indices) is not supported on this path");
-    if (h[0] != 231) fail("loadSMat expected type field 231 or 331 but was " + std::to_string(h[0]));
+    if (h[0] != 231 && h[0] != 331) fail("loadSMat expected type field 231 or 331 but was " + std::to_string(h[0]));
+    norows = h[0] == 331;
     nrows = h[1]; ncols = h[2]; nnz = h[3];
     if (nrows < 0 || ncols < 0 || nnz < 0) fail("loadSMat: negative dimensions in header");
+}
+
+// jc as read from a file (0-based): first pointer 0, non-decreasing, last pointer nnz
+void check_file_jc(const int* jc, int ncols, int nnz) {
+    if (jc[0] != 0) fail("loadSMat: malformed file, jc(0) should be 0");
+    for (int i = 0; i < ncols; ++i)
+        if (jc[i] > jc[i + 1]) fail("loadSMat: malformed file, jc(i) out of order " + std::to_string(i));
+    if (jc[ncols] != nnz) fail("loadSMat: malformed file, jc(ncols) should be " + std::to_string(nnz));
 }
 
 }  // namespace
@@ -78,10 +87,24 @@ void read_sparse_header(Reader& r, int& nrows, int& ncols, int& nnz) {
 SMat loadSMat(const std::string& fname) {
     Reader r(fname);
     int nrows, ncols, nnz;
-    read_sparse_header(r, nrows, ncols, nnz);
+    bool norows;
+    read_sparse_header(r, nrows, ncols, nnz, norows);
     SMat out(nrows, ncols, nnz);
     r.read(out.jc.data(), sizeof(int) * ((size_t)ncols + 1), "jc");
-    r.read(out.ir.data(), sizeof(int) * (size_t)nnz, "ir");
+    check_file_jc(out.jc.data(), ncols, nnz);
+    if (!norows) {
+        r.read(out.ir.data(), sizeof(int) * (size_t)nnz, "ir");
+        for (int j = 0; j < nnz; ++j)
+            if ((unsigned)out.ir[j] >= (unsigned)nrows) fail("loadSMat: malformed file, ir(" + std::to_string(j) + ") out of range");
+    } else {
+        // the rows such a matrix implies: element j of a column sits in row j. (The reference's
+        // SparseMat.explicitInds means this too; its inner loop bound, SparseMat.scala:86, stops after
+        // one element per column.)
+        for (int c = 0; c < ncols; ++c) {
+            if (out.jc[c + 1] - out.jc[c] > nrows) fail("loadSMat: malformed file, column longer than the matrix is tall");
+            for (int j = out.jc[c]; j < out.jc[c + 1]; ++j) out.ir[j] = j - out.jc[c];
+        }
+    }
     r.read(out.data.data(), sizeof(float) * (size_t)nnz, "data");
     if (Mat::ioneBased == 1) {          // files are 0-based, host matrices carry Mat.ioneBased
         for (auto& v : out.jc) v += 1;
@@ -130,53 +153,33 @@ void saveFMat(const std::string& fname, const FMat& m) {
 GSMatP loadGSMat(const std::string& fname) {
     Reader r(fname);
     int nrows, ncols, nnz;
-    read_sparse_header(r, nrows, ncols, nnz);
+    bool norows;
+    read_sparse_header(r, nrows, ncols, nnz, norows);
     GSMatP out = GSMat::make(nrows, ncols, nnz, nnz);
-    // two pinned staging buffers: while one is on its way to the device the other is being read
-    const size_t chunk = 8u << 20;
-    void* stage[2] = {nullptr, nullptr};
-    void* ev[2] = {nullptr, nullptr};
-    void* stream = nullptr;
-    auto cleanup = [&] {
-        for (int i = 0; i < 2; ++i) {
-            if (stage[i]) bidmat_host_free(stage[i]);
-            if (ev[i]) bidmat_event_destroy(ev[i]);
-        }
-        if (stream) bidmat_stream_destroy(stream);
-    };
-    try {
-        auto ok = [](int e, const char* what) { if (e != 0) fail(std::string(what) + " " + bidmat_error_string(e)); };
-        ok(bidmat_stream_create(&stream), "stream");
-        for (int i = 0; i < 2; ++i) {
-            ok(bidmat_host_alloc(&stage[i], (long long)chunk), "pinned alloc");
-            ok(bidmat_event_create(&ev[i]), "event");
-        }
-        bool busy[2] = {false, false};
-        int which = 0;
-        auto upload = [&](void* dst, size_t bytes, const char* what) {
-            char* d = static_cast<char*>(dst);
-            while (bytes > 0) {
-                const size_t n = bytes < chunk ? bytes : chunk;
-                if (busy[which]) ok(bidmat_event_synchronize(ev[which]), "event wait");
-                r.read(stage[which], n, what);
-                ok(bidmat_memcpy_h2d_async(d, stage[which], (long long)n, stream), "async copy");
-                ok(bidmat_event_record(ev[which], stream), "event record");
-                busy[which] = true;
-                which ^= 1;
-                d += n;
-                bytes -= n;
-            }
-        };
-        upload(out->pjc, sizeof(int) * ((size_t)ncols + 1), "jc");      // files are 0-based, like the device
-        upload(out->pir, sizeof(int) * (size_t)nnz, "ir");
-        upload(out->pdata, sizeof(float) * (size_t)nnz, "data");
-        ok(bidmat_csc_expand_cols(ncols, nnz, out->pjc, out->pic, stream), "expand cols");
-        ok(bidmat_stream_synchronize(stream), "sync");
-    } catch (...) {
-        cleanup();
-        throw;
+    auto ok = [](int e, const char* what) { if (e != 0) fail(std::string(what) + " " + bidmat_error_string(e)); };
+    Staging st;
+    const char* what = "jc";
+    auto from_file = [&](void* buf, size_t n) { r.read(buf, n, what); };
+    st.upload(out->pjc, sizeof(int) * ((size_t)ncols + 1), from_file);      // files are 0-based, like the device
+    if (!norows) {
+        what = "ir";
+        st.upload(out->pir, sizeof(int) * (size_t)nnz, from_file);
     }
-    cleanup();
+    what = "data";
+    st.upload(out->pdata, sizeof(float) * (size_t)nnz, from_file);
+    st.wait();
+    // nothing on the device has used the arrays yet: check them before the first kernel does
+    int rule = 0;
+    ok(bidmat_csc_validate(nrows, ncols, nnz, norows ? nullptr : out->pir, out->pjc, &rule), "validate");
+    if (rule != 0) fail("loadGSMat: malformed file (SparseMat.check rule " + std::to_string(rule) + "): " + fname);
+    if (norows) ok(bidmat_csc_implicit_rows(ncols, nnz, out->pjc, out->pir, nullptr), "implicit rows");
+    ok(bidmat_csc_expand_cols(ncols, nnz, out->pjc, out->pic, nullptr), "expand cols");
+    ok(bidmat_stream_synchronize(nullptr), "sync");
+    if (norows) {
+        // a column of such a file may not be longer than the matrix is tall
+        ok(bidmat_csc_validate(nrows, ncols, nnz, out->pir, out->pjc, &rule), "validate");
+        if (rule != 0) fail("loadGSMat: malformed file, column longer than the matrix is tall: " + fname);
+    }
     return out;
 }
 

@@ -50,13 +50,7 @@ API int bmh_gmat_to_host(void* h, float* out) {
 
 // host arrays carry the index base Mat::ioneBased, exactly like a host SMat
 API void* bmh_gsmat_from_host(int nr, int nc, int nnz, const float* data, const int* ir, const int* jc) {
-    return guard_ptr([&] {
-        SMat a(nr, nc, nnz);
-        memcpy(a.data.data(), data, sizeof(float) * (size_t)nnz);
-        memcpy(a.ir.data(), ir, sizeof(int) * (size_t)nnz);
-        memcpy(a.jc.data(), jc, sizeof(int) * ((size_t)nc + 1));
-        return wrap(GSMat::fromSMat(a));
-    });
+    return guard_ptr([&] { return wrap(GSMat::fromHost(nr, nc, nnz, data, ir, jc, Mat::ioneBased)); });
 }
 API int bmh_gsmat_dims(void* h, int* nr, int* nc, int* nnz) {
     *nr = S(h)->nrows; *nc = S(h)->ncols; *nnz = S(h)->nnz();
@@ -114,7 +108,7 @@ API void* bmh_reduce(void* a, void* out, int dir, float initv, int op) {
     return guard_ptr([&] { return wrap(G(a)->reduceOp(G(out), dir, initv, op)); });
 }
 API void* bmh_gop(void* a, void* b, void* out, int op) { return guard_ptr([&] { return wrap(G(a)->gOp(G(b), G(out), op)); }); }
-API void* bmh_contents(void* s) { return guard_ptr([&] { GMatP v = S(s)->contents(); v->keepalive = S(s); return wrap(v); }); }
+API void* bmh_contents(void* s) { return guard_ptr([&] { return wrap(S(s)->contents()); }); }
 API void* bmh_with_values(void* s, void* vals) { return guard_ptr([&] { return wrap(S(s)->withValues(G(vals))); }); }
 
 // ---- matrix files (host arrays carry Mat::ioneBased)

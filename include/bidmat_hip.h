@@ -204,6 +204,15 @@ int bidmat_spsum_rows_plan(bidmat_plan *plan, const float *Sdata, float *out, in
 /* jc[ncols+1] -> ic[nnz] (per-nonzero column index).  Replaces cusparseXcsr2coo at
  * GSMat.scala:639.  Enqueues on stream. */
 int bidmat_csc_expand_cols(int ncols, int nnz, const int *Sjc, int *Sic, void *stream);
+/* ir[j] = j - jc[c] for every nonzero j of column c: the row indices a sparse matrix stored
+ * WITHOUT row indices implies (BIDMat file type 331, HMat.scala:1246-1258; SparseMat.explicitInds,
+ * SparseMat.scala:79-93).  Enqueues on stream. */
+int bidmat_csc_implicit_rows(int ncols, int nnz, const int *Sjc, int *Sir, void *stream);
+/* Checks a device CSC pattern before kernels trust it: *rule = 0 when it is sound, otherwise the
+ * first violated rule, numbered like the branches of SparseMat.check (SparseMat.scala:710-740):
+ * 1 jc[0] != 0, 2 jc decreasing or outside [0, nnz], 5 a row index outside [0, nrows),
+ * 6 jc[ncols] != nnz.  Rows need not be sorted or unique.  Sir may be NULL.  Blocking. */
+int bidmat_csc_validate(int nrows, int ncols, int nnz, const int *Sir, const int *Sjc, int *rule);
 /* Transpose of a device CSC matrix (nrows x ncols, nnz nonzeros) without leaving the device:
  * out_jc (nrows+1), out_ir (nnz: the original columns, ascending inside every output column),
  * out_data (nnz).  The reference's GSMat.t downloads, transposes on the host and uploads
