@@ -21,7 +21,11 @@ namespace {
 std::atomic<int> g_seglen{1024};
 std::atomic<int> g_panel_kb{3072};
 std::atomic<int> g_heavy_min{8};
+std::atomic<int> g_col_classes{-1};
+std::atomic<int> g_class_strip{16};
 }  // namespace
+int opt_class_strip() { return g_class_strip.load(std::memory_order_relaxed); }
+int opt_col_classes() { return g_col_classes.load(std::memory_order_relaxed); }
 int opt_heavy_min() { return g_heavy_min.load(std::memory_order_relaxed); }
 int opt_seglen() { return g_seglen.load(std::memory_order_relaxed); }
 int opt_panel_kb() { return g_panel_kb.load(std::memory_order_relaxed); }
@@ -56,6 +60,9 @@ PlanRef own(bidmat_plan* p) { return PlanRef(p, [](bidmat_plan* q) { (void)bm::p
 std::mutex g_cache_mu;
 std::list<CacheEntry> g_cache;          // most recently used first
 constexpr size_t kMaxCachedPlans = 4;
+// the class-ordered DDS kernel walks a column's class in one wave: very long columns stay with the
+// segment-splitting kernel
+constexpr int kMaxClassedColumn = 1 << 16;
 
 hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_hint, PlanRef* out) {
     out->reset();
@@ -398,6 +405,8 @@ API int bidmat_dds_plan(bidmat_plan* plan, int k, const float* A, const float* B
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (plan->ncols == 0 || plan->nnz == 0) return 0;
     if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
+    if (plan->ncls == 8 && k > 0 && plan->maxlen <= kMaxClassedColumn)
+        return (int)bm::dds_classed(k, plan->ncols, A, B, plan->cir, plan->cperm, plan->cptr, P, beta, as_stream(stream), V, opn);
     const bm::ColTable tab = col_table(plan);
     return (int)bm::dds_csc(k, plan->ncols, plan->nnz, A, B, Sir, Sjc, P, beta, as_stream(stream), V, opn, &tab);
 }
@@ -735,6 +744,16 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_heavy_min.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "class_strip")) {
+        if (value < 1 || value > 64) return kInvalid;
+        bm::g_class_strip.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "col_classes")) {
+        if (value < -1 || value > 1) return kInvalid;
+        bm::g_col_classes.store((int)value);
+        return 0;
+    }
     return kInvalid;
 }
 
@@ -743,7 +762,9 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "seglen")) return bm::opt_seglen();
     if (!strcmp(name, "panel_kb")) return bm::opt_panel_kb();
     if (!strcmp(name, "heavy_min")) return bm::opt_heavy_min();
-    return -1;
+    if (!strcmp(name, "col_classes")) return bm::opt_col_classes();
+    if (!strcmp(name, "class_strip")) return bm::opt_class_strip();
+    return -2;
 }
 
 API int bidmat_release_caches(void) {

@@ -34,6 +34,59 @@ struct DdsArgs {
 template <int V, int LPN>
 struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw < 1 ? 1 : (raw > LPN ? LPN : raw); };
 
+// One round of a chunk: U nonzeros per group gathered back to back, dotted against the column of B
+// and reduced together; returns the running per-lane result (lane l keeps the l-th nonzero of the
+// chunk). PRED: the round may reach past the end of the segment; slots there issue no load at all
+// (so a short segment costs the memory pipeline nothing for its unused slots) and contribute zeros.
+template <int W, int V, int LPN, bool EXACT, bool PRED>
+__device__ __forceinline__ float dds_round(const float* __restrict__ A, int k, int myrow, int it0, int rem, int g, int l,
+                                           int label, const int (&eld)[V], const bool (&ev)[V], const Vec<W> (&b)[V],
+                                           float res) {
+    constexpr int NG = 64 / LPN;
+    constexpr int U = Unroll<V, LPN>::U;
+    constexpr bool MULTI = (LPN >= 8) && (U >= 2);       // U dot products reduced together
+    Vec<W> av[U][V];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        // slot u of the round belongs to the nonzero kept by lane it0 + slot_offset(u)
+        const int it = it0 + (MULTI ? slot_offset<U>(u, it0) : u);
+        int r;
+        if constexpr (LPN == 64) r = __builtin_amdgcn_readlane(myrow, it);
+        else r = lane_read(myrow, g * LPN + it);
+        const float* ap = A + (size_t)r * (size_t)k;
+        if (!PRED || (it * NG + g) < rem) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::zero();
+        }
+    }
+    float sums[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            Vec<W> x = av[u][i];
+            if (!EXACT) x = ev[i] ? x : Vec<W>::zero();   // lanes past k contribute nothing
+            s = x.dotacc(b[i], s);
+        }
+        sums[u] = s;
+    }
+    if constexpr (MULTI) {
+        const float red = group_multisum<LPN, U>(sums, label);
+        res = (l / U == it0 / U) ? red : res;
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float s = group_allsum<LPN>(sums[u]);
+            res = (l == it0 + u) ? s : res;
+        }
+    }
+    return res;
+}
+
 template <int W, int V, int LPN, bool EXACT, bool FULL>
 __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, int myrow, float* o, int rem, int g,
                                           int l, const int (&eld)[V], const bool (&ev)[V],
@@ -42,45 +95,21 @@ __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, in
     constexpr int U = Unroll<V, LPN>::U;
     const int q = l * NG + g;            // the nonzero of this chunk whose result this lane keeps
     float res = 0.f;
-    const int niter = FULL ? LPN : (rem + NG - 1) / NG;
-    constexpr bool MULTI = (LPN >= 8) && (U >= 2);       // U dot products reduced together
     const int label = slot_label(l);
+    if (FULL) {
 #pragma unroll 1
-    for (int it0 = 0; it0 < niter; it0 += U) {
-        Vec<W> av[U][V];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            // slot u of the round belongs to the nonzero kept by lane it0 + slot_offset(u)
-            const int it = it0 + (MULTI ? slot_offset<U>(u, it0) : u);
-            int r;
-            if constexpr (LPN == 64) r = __builtin_amdgcn_readlane(myrow, it);
-            else r = lane_read(myrow, g * LPN + it);
-            const float* ap = A + (size_t)r * (size_t)k;
-#pragma unroll
-            for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
-        }
-        float sums[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            float s = 0.f;
-#pragma unroll
-            for (int i = 0; i < V; ++i) {
-                Vec<W> x = av[u][i];
-                if (!EXACT) x = ev[i] ? x : Vec<W>::zero();   // lanes past k contribute nothing
-                s = x.dotacc(b[i], s);
-            }
-            sums[u] = s;
-        }
-        if constexpr (MULTI) {
-            const float red = group_multisum<LPN, U>(sums, label);
-            res = (l / U == it0 / U) ? red : res;
-        } else {
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const float s = group_allsum<LPN>(sums[u]);
-                res = (l == it0 + u) ? s : res;
-            }
-        }
+        for (int it0 = 0; it0 < LPN; it0 += U)
+            res = dds_round<W, V, LPN, EXACT, false>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
+    } else {
+        const int niter = (rem + NG - 1) / NG;
+        const int nwhole = (rem / (NG * U)) * U;         // rounds whose every slot lies inside the segment
+        int it0 = 0;
+#pragma unroll 1
+        for (; it0 < nwhole; it0 += U)
+            res = dds_round<W, V, LPN, EXACT, false>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
+#pragma unroll 1
+        for (; it0 < niter; it0 += U)
+            res = dds_round<W, V, LPN, EXACT, true>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
     }
     if (FULL || q < rem) {                                        // o: where this lane's nonzero goes
         if (accumulate) res += *o;
@@ -150,6 +179,79 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
     }
 }
 
+// ---- DDS over a row-class ordered pattern (plan.hpp): workgroup b runs on XCD b % 8 and only
+// touches the nonzeros whose row belongs to class b % 8, so the eight L2s cache disjoint rows.
+// A wave walks a strip of consecutive columns; for each it loads the column of B once and runs the
+// class's nonzeros of that column through the same chunk code as k_dds. Results go to their
+// original CSC positions through cperm, so the output is bit-identical to k_dds.
+struct DdsClassedArgs {
+    int k;
+    int ncols;
+    int strip;           // columns per wave (<= 64)
+    int beta;
+    int opn;
+    const float* A;
+    const float* B;
+    const float* V;
+    const int* cir;
+    const int* cperm;
+    const int* cptr;
+    float* P;
+};
+
+template <int W, int V, int LPN, bool EXACT>
+__global__ __launch_bounds__(BM_BLOCK) void k_dds_classed(DdsClassedArgs a) {
+    constexpr int KT = W * V * LPN;
+    const int lane = threadIdx.x & 63;
+    const int x = blockIdx.x & 7;
+    const long long strip = (long long)(blockIdx.x >> 3) * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+    const long long c0 = strip * a.strip;
+    if (c0 >= a.ncols) return;
+    const int nc = (int)((a.ncols - c0) < a.strip ? (a.ncols - c0) : a.strip);
+    const int g = lane / LPN, l = lane % LPN;
+    const int q = l * (64 / LPN) + g;
+    // lane i holds the bounds of class x in column c0 + i
+    int ps = 0, pe = 0;
+    if (lane < nc) {
+        const long long sc = (c0 + lane) * 8 + x;
+        ps = a.cptr[sc];
+        pe = a.cptr[sc + 1];
+    }
+    for (int ci = 0; ci < nc; ++ci) {
+        const int jstart = __builtin_amdgcn_readlane(ps, ci), jend = __builtin_amdgcn_readlane(pe, ci);
+        if (jstart >= jend) continue;
+        const float* bp = a.B + (size_t)(c0 + ci) * (size_t)a.k;
+        for (int k0 = 0; k0 < a.k; k0 += KT) {
+            int eld[V];
+            bool ev[V];
+            Vec<W> b[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const int e = k0 + (i * LPN + l) * W;
+                ev[i] = e < a.k;
+                eld[i] = ev[i] ? e : 0;
+                b[i] = ev[i] ? Vec<W>::load(bp + e) : Vec<W>::zero();
+            }
+            const bool accumulate = (a.beta != 0) || (k0 > 0);
+            const bool last = k0 + KT >= a.k;
+            int j0 = jstart, rem = jend - jstart;
+            int crow = 0, cpos = 0;
+            if (q < rem) { crow = a.cir[j0 + q]; cpos = a.cperm[j0 + q]; }
+            while (rem > 0) {
+                int nrow = 0, npos = 0;
+                if (q < rem - 64) { nrow = a.cir[j0 + 64 + q]; npos = a.cperm[j0 + 64 + q]; }
+                float* o = a.P + cpos;
+                const float* vq = (a.V != nullptr && last) ? a.V + cpos : nullptr;
+                if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, vq, a.opn);
+                else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, vq, a.opn);
+                crow = nrow; cpos = npos;
+                j0 += 64;
+                rem -= 64;
+            }
+        }
+    }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 hipError_t launch_dds(const Shape& sh, bool exact, const DdsArgs& a, long long nwaves, hipStream_t s) {
@@ -174,7 +276,44 @@ hipError_t launch_dds(const Shape& sh, bool exact, const DdsArgs& a, long long n
     return hipErrorInvalidValue;
 }
 
+hipError_t launch_dds_classed(const Shape& sh, bool exact, const DdsClassedArgs& a, hipStream_t s) {
+    const long long nstrips = ((long long)a.ncols + a.strip - 1) / a.strip;
+    const long long nblk = 8 * ((nstrips + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK);
+    if (nblk <= 0) return hipSuccess;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)nblk), block(BM_BLOCK);
+#define BM_CASE(W_, V_, L_, E_)                                                          \
+    if (sh.W == W_ && sh.V == V_ && sh.LPN == L_ && exact == E_) {                       \
+        hipLaunchKernelGGL((k_dds_classed<W_, V_, L_, E_>), grid, block, 0, s, a);       \
+        return hipGetLastError();                                                        \
+    }
+#define BM_CASES(W_, E_)                                                                 \
+    BM_CASE(W_, 1, 1, E_) BM_CASE(W_, 1, 2, E_) BM_CASE(W_, 1, 4, E_) BM_CASE(W_, 1, 8, E_) \
+    BM_CASE(W_, 1, 16, E_) BM_CASE(W_, 1, 32, E_) BM_CASE(W_, 1, 64, E_) BM_CASE(W_, 2, 64, E_) \
+    BM_CASE(W_, 4, 64, E_)
+    BM_CASES(1, false)
+    BM_CASES(4, false)
+    BM_CASES(4, true)
+#undef BM_CASES
+#undef BM_CASE
+    return hipErrorInvalidValue;
+}
+
 }  // namespace
+
+hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const int* cir, const int* cperm,
+                       const int* cptr, float* P, int beta, hipStream_t s, const float* V, int opn) {
+    if (ncols <= 0 || k <= 0) return hipErrorInvalidValue;          // callers route those cases to dds_csc
+    if (V != nullptr && (beta != 0 || opn < 0 || opn > 14)) return hipErrorInvalidValue;
+    Shape sh = pick_shape(k, aligned16(A) && aligned16(B));
+    if (sh.V > 4) sh.V = 4;
+    const bool exact = (sh.W == 4) && (k % (sh.W * sh.V * sh.LPN) == 0);
+    DdsClassedArgs a;
+    a.k = k; a.ncols = ncols; a.beta = beta; a.opn = opn;
+    a.strip = (int)opt_class_strip();
+    a.A = A; a.B = B; a.V = V; a.cir = cir; a.cperm = cperm; a.cptr = cptr; a.P = P;
+    return launch_dds_classed(sh, exact, a, s);
+}
 
 hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
                    const int* jc, float* P, int beta, hipStream_t s, const float* V, int opn,

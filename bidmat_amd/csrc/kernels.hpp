@@ -9,6 +9,8 @@ namespace bm {
 int opt_seglen();      // nonzeros per wave segment for long columns / rows
 int opt_panel_kb();    // KiB of A per column panel in a plan
 int opt_heavy_min();   // a row is cut by panels when it averages at least this many nonzeros per panel
+int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..64)
+int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always
 
 // ---- CSC utilities (csc_util.hip)
 hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);
@@ -72,6 +74,9 @@ hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const floa
 hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,
                    const int* jc, float* P, int beta, hipStream_t s, const float* V = nullptr, int opn = 0,
                    const ColTable* tab = nullptr);
+// DDS over a row-class ordered pattern (a plan's cir / cperm / cptr); same results, bit for bit.
+hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const int* cir, const int* cperm,
+                       const int* cptr, float* P, int beta, hipStream_t s, const float* V = nullptr, int opn = 0);
 // The same with no allocation at all: the overflow table lives in a fixed device array of the
 // library (one copy per device). ncols may not exceed dds_static_max_cols().
 int dds_static_max_cols();

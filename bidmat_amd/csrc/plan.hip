@@ -151,6 +151,75 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_bounds(int nseg, const unsig
     for (int c = prev + 1; c <= cls; ++c) start[c] = (int)s;
 }
 
+// One wavefront per column: counts the column's nonzeros per row class (row & 7), then writes them
+// out class by class, keeping the stored order inside a class. cptr[8*c + x] = start of class x of
+// column c; the last entry closes the last column.
+__global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, const int* __restrict__ ir,
+                                                              const int* __restrict__ jc, int* __restrict__ cir,
+                                                              int* __restrict__ cperm, int* __restrict__ cptr,
+                                                              int* __restrict__ maxlen) {
+    const int lane = threadIdx.x & 63;
+    const long long c = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+    if (c >= ncols) return;
+    const int s = jc[c], e = jc[c + 1];
+    int cnt[8];
+#pragma unroll
+    for (int x = 0; x < 8; ++x) cnt[x] = 0;
+    for (int j0 = s; j0 < e; j0 += 64) {
+        const int j = j0 + lane;
+        const bool valid = j < e;
+        const int r = valid ? ir[j] : 0;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) cnt[x] += __popcll(__ballot(valid && (r & 7) == x));
+    }
+    int base[8], run = 0;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) { base[x] = run; run += cnt[x]; }
+    if (lane < 8) {
+        int b = 0;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) b = (lane == x) ? base[x] : b;
+        cptr[c * 8 + lane] = s + b;
+    }
+    if (c == ncols - 1 && lane == 0) cptr[(long long)ncols * 8] = e;
+    if (lane == 0) atomicMax(maxlen, e - s);
+    const unsigned long long below = (1ULL << lane) - 1ULL;
+    for (int j0 = s; j0 < e; j0 += 64) {
+        const int j = j0 + lane;
+        const bool valid = j < e;
+        const int r = valid ? ir[j] : 0;
+        int dest = -1;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const bool mine = valid && (r & 7) == x;
+            const unsigned long long m = __ballot(mine);
+            if (mine) dest = s + base[x] + __popcll(m & below);
+            base[x] += __popcll(m);
+        }
+        if (valid) { cir[dest] = r; cperm[dest] = j; }
+    }
+}
+
+// out[0] = number of nonzeros in the n1 most frequent rows, out[1] = in the n8 most frequent rows;
+// sorted = row counts in descending order. One workgroup, integer sums.
+__global__ __launch_bounds__(BM_BLOCK) void k_top_coverage(int nrows, const int* __restrict__ sorted, int n1, int n8,
+                                                           unsigned long long* __restrict__ out) {
+    __shared__ unsigned long long s1[BM_BLOCK], s8[BM_BLOCK];
+    unsigned long long a = 0, b = 0;
+    for (int i = threadIdx.x; i < nrows && i < n8; i += BM_BLOCK) {
+        const unsigned long long v = (unsigned long long)sorted[i];
+        if (i < n1) a += v;
+        b += v;
+    }
+    s1[threadIdx.x] = a; s8[threadIdx.x] = b;
+    __syncthreads();
+    for (int d = BM_BLOCK / 2; d > 0; d >>= 1) {
+        if ((int)threadIdx.x < d) { s1[threadIdx.x] += s1[threadIdx.x + d]; s8[threadIdx.x] += s8[threadIdx.x + d]; }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) { out[0] = s1[0]; out[1] = s8[0]; }
+}
+
 inline unsigned grid_for(long long n, int maxblocks = 16384) {
     long long b = (n + BM_BLOCK - 1) / BM_BLOCK;
     if (b < 1) b = 1;
@@ -169,7 +238,7 @@ inline int bits_for(unsigned long long maxval) {
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
     hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals};
+    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals, p->cir, p->cperm, p->cptr};
     for (void* b : bufs)
         if (b && (f = hipFree(b)) != hipSuccess) e = f;
     delete p;
@@ -233,6 +302,28 @@ hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s) {
     hipLaunchKernelGGL(k_permute_values, dim3(grid_for(((long long)p->nnz + 3) / 4, 8192)), dim3(BM_BLOCK), 0, s,
                        (long long)p->nnz, data, p->perm, p->pvals);
     return hipGetLastError();
+}
+
+// Builds the row-class ordering of the columns (see plan.hpp). Row indices must be valid (the row
+// histogram has checked them, or does so right after).
+static hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, hipStream_t s) {
+    const int ncols = plan->ncols, nnz = plan->nnz;
+    if (ncols <= 0 || nnz <= 0 || (long long)ncols * 8 + 1 > 0x7fffffffLL) return hipSuccess;
+    hipError_t e;
+    const size_t nsub = (size_t)ncols * 8 + 1;
+    if ((e = hipMalloc((void**)&plan->cptr, sizeof(int) * (nsub + 1))) != hipSuccess) { (void)hipGetLastError(); return e; }
+    if ((e = hipMalloc((void**)&plan->cir, sizeof(int) * (size_t)nnz)) != hipSuccess) { (void)hipGetLastError(); return e; }
+    if ((e = hipMalloc((void**)&plan->cperm, sizeof(int) * (size_t)nnz)) != hipSuccess) { (void)hipGetLastError(); return e; }
+    int* d_maxlen = plan->cptr + nsub;                   // one spare int behind the table
+    if ((e = fill_i32(d_maxlen, 1, 0, s)) != hipSuccess) return e;
+    const long long nblk = ((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
+    hipLaunchKernelGGL(k_class_partition, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, ir, jc, plan->cir,
+                       plan->cperm, plan->cptr, d_maxlen);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if ((e = hipMemcpy(&plan->maxlen, d_maxlen, sizeof(int), hipMemcpyDeviceToHost)) != hipSuccess) return e;
+    plan->ncls = 8;
+    plan->index_bytes += sizeof(int) * (nsub + 1 + 2 * (size_t)nnz);
+    return hipSuccess;
 }
 
 #define PB_CHECK(expr)                                          \
@@ -366,6 +457,31 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     PB_CHECK(fill_i32(hrank + nrows, 2, 0, s));
     // few, long-lived workgroups: every one flushes its LDS histogram once at the end
     hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, ir, cnt, bad);
+
+    // 1b. column classes for DDS: worth it when one L2 (4 MiB) holds clearly fewer of the gathered
+    // rows' nonzeros than eight L2s with disjoint rows would. The row counts are sorted (descending)
+    // and the nonzeros of the top n1 and top 8*n1 rows compared, n1 = rows of the operand per L2.
+    {
+        const int mode = opt_col_classes();              // -1 auto, 0 never, 1 always
+        bool want = mode == 1;
+        if (mode < 0 && ncols > 0 && nnz / ncols >= 64 && (long long)nrows * 4 * k_hint > (8LL << 20)) {
+            const long long n1 = (4LL << 20) / (4LL * k_hint);
+            int* sorted = keys_out ? reinterpret_cast<int*>(keys_out) : nullptr;      // free until the key sort
+            unsigned long long* cov = reinterpret_cast<unsigned long long*>(colpos_out);
+            size_t tb = 0;
+            PB_CHECK(rocprim::radix_sort_keys_desc(nullptr, tb, cnt, sorted, (size_t)nrows, 0, 32, s));
+            if (tb <= sort_bytes && (size_t)nrows <= (size_t)nnz) {
+                PB_CHECK(rocprim::radix_sort_keys_desc(sorttmp, tb, cnt, sorted, (size_t)nrows, 0, 32, s));
+                hipLaunchKernelGGL(k_top_coverage, dim3(1), dim3(BM_BLOCK), 0, s, nrows, sorted,
+                                   (int)(n1 < nrows ? n1 : nrows), (int)(8 * n1 < nrows ? 8 * n1 : nrows), cov);
+                unsigned long long h[2] = {0, 0};
+                PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
+                // at least a tenth of all gathers must move from "misses L2" to "hits L2"
+                want = (double)(h[1] - h[0]) >= 0.10 * (double)nnz;
+            }
+        }
+        if (want) PB_CHECK(plan_build_classes(plan, ir, jc, s));
+    }
 
     // 2. heavy rows and their ranks
     int nheavy = 0;

@@ -41,6 +41,17 @@ struct bidmat_plan {
     int* ovf = nullptr;          // [ncols+1] exclusive scan of extra segments per column (only when novf > 0)
     float* ovf_partial = nullptr;        // A*S: partial sums of the overflow segments (novf*k floats)
     size_t ovf_partial_floats = 0;
+    // Row-class ordering of every column (DDS through the plan). The eight XCDs have one L2 each;
+    // when each of them gathers from the whole dense operand, all eight L2s end up holding the same
+    // popular rows. Rows are dealt to eight classes (row & 7) and the nonzeros of every column are
+    // grouped by the class of their row (stored order kept inside a class); a workgroup that runs
+    // on XCD x only touches class-x nonzeros, so every L2 caches one eighth of the rows.
+    // Built when the pattern promises a gain (plan.hip: wants_classes) or when the option says so.
+    int ncls = 0;                // 0: no class ordering; otherwise 8
+    int maxlen = 0;              // longest column
+    int* cir = nullptr;          // [nnz]         row of the p-th nonzero in class order
+    int* cperm = nullptr;        // [nnz]         its position in the original CSC order
+    int* cptr = nullptr;         // [8*ncols + 1] start of (column c, class x) at cptr[8*c + x]
     // Values in plan order (optional, bidmat_plan_set_values): pvals[p] = data[perm[p]], so that
     // A*^S and row sums stream their values instead of fetching each one through perm.
     float* pvals = nullptr;

@@ -330,7 +330,12 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "panel_kb" target size in KiB of one column panel of A in a plan (default 3072)
  *   "heavy_min" a row is cut by column panels when it averages at least this many nonzeros
  *              per panel (default 8)
- * Returns 0, or hipErrorInvalidValue for an unknown name / bad value. */
+ *   "col_classes" row-class ordering of the columns inside a plan, used by bidmat_dds_plan so that the
+ *              eight L2s of the device cache disjoint rows: -1 = decide from the pattern (default),
+ *              0 = never, 1 = always
+ *   "class_strip" columns per wavefront in the class-ordered DDS kernel (default 16, 1..64)
+ * Returns 0, or hipErrorInvalidValue for an unknown name / bad value; bidmat_get_option returns -2
+ * for an unknown name. */
 int bidmat_set_option(const char *name, long long value);
 long long bidmat_get_option(const char *name);
 

@@ -361,6 +361,57 @@ def test_dds_with_fused_elementwise_step(hip, k):
     d.free()
 
 
+@pytest.mark.parametrize("k", [1, 3, 32, 100, 128, 256, 260, 1024, 1100])
+def test_class_ordered_dds_equals_plain_dds(hip, k):
+    """DDS through a plan whose columns are ordered by row class (the kernel in which every XCD only
+    touches its own eighth of the rows) against bidmat_dds_csc, bit for bit: unsorted and repeated
+    rows, empty columns, classes that are empty everywhere, a column count that is no multiple of
+    the strip, every strip width, beta 0 / 1 and the fused elementwise step."""
+    rng = np.random.default_rng(88 + k)
+    old_cls, old_strip = hip.bidmat_get_option(b"col_classes"), hip.bidmat_get_option(b"class_strip")
+    hip_abi.check(hip.bidmat_set_option(b"col_classes", 1))
+    try:
+        for variant in ("mixed", "one_class", "two_rows"):
+            nrows, ncols = 700, 333
+            lengths = rng.integers(0, 90, size=ncols)
+            lengths[0], lengths[5], lengths[332] = 0, 700, 130
+            _, ir, jc = random_csc(rng, nrows, ncols, lengths=lengths, sort_rows=False, unique=False)
+            if variant == "one_class":
+                ir = (ir // 8 * 8 + 3).astype(np.int32)          # every row in class 3
+                ir[ir >= nrows] = 3
+            elif variant == "two_rows":
+                ir = np.where(rng.random(ir.size) < 0.5, 0, 9).astype(np.int32)
+            nnz = int(ir.size)
+            A = rng.standard_normal(k * nrows).astype(np.float32)
+            B = rng.standard_normal(k * ncols).astype(np.float32)
+            V = rng.standard_normal(nnz).astype(np.float32)
+            d = Dev(A=A, B=B, ir=ir, jc=jc, V=V)
+            plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+            for strip in (1, 16, 64):
+                hip_abi.check(hip.bidmat_set_option(b"class_strip", strip))
+                for beta in (0, 1):
+                    P0 = rng.standard_normal(nnz).astype(np.float32)
+                    p1, p2 = DeviceArray.from_numpy(P0), DeviceArray.from_numpy(P0)
+                    hip_abi.check(hip.bidmat_dds_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, p1.ptr, beta, None))
+                    hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, None, 0, p2.ptr, beta, None))
+                    hip_abi.check(hip.bidmat_synchronize())
+                    assert np.array_equal(p1.numpy(), p2.numpy()), (variant, strip, beta)
+                q1, q2 = DeviceArray.zeros(nnz), DeviceArray.zeros(nnz)
+                hip_abi.check(hip.bidmat_dds_csc_op(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, 3, q1.ptr, None))
+                hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, 3, q2.ptr, 0, None))
+                hip_abi.check(hip.bidmat_synchronize())
+                assert np.array_equal(q1.numpy(), q2.numpy(), equal_nan=True), (variant, strip)
+            ref64, sa = oracle.dds_f64(A, B, k, ir, jc)
+            hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, None, 0, p2.ptr, 0, None))
+            hip_abi.check(hip.bidmat_synchronize())
+            close(p2.numpy(), ref64, sa, "class-ordered DDS k=%d %s" % (k, variant))
+            hip_abi.check(hip.bidmat_plan_destroy(plan))
+            d.free()
+    finally:
+        hip_abi.check(hip.bidmat_set_option(b"col_classes", old_cls))
+        hip_abi.check(hip.bidmat_set_option(b"class_strip", old_strip))
+
+
 def test_config2_dds_pure_relative_error(hip):
     """configs[1] scaled to 10 %: every term of every dot product is positive (A, B ~ U(0,1)), so the
     plain relative error is well defined; it must stay below 1e-4 for every one of the ~10 M values."""
