@@ -23,7 +23,11 @@ std::atomic<int> g_panel_kb{3072};
 std::atomic<int> g_heavy_min{8};
 std::atomic<int> g_col_classes{-1};
 std::atomic<int> g_class_strip{16};
+std::atomic<int> g_class_hot{0};
+std::atomic<int> g_class_threads{1024};
 }  // namespace
+int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
+int opt_class_hot() { return g_class_hot.load(std::memory_order_relaxed); }
 int opt_class_strip() { return g_class_strip.load(std::memory_order_relaxed); }
 int opt_col_classes() { return g_col_classes.load(std::memory_order_relaxed); }
 int opt_heavy_min() { return g_heavy_min.load(std::memory_order_relaxed); }
@@ -405,8 +409,10 @@ API int bidmat_dds_plan(bidmat_plan* plan, int k, const float* A, const float* B
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (plan->ncols == 0 || plan->nnz == 0) return 0;
     if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
-    if (plan->ncls == 8 && k > 0 && plan->maxlen <= kMaxClassedColumn)
-        return (int)bm::dds_classed(k, plan->ncols, A, B, plan->cir, plan->cperm, plan->cptr, P, beta, as_stream(stream), V, opn);
+    if (plan->ncls == 8 && k > 0 && plan->maxlen <= kMaxClassedColumn &&
+        (size_t)plan->hcap * (size_t)k * sizeof(float) <= bm::dds_classed_lds_budget())
+        return (int)bm::dds_classed(k, plan->ncols, A, B, plan->cir, plan->cperm, plan->cptr, plan->hcap, plan->hotrows, P, beta,
+                                    as_stream(stream), V, opn);
     const bm::ColTable tab = col_table(plan);
     return (int)bm::dds_csc(k, plan->ncols, plan->nnz, A, B, Sir, Sjc, P, beta, as_stream(stream), V, opn, &tab);
 }
@@ -744,6 +750,16 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_heavy_min.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "class_threads")) {
+        if (value != 256 && value != 512 && value != 1024) return kInvalid;
+        bm::g_class_threads.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "class_hot")) {
+        if (value < -1 || value > 1024) return kInvalid;
+        bm::g_class_hot.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "class_strip")) {
         if (value < 1 || value > 64) return kInvalid;
         bm::g_class_strip.store((int)value);
@@ -764,6 +780,8 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "heavy_min")) return bm::opt_heavy_min();
     if (!strcmp(name, "col_classes")) return bm::opt_col_classes();
     if (!strcmp(name, "class_strip")) return bm::opt_class_strip();
+    if (!strcmp(name, "class_hot")) return bm::opt_class_hot();
+    if (!strcmp(name, "class_threads")) return bm::opt_class_threads();
     return -2;
 }
 

@@ -38,7 +38,10 @@ struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw <
 // and reduced together; returns the running per-lane result (lane l keeps the l-th nonzero of the
 // chunk). PRED: the round may reach past the end of the segment; slots there issue no load at all
 // (so a short segment costs the memory pipeline nothing for its unused slots) and contribute zeros.
-template <int W, int V, int LPN, bool EXACT, bool PRED>
+// LDSROWS: myrow holds ranks of hot rows, which sit in the workgroup's LDS (hot_lds) instead of A.
+extern __shared__ __align__(16) float hot_lds[];
+
+template <int W, int V, int LPN, bool EXACT, bool PRED, bool LDSROWS = false>
 __device__ __forceinline__ float dds_round(const float* __restrict__ A, int k, int myrow, int it0, int rem, int g, int l,
                                            int label, const int (&eld)[V], const bool (&ev)[V], const Vec<W> (&b)[V],
                                            float res) {
@@ -53,10 +56,16 @@ __device__ __forceinline__ float dds_round(const float* __restrict__ A, int k, i
         int r;
         if constexpr (LPN == 64) r = __builtin_amdgcn_readlane(myrow, it);
         else r = lane_read(myrow, g * LPN + it);
-        const float* ap = A + (size_t)r * (size_t)k;
         if (!PRED || (it * NG + g) < rem) {
+            if constexpr (LDSROWS) {
+                const float* hp = hot_lds + r * k;
 #pragma unroll
-            for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
+                for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(hp + eld[i]);
+            } else {
+                const float* ap = A + (size_t)r * (size_t)k;
+#pragma unroll
+                for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::zero();
@@ -87,7 +96,7 @@ __device__ __forceinline__ float dds_round(const float* __restrict__ A, int k, i
     return res;
 }
 
-template <int W, int V, int LPN, bool EXACT, bool FULL>
+template <int W, int V, int LPN, bool EXACT, bool FULL, bool LDSROWS = false>
 __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, int myrow, float* o, int rem, int g,
                                           int l, const int (&eld)[V], const bool (&ev)[V],
                                           const Vec<W> (&b)[V], bool accumulate, const float* vq, int opn) {
@@ -99,17 +108,17 @@ __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, in
     if (FULL) {
 #pragma unroll 1
         for (int it0 = 0; it0 < LPN; it0 += U)
-            res = dds_round<W, V, LPN, EXACT, false>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
+            res = dds_round<W, V, LPN, EXACT, false, LDSROWS>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
     } else {
         const int niter = (rem + NG - 1) / NG;
         const int nwhole = (rem / (NG * U)) * U;         // rounds whose every slot lies inside the segment
         int it0 = 0;
 #pragma unroll 1
         for (; it0 < nwhole; it0 += U)
-            res = dds_round<W, V, LPN, EXACT, false>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
+            res = dds_round<W, V, LPN, EXACT, false, LDSROWS>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
 #pragma unroll 1
         for (; it0 < niter; it0 += U)
-            res = dds_round<W, V, LPN, EXACT, true>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
+            res = dds_round<W, V, LPN, EXACT, true, LDSROWS>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
     }
     if (FULL || q < rem) {                                        // o: where this lane's nonzero goes
         if (accumulate) res += *o;
@@ -180,73 +189,137 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
 }
 
 // ---- DDS over a row-class ordered pattern (plan.hpp): workgroup b runs on XCD b % 8 and only
-// touches the nonzeros whose row belongs to class b % 8, so the eight L2s cache disjoint rows.
-// A wave walks a strip of consecutive columns; for each it loads the column of B once and runs the
-// class's nonzeros of that column through the same chunk code as k_dds. Results go to their
-// original CSC positions through cperm, so the output is bit-identical to k_dds.
+// touches the nonzeros whose row belongs to class b % 8, so the eight L2s cache disjoint rows, and
+// the class's most frequent rows sit in the workgroup's LDS (filled once; workgroups are persistent
+// and walk strips of consecutive columns). For each column a wave loads the column of B once, runs
+// the class's hot-row nonzeros against LDS and the others against global memory, through the same
+// chunk code as k_dds. Results go to their CSC positions through cperm: bit-identical to k_dds.
+constexpr int CL_MAX_THREADS = 1024;
+constexpr size_t CL_LDS_MAX = size_t(128) << 10;         // most LDS one workgroup may ask for
+constexpr size_t CL_LDS_PER_CU = size_t(160) << 10;
+
 struct DdsClassedArgs {
     int k;
     int ncols;
-    int strip;           // columns per wave (<= 64)
+    int strip;           // columns per wave and step (<= 64)
     int beta;
     int opn;
+    int hcap;            // hot rows per class
     const float* A;
     const float* B;
     const float* V;
     const int* cir;
     const int* cperm;
     const int* cptr;
+    const int* hotrows;
     float* P;
 };
 
+// One run of nonzeros [jstart, jend) of the current column. (crow, cpos): row / output position of
+// this lane's nonzero of the run's first chunk, loaded by the caller ahead of time.
+template <int W, int V, int LPN, bool EXACT, bool LDSROWS>
+__device__ __forceinline__ void dds_classed_run(const DdsClassedArgs& a, int jstart, int jend, int crow, int cpos, int q,
+                                                int g, int l, const int (&eld)[V], const bool (&ev)[V],
+                                                const Vec<W> (&b)[V], bool accumulate, bool last) {
+    int j0 = jstart, rem = jend - jstart;
+    while (rem > 0) {
+        int nrow = 0, npos = 0;
+        if (q < rem - 64) { nrow = a.cir[j0 + 64 + q]; npos = a.cperm[j0 + 64 + q]; }
+        float* o = a.P + cpos;
+        const float* vq = (a.V != nullptr && last) ? a.V + cpos : nullptr;
+        if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true, LDSROWS>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, vq, a.opn);
+        else dds_chunk<W, V, LPN, EXACT, false, LDSROWS>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, vq, a.opn);
+        crow = nrow; cpos = npos;
+        j0 += 64;
+        rem -= 64;
+    }
+}
+
+// What a wave loads ahead for one column: bounds of its two runs, this lane's nonzero of each run's
+// first chunk, and the first pass of the column of B.
+template <int W, int V>
+struct ColumnAhead {
+    int js, jm, je;
+    int hrow, hpos, trow, tpos;
+    Vec<W> b[V];
+};
+
+template <int W, int V, int LPN>
+__device__ __forceinline__ void load_column_ahead(const DdsClassedArgs& a, long long c, int js, int jm, int je, int q,
+                                                  int l, ColumnAhead<W, V>& n) {
+    n.js = js; n.jm = jm; n.je = je;
+    n.hrow = n.hpos = n.trow = n.tpos = 0;
+    if (q < jm - js) { n.hrow = a.cir[js + q]; n.hpos = a.cperm[js + q]; }
+    if (q < je - jm) { n.trow = a.cir[jm + q]; n.tpos = a.cperm[jm + q]; }
+    const float* bp = a.B + (size_t)c * (size_t)a.k;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        const int e = (i * LPN + l) * W;
+        n.b[i] = (e < a.k && js < je) ? Vec<W>::load(bp + e) : Vec<W>::zero();
+    }
+}
+
 template <int W, int V, int LPN, bool EXACT>
-__global__ __launch_bounds__(BM_BLOCK) void k_dds_classed(DdsClassedArgs a) {
+__global__ __launch_bounds__(CL_MAX_THREADS) void k_dds_classed(DdsClassedArgs a) {
     constexpr int KT = W * V * LPN;
     const int lane = threadIdx.x & 63;
+    const int wave = wave_uniform(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
     const int x = blockIdx.x & 7;
-    const long long strip = (long long)(blockIdx.x >> 3) * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
-    const long long c0 = strip * a.strip;
-    if (c0 >= a.ncols) return;
-    const int nc = (int)((a.ncols - c0) < a.strip ? (a.ncols - c0) : a.strip);
+    // ---- this class's hot rows into LDS, row h at hot_lds[h*k ..]
+    if (a.hcap > 0) {
+        const int vpr = (a.k + W - 1) / W;                // vectors per row (W == 4 implies k % 4 == 0)
+        const int total = a.hcap * vpr;
+        for (int i = threadIdx.x; i < total; i += blockDim.x) {
+            const int h = i / vpr, e = (i - h * vpr) * W;
+            const int row = a.hotrows[x * a.hcap + h];
+            const Vec<W> v = row >= 0 ? Vec<W>::load(a.A + (size_t)row * (size_t)a.k + e) : Vec<W>::zero();
+            v.store(hot_lds + h * a.k + e);
+        }
+        __syncthreads();
+    }
     const int g = lane / LPN, l = lane % LPN;
     const int q = l * (64 / LPN) + g;
-    // lane i holds the bounds of class x in column c0 + i
-    int ps = 0, pe = 0;
-    if (lane < nc) {
-        const long long sc = (c0 + lane) * 8 + x;
-        ps = a.cptr[sc];
-        pe = a.cptr[sc + 1];
-    }
-    for (int ci = 0; ci < nc; ++ci) {
-        const int jstart = __builtin_amdgcn_readlane(ps, ci), jend = __builtin_amdgcn_readlane(pe, ci);
-        if (jstart >= jend) continue;
-        const float* bp = a.B + (size_t)(c0 + ci) * (size_t)a.k;
-        for (int k0 = 0; k0 < a.k; k0 += KT) {
-            int eld[V];
-            bool ev[V];
-            Vec<W> b[V];
+    const long long nstrips = ((long long)a.ncols + a.strip - 1) / a.strip;
+    const long long wstride = (long long)(gridDim.x >> 3) * nwaves;
+    for (long long strip = (long long)(blockIdx.x >> 3) * nwaves + wave; strip < nstrips; strip += wstride) {
+        const long long c0 = strip * a.strip;
+        const int nc = (int)((a.ncols - c0) < a.strip ? (a.ncols - c0) : a.strip);
+        // lane i holds the bounds of class x in column c0 + i: hot-row nonzeros [ps, pm), the others [pm, pe)
+        int ps = 0, pm = 0, pe = 0;
+        if (lane < nc) {
+            const long long sc = (c0 + lane) * 16 + 2 * x;
+            ps = a.cptr[sc];
+            pm = a.cptr[sc + 1];
+            pe = a.cptr[sc + 2];
+        }
+        ColumnAhead<W, V> nx;
+        load_column_ahead<W, V, LPN>(a, c0, __builtin_amdgcn_readlane(ps, 0), __builtin_amdgcn_readlane(pm, 0),
+                                     __builtin_amdgcn_readlane(pe, 0), q, l, nx);
+        for (int ci = 0; ci < nc; ++ci) {
+            const ColumnAhead<W, V> cur = nx;
+            // the next column's index chunks and its column of B are requested before this column's gathers
+            if (ci + 1 < nc)
+                load_column_ahead<W, V, LPN>(a, c0 + ci + 1, __builtin_amdgcn_readlane(ps, ci + 1),
+                                             __builtin_amdgcn_readlane(pm, ci + 1), __builtin_amdgcn_readlane(pe, ci + 1), q, l, nx);
+            if (cur.js >= cur.je) continue;
+            const float* bp = a.B + (size_t)(c0 + ci) * (size_t)a.k;
+            for (int k0 = 0; k0 < a.k; k0 += KT) {
+                int eld[V];
+                bool ev[V];
+                Vec<W> b[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) {
-                const int e = k0 + (i * LPN + l) * W;
-                ev[i] = e < a.k;
-                eld[i] = ev[i] ? e : 0;
-                b[i] = ev[i] ? Vec<W>::load(bp + e) : Vec<W>::zero();
-            }
-            const bool accumulate = (a.beta != 0) || (k0 > 0);
-            const bool last = k0 + KT >= a.k;
-            int j0 = jstart, rem = jend - jstart;
-            int crow = 0, cpos = 0;
-            if (q < rem) { crow = a.cir[j0 + q]; cpos = a.cperm[j0 + q]; }
-            while (rem > 0) {
-                int nrow = 0, npos = 0;
-                if (q < rem - 64) { nrow = a.cir[j0 + 64 + q]; npos = a.cperm[j0 + 64 + q]; }
-                float* o = a.P + cpos;
-                const float* vq = (a.V != nullptr && last) ? a.V + cpos : nullptr;
-                if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, vq, a.opn);
-                else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, vq, a.opn);
-                crow = nrow; cpos = npos;
-                j0 += 64;
-                rem -= 64;
+                for (int i = 0; i < V; ++i) {
+                    const int e = k0 + (i * LPN + l) * W;
+                    ev[i] = e < a.k;
+                    eld[i] = ev[i] ? e : 0;
+                    if (k0 == 0) b[i] = cur.b[i];
+                    else b[i] = ev[i] ? Vec<W>::load(bp + e) : Vec<W>::zero();
+                }
+                const bool accumulate = (a.beta != 0) || (k0 > 0);
+                const bool last = k0 + KT >= a.k;
+                dds_classed_run<W, V, LPN, EXACT, true>(a, cur.js, cur.jm, cur.hrow, cur.hpos, q, g, l, eld, ev, b, accumulate, last);
+                dds_classed_run<W, V, LPN, EXACT, false>(a, cur.jm, cur.je, cur.trow, cur.tpos, q, g, l, eld, ev, b, accumulate, last);
             }
         }
     }
@@ -276,15 +349,41 @@ hipError_t launch_dds(const Shape& sh, bool exact, const DdsArgs& a, long long n
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_dds_classed(const Shape& sh, bool exact, const DdsClassedArgs& a, hipStream_t s) {
+hipError_t launch_dds_classed(const Shape& sh, bool exact, const DdsClassedArgs& a, size_t lds_bytes, hipStream_t s) {
+    int dev = 0, cus = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
     const long long nstrips = ((long long)a.ncols + a.strip - 1) / a.strip;
-    const long long nblk = 8 * ((nstrips + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK);
+    int threads = (int)opt_class_threads();
+    long long nblk;
+    if (lds_bytes == 0) {
+        // nothing to keep per workgroup: one strip per wave, small workgroups
+        threads = BM_BLOCK;
+        nblk = 8 * ((nstrips + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK);
+    } else {
+        // persistent workgroups (each fills its LDS once): as many per CU as LDS and wave slots allow,
+        // a multiple of 8 so that every XCD gets the same number
+        const int waves = threads / 64;
+        long long per_cu = (long long)(CL_LDS_PER_CU / lds_bytes);
+        if (per_cu > 32 / waves) per_cu = 32 / waves;
+        if (per_cu < 1) per_cu = 1;
+        long long per_xcd = per_cu * (cus / 8 > 0 ? cus / 8 : 1);
+        const long long need = ((nstrips + 7) / 8 + waves - 1) / waves;    // workgroups per XCD that still find a strip
+        if (need < per_xcd) per_xcd = need > 0 ? need : 1;
+        nblk = 8 * per_xcd;
+    }
     if (nblk <= 0) return hipSuccess;
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
-    dim3 grid((unsigned)nblk), block(BM_BLOCK);
+    dim3 grid((unsigned)nblk), block((unsigned)threads);
 #define BM_CASE(W_, V_, L_, E_)                                                          \
     if (sh.W == W_ && sh.V == V_ && sh.LPN == L_ && exact == E_) {                       \
-        hipLaunchKernelGGL((k_dds_classed<W_, V_, L_, E_>), grid, block, 0, s, a);       \
+        auto kern = k_dds_classed<W_, V_, L_, E_>;                                       \
+        if (lds_bytes > (48u << 10)) {                                                   \
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); \
+            if (e != hipSuccess) return e;                                               \
+        }                                                                                \
+        hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, a);                          \
         return hipGetLastError();                                                        \
     }
 #define BM_CASES(W_, E_)                                                                 \
@@ -301,18 +400,23 @@ hipError_t launch_dds_classed(const Shape& sh, bool exact, const DdsClassedArgs&
 
 }  // namespace
 
+size_t dds_classed_lds_budget() { return CL_LDS_MAX; }
+
 hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const int* cir, const int* cperm,
-                       const int* cptr, float* P, int beta, hipStream_t s, const float* V, int opn) {
+                       const int* cptr, int hcap, const int* hotrows, float* P, int beta, hipStream_t s,
+                       const float* V, int opn) {
     if (ncols <= 0 || k <= 0) return hipErrorInvalidValue;          // callers route those cases to dds_csc
     if (V != nullptr && (beta != 0 || opn < 0 || opn > 14)) return hipErrorInvalidValue;
+    const size_t lds_bytes = (size_t)hcap * (size_t)k * sizeof(float);
+    if (lds_bytes > CL_LDS_MAX || (hcap > 0 && !hotrows)) return hipErrorInvalidValue;
     Shape sh = pick_shape(k, aligned16(A) && aligned16(B));
     if (sh.V > 4) sh.V = 4;
     const bool exact = (sh.W == 4) && (k % (sh.W * sh.V * sh.LPN) == 0);
     DdsClassedArgs a;
-    a.k = k; a.ncols = ncols; a.beta = beta; a.opn = opn;
+    a.k = k; a.ncols = ncols; a.beta = beta; a.opn = opn; a.hcap = hcap;
     a.strip = (int)opt_class_strip();
-    a.A = A; a.B = B; a.V = V; a.cir = cir; a.cperm = cperm; a.cptr = cptr; a.P = P;
-    return launch_dds_classed(sh, exact, a, s);
+    a.A = A; a.B = B; a.V = V; a.cir = cir; a.cperm = cperm; a.cptr = cptr; a.hotrows = hotrows; a.P = P;
+    return launch_dds_classed(sh, exact, a, lds_bytes, s);
 }
 
 hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* ir,

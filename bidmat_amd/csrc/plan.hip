@@ -10,6 +10,7 @@
 #include <rocprim/device/device_radix_sort.hpp>
 #include <mutex>
 #include <new>
+#include <vector>
 
 namespace bm {
 namespace {
@@ -151,53 +152,74 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_bounds(int nseg, const unsig
     for (int c = prev + 1; c <= cls; ++c) start[c] = (int)s;
 }
 
-// One wavefront per column: counts the column's nonzeros per row class (row & 7), then writes them
-// out class by class, keeping the stored order inside a class. cptr[8*c + x] = start of class x of
-// column c; the last entry closes the last column.
+// One wavefront per column: counts the column's nonzeros per bucket, bucket = 2 * (row & 7) + (0 if the
+// row is one of its class's hot rows, else 1), then writes them out bucket by bucket, keeping the
+// stored order inside a bucket. cptr[16*c + b] = start of bucket b of column c; the last entry closes
+// the last column. For a hot row cir holds its rank among the hot rows of its class, otherwise the row.
 __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, const int* __restrict__ ir,
-                                                              const int* __restrict__ jc, int* __restrict__ cir,
+                                                              const int* __restrict__ jc,
+                                                              const int* __restrict__ hotrank,
+                                                              int* __restrict__ cir,
                                                               int* __restrict__ cperm, int* __restrict__ cptr,
                                                               int* __restrict__ maxlen) {
     const int lane = threadIdx.x & 63;
     const long long c = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
     if (c >= ncols) return;
     const int s = jc[c], e = jc[c + 1];
-    int cnt[8];
+    int cnt[16];
 #pragma unroll
-    for (int x = 0; x < 8; ++x) cnt[x] = 0;
+    for (int x = 0; x < 16; ++x) cnt[x] = 0;
     for (int j0 = s; j0 < e; j0 += 64) {
         const int j = j0 + lane;
         const bool valid = j < e;
         const int r = valid ? ir[j] : 0;
+        const int hr = (valid && hotrank != nullptr) ? hotrank[r] : -1;
+        const int bucket = 2 * (r & 7) + (hr < 0 ? 1 : 0);
 #pragma unroll
-        for (int x = 0; x < 8; ++x) cnt[x] += __popcll(__ballot(valid && (r & 7) == x));
+        for (int x = 0; x < 16; ++x) cnt[x] += __popcll(__ballot(valid && bucket == x));
     }
-    int base[8], run = 0;
+    int base[16], run = 0;
 #pragma unroll
-    for (int x = 0; x < 8; ++x) { base[x] = run; run += cnt[x]; }
-    if (lane < 8) {
-        int b = 0;
+    for (int x = 0; x < 16; ++x) { base[x] = run; run += cnt[x]; }
+    if (lane < 16) {
+        int bb = 0;
 #pragma unroll
-        for (int x = 0; x < 8; ++x) b = (lane == x) ? base[x] : b;
-        cptr[c * 8 + lane] = s + b;
+        for (int x = 0; x < 16; ++x) bb = (lane == x) ? base[x] : bb;
+        cptr[c * 16 + lane] = s + bb;
     }
-    if (c == ncols - 1 && lane == 0) cptr[(long long)ncols * 8] = e;
-    if (lane == 0) atomicMax(maxlen, e - s);
+    if (c == ncols - 1 && lane == 0) cptr[(long long)ncols * 16] = e;
+    // every column would hit the same address: only columns longer than the longest seen so far do
+    // (the plain read may be stale, which only costs a redundant atomic)
+    if (lane == 0 && e - s > __hip_atomic_load(maxlen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(maxlen, e - s);
     const unsigned long long below = (1ULL << lane) - 1ULL;
     for (int j0 = s; j0 < e; j0 += 64) {
         const int j = j0 + lane;
         const bool valid = j < e;
         const int r = valid ? ir[j] : 0;
+        const int hr = (valid && hotrank != nullptr) ? hotrank[r] : -1;
+        const int bucket = 2 * (r & 7) + (hr < 0 ? 1 : 0);
         int dest = -1;
 #pragma unroll
-        for (int x = 0; x < 8; ++x) {
-            const bool mine = valid && (r & 7) == x;
+        for (int x = 0; x < 16; ++x) {
+            const bool mine = valid && bucket == x;
             const unsigned long long m = __ballot(mine);
             if (mine) dest = s + base[x] + __popcll(m & below);
             base[x] += __popcll(m);
         }
-        if (valid) { cir[dest] = r; cperm[dest] = j; }
+        if (valid) { cir[dest] = hr < 0 ? r : hr; cperm[dest] = j; }
     }
+}
+
+__global__ __launch_bounds__(BM_BLOCK) void k_iota(int n, int* __restrict__ out) {
+    const long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    if (i < n) out[i] = (int)i;
+}
+
+// hotrank[rows[i]] = ranks[i]
+__global__ __launch_bounds__(BM_BLOCK) void k_scatter_rank(int n, const int* __restrict__ rows,
+                                                           const int* __restrict__ ranks, int* __restrict__ hotrank) {
+    const int i = blockIdx.x * BM_BLOCK + threadIdx.x;
+    if (i < n) hotrank[rows[i]] = ranks[i];
 }
 
 // out[0] = number of nonzeros in the n1 most frequent rows, out[1] = in the n8 most frequent rows;
@@ -238,7 +260,7 @@ inline int bits_for(unsigned long long maxval) {
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
     hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals, p->cir, p->cperm, p->cptr};
+    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals, p->cir, p->cperm, p->cptr, p->hotrows};
     for (void* b : bufs)
         if (b && (f = hipFree(b)) != hipSuccess) e = f;
     delete p;
@@ -306,18 +328,18 @@ hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s) {
 
 // Builds the row-class ordering of the columns (see plan.hpp). Row indices must be valid (the row
 // histogram has checked them, or does so right after).
-static hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, hipStream_t s) {
+static hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, const int* hotrank, hipStream_t s) {
     const int ncols = plan->ncols, nnz = plan->nnz;
-    if (ncols <= 0 || nnz <= 0 || (long long)ncols * 8 + 1 > 0x7fffffffLL) return hipSuccess;
+    if (ncols <= 0 || nnz <= 0 || (long long)ncols * 16 + 1 > 0x7fffffffLL) return hipSuccess;
     hipError_t e;
-    const size_t nsub = (size_t)ncols * 8 + 1;
+    const size_t nsub = (size_t)ncols * 16 + 1;
     if ((e = hipMalloc((void**)&plan->cptr, sizeof(int) * (nsub + 1))) != hipSuccess) { (void)hipGetLastError(); return e; }
     if ((e = hipMalloc((void**)&plan->cir, sizeof(int) * (size_t)nnz)) != hipSuccess) { (void)hipGetLastError(); return e; }
     if ((e = hipMalloc((void**)&plan->cperm, sizeof(int) * (size_t)nnz)) != hipSuccess) { (void)hipGetLastError(); return e; }
     int* d_maxlen = plan->cptr + nsub;                   // one spare int behind the table
     if ((e = fill_i32(d_maxlen, 1, 0, s)) != hipSuccess) return e;
     const long long nblk = ((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
-    hipLaunchKernelGGL(k_class_partition, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, ir, jc, plan->cir,
+    hipLaunchKernelGGL(k_class_partition, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, ir, jc, hotrank, plan->cir,
                        plan->cperm, plan->cptr, d_maxlen);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if ((e = hipMemcpy(&plan->maxlen, d_maxlen, sizeof(int), hipMemcpyDeviceToHost)) != hipSuccess) return e;
@@ -421,7 +443,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         sort_bytes = b1 > b2 ? b1 : b2;
     }
     Arena tmp;
-    int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *scantmp = nullptr, *class_count = nullptr;
+    int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *crank = nullptr, *scantmp = nullptr, *class_count = nullptr;
     int *flag = nullptr, *segidx = nullptr;
     unsigned *keys_in = nullptr, *keys_out = nullptr;
     unsigned long long *colpos_in = nullptr, *colpos_out = nullptr;
@@ -433,6 +455,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         hflag = tmp.take<int>((size_t)nrows);
         hrank = tmp.take<int>((size_t)nrows + 2);        // [nrows] = number of heavy rows, [nrows+1] = bad-index flag
         hrow = tmp.take<int>((size_t)nrows);
+        crank = tmp.take<int>((size_t)nrows);            // rank of a row among its class's hot rows, or -1
         scantmp = tmp.take<int>(scan_tmp_ints((long long)scan_n));
         class_count = tmp.take<int>(9);
         keys_in = tmp.take<unsigned>((size_t)nnz);       // later: ids of the segments
@@ -459,28 +482,77 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, ir, cnt, bad);
 
     // 1b. column classes for DDS: worth it when one L2 (4 MiB) holds clearly fewer of the gathered
-    // rows' nonzeros than eight L2s with disjoint rows would. The row counts are sorted (descending)
-    // and the nonzeros of the top n1 and top 8*n1 rows compared, n1 = rows of the operand per L2.
+    // rows' nonzeros than eight L2s with disjoint rows would. The rows are sorted by count (descending)
+    // and the nonzeros of the top n1 and top 8*n1 rows compared, n1 = rows of the operand per L2. The
+    // same ranking names every class's hot rows, the ones the DDS kernel keeps in LDS.
     {
         const int mode = opt_col_classes();              // -1 auto, 0 never, 1 always
         bool want = mode == 1;
-        if (mode < 0 && ncols > 0 && nnz / ncols >= 64 && (long long)nrows * 4 * k_hint > (8LL << 20)) {
+        // Measured (100 M nonzeros, Zipf(1.1) rows, k = 256): 5.53 -> 4.78 ms. With rows of 512 bytes
+        // (k = 128, 400 M nonzeros, Zipf(1.05)) the class-ordered kernel is bound by its instruction
+        // stream, not by the memory path, and loses (14.8 -> 16.1 ms): full-wave rows only.
+        const bool candidate = mode == 1 || (mode < 0 && ncols > 0 && nnz / ncols >= 64 && k_hint >= 256 &&
+                                             (long long)nrows * 4 * k_hint > (8LL << 20));
+        int* hotrank = nullptr;
+        if (candidate && (size_t)nrows <= (size_t)nnz) {
             const long long n1 = (4LL << 20) / (4LL * k_hint);
-            int* sorted = keys_out ? reinterpret_cast<int*>(keys_out) : nullptr;      // free until the key sort
+            int* iota = reinterpret_cast<int*>(keys_in);             // all free until the key sort
+            unsigned* cnt_sorted = keys_out;
+            int* rows_sorted = reinterpret_cast<int*>(colpos_in);
             unsigned long long* cov = reinterpret_cast<unsigned long long*>(colpos_out);
             size_t tb = 0;
-            PB_CHECK(rocprim::radix_sort_keys_desc(nullptr, tb, cnt, sorted, (size_t)nrows, 0, 32, s));
-            if (tb <= sort_bytes && (size_t)nrows <= (size_t)nnz) {
-                PB_CHECK(rocprim::radix_sort_keys_desc(sorttmp, tb, cnt, sorted, (size_t)nrows, 0, 32, s));
-                hipLaunchKernelGGL(k_top_coverage, dim3(1), dim3(BM_BLOCK), 0, s, nrows, sorted,
+            PB_CHECK(rocprim::radix_sort_pairs_desc(nullptr, tb, reinterpret_cast<unsigned*>(cnt), cnt_sorted, iota, rows_sorted,
+                                                    (size_t)nrows, 0, 32, s));
+            if (tb <= sort_bytes) {
+                hipLaunchKernelGGL(k_iota, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, iota);
+                PB_CHECK(rocprim::radix_sort_pairs_desc(sorttmp, tb, reinterpret_cast<unsigned*>(cnt), cnt_sorted, iota, rows_sorted,
+                                                        (size_t)nrows, 0, 32, s));
+                hipLaunchKernelGGL(k_top_coverage, dim3(1), dim3(BM_BLOCK), 0, s, nrows, reinterpret_cast<const int*>(cnt_sorted),
                                    (int)(n1 < nrows ? n1 : nrows), (int)(8 * n1 < nrows ? 8 * n1 : nrows), cov);
                 unsigned long long h[2] = {0, 0};
                 PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
                 // at least a tenth of all gathers must move from "misses L2" to "hits L2"
-                want = (double)(h[1] - h[0]) >= 0.10 * (double)nnz;
+                if (mode < 0) want = (double)(h[1] - h[0]) >= 0.10 * (double)nnz;
+                // hot rows per class kept in LDS: off unless asked for (-1: what 128 KiB hold at k_hint).
+                // Measured: no gain at k = 256 (4.78 ms without, 4.85 ms with 128 rows per class: the
+                // 1024-thread persistent workgroups that share the LDS rows cost what the rows save);
+                // at k = 128 they recover the class-ordered kernel's loss (16.1 -> 14.1 ms, plain 14.8).
+                long long hcap = opt_class_hot();
+                if (hcap < 0) hcap = (128LL << 10) / (4LL * k_hint);     // one workgroup of 1024 threads per CU
+                if (hcap > 1024) hcap = 1024;
+                if (want && hcap > 0) {
+                    const int ntop = (int)(8 * hcap < nrows ? 8 * hcap : nrows);
+                    std::vector<int> top((size_t)ntop), cnts((size_t)ntop);
+                    PB_CHECK(hipMemcpy(top.data(), rows_sorted, sizeof(int) * (size_t)ntop, hipMemcpyDeviceToHost));
+                    PB_CHECK(hipMemcpy(cnts.data(), cnt_sorted, sizeof(int) * (size_t)ntop, hipMemcpyDeviceToHost));
+                    std::vector<int> hotrows((size_t)(8 * hcap), -1), rows, ranks;
+                    int filled[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                    for (int i = 0; i < ntop; ++i) {
+                        const int r = top[i], x = r & 7;
+                        if (cnts[i] < 2 || filled[x] >= hcap) continue;      // a row used once gains nothing
+                        hotrows[(size_t)x * hcap + filled[x]] = r;
+                        rows.push_back(r);
+                        ranks.push_back(filled[x]++);
+                    }
+                    if (!rows.empty()) {
+                        PB_CHECK(hipMalloc((void**)&plan->hotrows, sizeof(int) * hotrows.size()));
+                        PB_CHECK(hipMemcpy(plan->hotrows, hotrows.data(), sizeof(int) * hotrows.size(), hipMemcpyHostToDevice));
+                        plan->hcap = (int)hcap;
+                        plan->index_bytes += sizeof(int) * hotrows.size();
+                        hotrank = crank;
+                        PB_CHECK(fill_i32(hotrank, nrows, -1, s));
+                        // the two small lists ride in the (still free) coverage area
+                        int* d_rows = reinterpret_cast<int*>(colpos_out);
+                        int* d_ranks = d_rows + rows.size();
+                        PB_CHECK(hipMemcpy(d_rows, rows.data(), sizeof(int) * rows.size(), hipMemcpyHostToDevice));
+                        PB_CHECK(hipMemcpy(d_ranks, ranks.data(), sizeof(int) * ranks.size(), hipMemcpyHostToDevice));
+                        hipLaunchKernelGGL(k_scatter_rank, dim3(grid_for((long long)rows.size(), 1 << 30)), dim3(BM_BLOCK), 0, s,
+                                           (int)rows.size(), d_rows, d_ranks, hotrank);
+                    }
+                }
             }
         }
-        if (want) PB_CHECK(plan_build_classes(plan, ir, jc, s));
+        if (want) PB_CHECK(plan_build_classes(plan, ir, jc, hotrank, s));
     }
 
     // 2. heavy rows and their ranks

@@ -44,14 +44,19 @@ struct bidmat_plan {
     // Row-class ordering of every column (DDS through the plan). The eight XCDs have one L2 each;
     // when each of them gathers from the whole dense operand, all eight L2s end up holding the same
     // popular rows. Rows are dealt to eight classes (row & 7) and the nonzeros of every column are
-    // grouped by the class of their row (stored order kept inside a class); a workgroup that runs
+    // grouped by the class of their row (stored order kept inside a group); a workgroup that runs
     // on XCD x only touches class-x nonzeros, so every L2 caches one eighth of the rows.
     // Built when the pattern promises a gain (plan.hip: wants_classes) or when the option says so.
     int ncls = 0;                // 0: no class ordering; otherwise 8
     int maxlen = 0;              // longest column
     int* cir = nullptr;          // [nnz]         row of the p-th nonzero in class order
     int* cperm = nullptr;        // [nnz]         its position in the original CSC order
-    int* cptr = nullptr;         // [8*ncols + 1] start of (column c, class x) at cptr[8*c + x]
+    int* cptr = nullptr;         // [16*ncols + 1] column c, class x: hot-row nonzeros from cptr[16*c + 2*x],
+                                 //               the others from cptr[16*c + 2*x + 1]
+    // The most frequent rows of every class ("hot": at most hcap per class) are kept in LDS by the DDS
+    // kernel. For their nonzeros cir holds the row's rank among its class's hot rows, not the row.
+    int hcap = 0;                // hot rows per class the ordering was built for (0: none)
+    int* hotrows = nullptr;      // [8*hcap] row of rank h of class x at hotrows[x*hcap + h], -1 = unused
     // Values in plan order (optional, bidmat_plan_set_values): pvals[p] = data[perm[p]], so that
     // A*^S and row sums stream their values instead of fetching each one through perm.
     float* pvals = nullptr;

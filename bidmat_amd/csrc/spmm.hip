@@ -96,15 +96,22 @@ __device__ __forceinline__ void gather_chunk(const GatherArgs& a, int myrow, flo
                 vv[u] = lane_read(myval, src);
             }
             const float* ap = a.A + (size_t)r * (size_t)a.lda;
-#pragma unroll
-            for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
             if (!FULL || TILE) {
-                // past the end of the segment (or outside the tile): lane data is (row 0, value 0);
-                // drop the load so that a non-finite entry of A's column 0 cannot leak in as 0*inf.
+                // past the end of the segment (or outside the tile) no load is issued at all: the slot
+                // costs the memory pipeline nothing, and a non-finite entry of A's column 0 cannot
+                // leak in as 0*inf.
                 bool ok = FULL || (it * NG + g) < rem;
                 if (TILE) ok = ok && ((inmask >> (LPN == 64 ? it : g * LPN + it)) & 1ULL);
+                if (ok) {
 #pragma unroll
-                for (int i = 0; i < V; ++i) av[u][i] = ok ? av[u][i] : Vec<W>::zero();
+                    for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::zero();
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(ap + eld[i]);
             }
         }
 #pragma unroll

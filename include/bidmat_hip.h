@@ -331,8 +331,11 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "heavy_min" a row is cut by column panels when it averages at least this many nonzeros
  *              per panel (default 8)
  *   "col_classes" row-class ordering of the columns inside a plan, used by bidmat_dds_plan so that the
- *              eight L2s of the device cache disjoint rows: -1 = decide from the pattern (default),
- *              0 = never, 1 = always
+ *              eight L2s of the device cache disjoint rows: -1 = decide from the pattern and k_hint
+ *              (default; needs k_hint >= 256), 0 = never, 1 = always
+ *   "class_hot" most frequent rows per class that the class-ordered DDS kernel keeps in LDS: 0 = none
+ *              (default), -1 = as many as 128 KiB hold at the plan's k_hint, otherwise the number
+ *   "class_threads" workgroup size of that kernel when it keeps rows in LDS (256, 512 or 1024; default 1024)
  *   "class_strip" columns per wavefront in the class-ordered DDS kernel (default 16, 1..64)
  * Returns 0, or hipErrorInvalidValue for an unknown name / bad value; bidmat_get_option returns -2
  * for an unknown name. */

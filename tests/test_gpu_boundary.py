@@ -369,9 +369,13 @@ def test_class_ordered_dds_equals_plain_dds(hip, k):
     the strip, every strip width, beta 0 / 1 and the fused elementwise step."""
     rng = np.random.default_rng(88 + k)
     old_cls, old_strip = hip.bidmat_get_option(b"col_classes"), hip.bidmat_get_option(b"class_strip")
+    old_hot = hip.bidmat_get_option(b"class_hot")
     hip_abi.check(hip.bidmat_set_option(b"col_classes", 1))
     try:
-        for variant in ("mixed", "one_class", "two_rows"):
+        # hot rows per class kept in LDS: none (everything gathered from memory), two (both kinds of
+        # nonzero in most columns), as many as fit (with "two_rows": every nonzero is a hot one)
+        for variant, hot in (("mixed", 0), ("mixed", 2), ("mixed", -1), ("one_class", 3), ("two_rows", -1), ("two_rows", 0)):
+            hip_abi.check(hip.bidmat_set_option(b"class_hot", hot))
             nrows, ncols = 700, 333
             lengths = rng.integers(0, 90, size=ncols)
             lengths[0], lengths[5], lengths[332] = 0, 700, 130
@@ -401,15 +405,18 @@ def test_class_ordered_dds_equals_plain_dds(hip, k):
                 hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, 3, q2.ptr, 0, None))
                 hip_abi.check(hip.bidmat_synchronize())
                 assert np.array_equal(q1.numpy(), q2.numpy(), equal_nan=True), (variant, strip)
+            # the pattern arrays and the dense operands are inputs only
+            assert np.array_equal(d.ir.numpy(), ir) and np.array_equal(d.A.numpy(), A)
             ref64, sa = oracle.dds_f64(A, B, k, ir, jc)
             hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, None, 0, p2.ptr, 0, None))
             hip_abi.check(hip.bidmat_synchronize())
-            close(p2.numpy(), ref64, sa, "class-ordered DDS k=%d %s" % (k, variant))
+            close(p2.numpy(), ref64, sa, "class-ordered DDS k=%d %s hot=%d" % (k, variant, hot))
             hip_abi.check(hip.bidmat_plan_destroy(plan))
             d.free()
     finally:
         hip_abi.check(hip.bidmat_set_option(b"col_classes", old_cls))
         hip_abi.check(hip.bidmat_set_option(b"class_strip", old_strip))
+        hip_abi.check(hip.bidmat_set_option(b"class_hot", old_hot))
 
 
 def test_config2_dds_pure_relative_error(hip):
