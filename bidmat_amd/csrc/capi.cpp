@@ -25,8 +25,10 @@ std::atomic<int> g_col_classes{-1};
 std::atomic<int> g_class_strip{16};
 std::atomic<int> g_class_hot{0};
 std::atomic<int> g_class_threads{1024};
+std::atomic<int> g_class_phases{2};
 }  // namespace
 int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
+int opt_class_phases() { return g_class_phases.load(std::memory_order_relaxed); }
 int opt_class_hot() { return g_class_hot.load(std::memory_order_relaxed); }
 int opt_class_strip() { return g_class_strip.load(std::memory_order_relaxed); }
 int opt_col_classes() { return g_col_classes.load(std::memory_order_relaxed); }
@@ -393,6 +395,10 @@ API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (k == 0 || plan->ncols == 0) return 0;
     if (!Sjc || !C || (plan->nnz > 0 && (!A || !Sdata || !Sir))) return kInvalid;
+    const int nphase = bm::opt_class_phases();
+    if (plan->ncls == 8 && plan->hcap == 0 && nphase > 0 && plan->maxlen <= kMaxClassedColumn && plan->nnz > 0)
+        return (int)bm::dsmult_phased(k, plan->ncols, A, Sdata, plan->cir, plan->cperm, plan->cptr, nphase, C, beta,
+                                      as_stream(stream));
     if (plan->novf > 0) {
         hipError_t err = bm::plan_reserve_ovf_partial(plan, k);
         if (err != hipSuccess) return (int)err;
@@ -750,6 +756,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_heavy_min.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "class_phases")) {
+        if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8) return kInvalid;
+        bm::g_class_phases.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "class_threads")) {
         if (value != 256 && value != 512 && value != 1024) return kInvalid;
         bm::g_class_threads.store((int)value);
@@ -782,6 +793,7 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "class_strip")) return bm::opt_class_strip();
     if (!strcmp(name, "class_hot")) return bm::opt_class_hot();
     if (!strcmp(name, "class_threads")) return bm::opt_class_threads();
+    if (!strcmp(name, "class_phases")) return bm::opt_class_phases();
     return -2;
 }
 

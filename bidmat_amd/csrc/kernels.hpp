@@ -10,6 +10,7 @@ int opt_seglen();      // nonzeros per wave segment for long columns / rows
 int opt_panel_kb();    // KiB of A per column panel in a plan
 int opt_heavy_min();   // a row is cut by panels when it averages at least this many nonzeros per panel
 int opt_class_threads(); // workgroup size of the class-ordered DDS kernel when it keeps hot rows in LDS (256, 512, 1024)
+int opt_class_phases(); // passes of A*S over a class-ordered pattern (1, 2, 4, 8), 0 = plain kernel
 int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..64)
 int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: 0 = none (default), -1 = what 128 KiB hold
 int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always
@@ -70,6 +71,10 @@ hipError_t dsmult_csc(int k, int ncols, int nnz, const float* A, const float* va
 hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const float* A, const float* vals,
                          const int* ir, const int* jc, float* C, int beta, Window rows, hipStream_t s,
                          const ColTable* tab = nullptr);
+// A*S on a plan's class-ordered pattern (cir / cperm / cptr with 16 groups per column, no hot-row
+// ranks) in nphase passes over disjoint row classes; see spmm.hip.
+hipError_t dsmult_phased(int k, int ncols, const float* A, const float* vals, const int* cir, const int* cperm,
+                         const int* cptr, int nphase, float* C, int beta, hipStream_t s);
 // ---- DDS (dds.hip)
 // V != nullptr: P[j] = op(V[j], dot_j) with the BinOp code opn (beta must be 0) - the elementwise
 // step that follows DDS in an NMF update, applied before the result leaves the registers.

@@ -42,6 +42,9 @@ struct GatherArgs {
     float* out;          // C (CSC mode) / partial (plan mode)
     float* partial;      // CSC mode: partial sums of overflow segments
     int xcd_start[9];    // plan mode: segment groups per XCD, light segments from xcd_start[8]
+    // CSC mode on a class-ordered pattern: the wave of column w takes the nonzeros
+    // [ptr[w*pstride + poff], ptr[w*pstride + poff + pspan]) (plain CSC: 1, 0, 1)
+    int pstride, poff, pspan;
 };
 
 template <int V, int LPN>
@@ -57,7 +60,7 @@ __device__ __forceinline__ void load_chunk(const GatherArgs& a, int j0, int ahea
     if (q < rem) {
         const int p = j0 + ahead + q;
         myrow = a.idx[p];
-        myval = (PLAN && a.perm != nullptr) ? a.vals[a.perm[p]] : a.vals[p];     // perm == nullptr: values already in plan order
+        myval = a.perm != nullptr ? a.vals[a.perm[p]] : a.vals[p];     // perm == nullptr: vals is in the order of idx
     }
 }
 
@@ -168,7 +171,8 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
         outp = a.out + (size_t)seg * (size_t)a.k;
         accumulate = false;
     } else if (w < a.nfirst) {
-        const int s = a.ptr[w], e = a.ptr[w + 1];
+        const long long pi = w * a.pstride + a.poff;
+        const int s = a.ptr[pi], e = a.ptr[pi + a.pspan];
         jstart = s;
         jend = (e - s > a.seglen) ? s + a.seglen : e;
         outp = a.out + (size_t)w * (size_t)a.ldo;
@@ -403,6 +407,7 @@ void init_args(GatherArgs& a) {
     a.win_on = 0; a.win_off = 0; a.win_len = 0;
     a.segrow = nullptr; a.row_off = 0; a.row_len = 0;
     for (int x = 0; x < 9; ++x) a.xcd_start[x] = 0;
+    a.pstride = 1; a.poff = 0; a.pspan = 1;
 }
 }  // namespace
 
@@ -449,6 +454,33 @@ hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const floa
         err = hipGetLastError();
     }
     return err;
+}
+
+// A*S over a class-ordered pattern in `nphase` passes, one launch each: pass p only gathers the rows
+// of classes [8*p/nphase, 8*(p+1)/nphase), and the passes follow each other on the stream. While
+// a pass runs, every L2 of the device only sees that pass's share of the rows, so it holds
+// nphase times as many of the rows that matter as when all rows compete for it; the price is one
+// read-modify-write of C per extra pass. The order of the additions (pass by pass, class by class,
+// stored order inside a class) depends on the pattern alone.
+hipError_t dsmult_phased(int k, int ncols, const float* A, const float* vals, const int* cir, const int* cperm,
+                         const int* cptr, int nphase, float* C, int beta, hipStream_t s) {
+    if (k <= 0 || ncols <= 0) return hipSuccess;
+    if (nphase != 1 && nphase != 2 && nphase != 4 && nphase != 8) return hipErrorInvalidValue;
+    const bool al = aligned16(A) && aligned16(C);
+    Shape sh = clamp_shape(pick_shape(k, al));
+    GatherArgs a;
+    init_args(a);
+    a.k = k; a.lda = k; a.ldo = k; a.nfirst = ncols; a.seglen = 0x7fffffff;
+    a.A = A; a.vals = vals; a.idx = cir; a.perm = cperm; a.ptr = cptr; a.ovf = nullptr;
+    a.out = C; a.partial = nullptr;
+    a.pstride = 16; a.pspan = 16 / nphase;
+    for (int p = 0; p < nphase; ++p) {
+        a.poff = p * a.pspan;
+        a.beta = p == 0 ? beta : 1;
+        hipError_t err = launch_gather<false>(sh, a, (long long)ncols, s);
+        if (err != hipSuccess) return err;
+    }
+    return hipSuccess;
 }
 
 hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A, const float* vals,

@@ -184,8 +184,12 @@ int bidmat_plan_set_values(bidmat_plan *plan, const float *Sdata, void *stream);
 
 /* A*S and DDS through a plan: the plan holds what is a function of the pattern alone (whether any
  * column is longer than a wave segment, and the table of the extra segments if so), so a call is
- * one launch when no column is long, and never builds or allocates per call.  Same results, bit for
- * bit, as bidmat_dsmult_csc / bidmat_dds_csc / bidmat_dds_csc_op.  Sir / Sjc: the pattern the plan
+ * one launch when no column is long, and never builds or allocates per call.  bidmat_dds_plan gives
+ * the same results, bit for bit, as bidmat_dds_csc / bidmat_dds_csc_op, whichever kernel the plan
+ * selects; so does bidmat_dsmult_plan unless the plan carries a row-class ordering of its columns
+ * (see "col_classes" below): then the nonzeros of a column are added class by class instead of in
+ * stored order - a fixed order that depends on the pattern alone, so results repeat bit for bit
+ * from run to run, and stay within the 1e-4 tolerance of the path.  Sir / Sjc: the pattern the plan
  * was made from.  bidmat_dds_plan: V == NULL gives P = beta*P + DDS, otherwise P = op(V, DDS). */
 int bidmat_dsmult_plan(bidmat_plan *plan, int k, const float *A, const float *Sdata, const int *Sir,
                        const int *Sjc, float *C, int beta, void *stream);
@@ -336,6 +340,9 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "class_hot" most frequent rows per class that the class-ordered DDS kernel keeps in LDS: 0 = none
  *              (default), -1 = as many as 128 KiB hold at the plan's k_hint, otherwise the number
  *   "class_threads" workgroup size of that kernel when it keeps rows in LDS (256, 512 or 1024; default 1024)
+ *   "class_phases" passes of bidmat_dsmult_plan over a class-ordered pattern, each pass gathering a
+ *              disjoint share of the row classes so that the L2s hold more of the rows that matter
+ *              (1, 2, 4 or 8; default 2; 0 = always the plain one-pass kernel)
  *   "class_strip" columns per wavefront in the class-ordered DDS kernel (default 16, 1..64)
  * Returns 0, or hipErrorInvalidValue for an unknown name / bad value; bidmat_get_option returns -2
  * for an unknown name. */

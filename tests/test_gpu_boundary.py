@@ -405,6 +405,26 @@ def test_class_ordered_dds_equals_plain_dds(hip, k):
                 hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, 3, q2.ptr, 0, None))
                 hip_abi.check(hip.bidmat_synchronize())
                 assert np.array_equal(q1.numpy(), q2.numpy(), equal_nan=True), (variant, strip)
+            # A*S through the same plan: passes over disjoint row classes (only without hot-row ranks)
+            if hot == 0:
+                vals = (1.0 - rng.random(nnz)).astype(np.float32)
+                dv = DeviceArray.from_numpy(vals)
+                ref64, sa = oracle.fsmult_f64(A, k, vals, ir, jc)
+                old_ph = hip.bidmat_get_option(b"class_phases")
+                try:
+                    for phases in (0, 1, 2, 4, 8):
+                        hip_abi.check(hip.bidmat_set_option(b"class_phases", phases))
+                        for beta in (0, 1):
+                            C0 = rng.standard_normal(k * ncols).astype(np.float32)
+                            c1, c2 = DeviceArray.from_numpy(C0), DeviceArray.from_numpy(C0)
+                            hip_abi.check(hip.bidmat_dsmult_plan(plan, k, d.A.ptr, dv.ptr, d.ir.ptr, d.jc.ptr, c1.ptr, beta, None))
+                            hip_abi.check(hip.bidmat_dsmult_plan(plan, k, d.A.ptr, dv.ptr, d.ir.ptr, d.jc.ptr, c2.ptr, beta, None))
+                            hip_abi.check(hip.bidmat_synchronize())
+                            assert np.array_equal(c1.numpy(), c2.numpy())           # same bits run to run
+                            r, s_ = (ref64 + C0, sa + np.abs(C0)) if beta else (ref64, sa)
+                            close(c1.numpy(), r, s_, "A*S in %d passes, k=%d %s beta=%d" % (phases, k, variant, beta))
+                finally:
+                    hip_abi.check(hip.bidmat_set_option(b"class_phases", old_ph))
             # the pattern arrays and the dense operands are inputs only
             assert np.array_equal(d.ir.numpy(), ir) and np.array_equal(d.A.numpy(), A)
             ref64, sa = oracle.dds_f64(A, B, k, ir, jc)
