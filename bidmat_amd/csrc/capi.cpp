@@ -23,7 +23,7 @@ std::atomic<int> g_panel_kb{3072};
 std::atomic<int> g_heavy_min{8};
 std::atomic<int> g_col_classes{-1};
 std::atomic<int> g_class_strip{16};
-std::atomic<int> g_class_hot{0};
+std::atomic<int> g_class_hot{-1};
 std::atomic<int> g_class_threads{1024};
 std::atomic<int> g_class_phases{2};
 }  // namespace
@@ -366,7 +366,7 @@ API int bidmat_plan_destroy(bidmat_plan* plan) {
 API long long bidmat_plan_bytes(const bidmat_plan* plan) {
     if (!plan) return 0;
     return (long long)(plan->index_bytes + (plan->partial_floats + plan->ovf_partial_floats) * sizeof(float) +
-                       (plan->pvals ? (size_t)plan->nnz * sizeof(float) : 0));
+                       ((plan->pvals ? 1 : 0) + (plan->cvals ? 1 : 0) + (plan->svals ? 1 : 0)) * (size_t)plan->nnz * sizeof(float));
 }
 
 API int bidmat_plan_segments(const bidmat_plan* plan) { return plan ? plan->nseg : 0; }
@@ -394,11 +394,14 @@ API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float
     if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (k == 0 || plan->ncols == 0) return 0;
-    if (!Sjc || !C || (plan->nnz > 0 && (!A || !Sdata || !Sir))) return kInvalid;
     const int nphase = bm::opt_class_phases();
-    if (plan->ncls == 8 && plan->hcap == 0 && nphase > 0 && plan->maxlen <= kMaxClassedColumn && plan->nnz > 0)
-        return (int)bm::dsmult_phased(k, plan->ncols, A, Sdata, plan->cir, plan->cperm, plan->cptr, nphase, C, beta,
-                                      as_stream(stream));
+    const bool phased = plan->ncls == 8 && plan->hcap == 0 && nphase > 0 && plan->maxlen <= kMaxClassedColumn && plan->nnz > 0;
+    if (!Sdata && !phased) return kInvalid;
+    // Sdata == NULL: the values stored by bidmat_plan_set_values, which exist in class order only
+    if (!Sjc || !C || (plan->nnz > 0 && (!A || !Sir || (!Sdata && !(phased && plan->cvals))))) return kInvalid;
+    if (phased)
+        return (int)bm::dsmult_phased(k, plan->ncols, A, Sdata ? Sdata : plan->cvals, plan->cir, Sdata ? plan->cperm : nullptr,
+                                      plan->cptr, nphase, C, beta, as_stream(stream));
     if (plan->novf > 0) {
         hipError_t err = bm::plan_reserve_ovf_partial(plan, k);
         if (err != hipSuccess) return (int)err;
@@ -407,20 +410,38 @@ API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float
     return (int)bm::dsmult_csc(k, plan->ncols, plan->nnz, A, Sdata, Sir, Sjc, C, beta, as_stream(stream), &tab);
 }
 
-API int bidmat_dds_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc,
-                        const float* V, int opn, float* P, int beta, void* stream) {
+namespace {
+// DDS through a plan. stored: the epilogue operand is the plan's stored values (V ignored).
+int dds_through_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc, const float* V,
+                     bool stored, int opn, float* P, int beta, void* stream) {
     auto lock = bm::device_lock();
     if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
-    if (V && (beta != 0 || opn < 0 || opn > 14)) return kInvalid;
+    if ((V || stored) && (beta != 0 || opn < 0 || opn > 14)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (plan->ncols == 0 || plan->nnz == 0) return 0;
     if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
-    if (plan->ncls == 8 && k > 0 && plan->maxlen <= kMaxClassedColumn &&
-        (size_t)plan->hcap * (size_t)k * sizeof(float) <= bm::dds_classed_lds_budget())
+    const bool classed = plan->ncls == 8 && k > 0 && plan->maxlen <= kMaxClassedColumn &&
+                         (size_t)plan->hcap * (size_t)k * sizeof(float) <= bm::dds_classed_lds_budget();
+    if (stored) {
+        V = plan->ncls == 8 ? (classed ? plan->cvals : nullptr) : plan->svals;
+        if (!V) return kInvalid;              // bidmat_plan_set_values has not been called (or k does not fit the ordering)
+    }
+    if (classed)
         return (int)bm::dds_classed(k, plan->ncols, A, B, plan->cir, plan->cperm, plan->cptr, plan->hcap, plan->hotrows, P, beta,
-                                    as_stream(stream), V, opn);
+                                    as_stream(stream), V, opn, stored);
     const bm::ColTable tab = col_table(plan);
     return (int)bm::dds_csc(k, plan->ncols, plan->nnz, A, B, Sir, Sjc, P, beta, as_stream(stream), V, opn, &tab);
+}
+}  // namespace
+
+API int bidmat_dds_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc,
+                        const float* V, int opn, float* P, int beta, void* stream) {
+    return dds_through_plan(plan, k, A, B, Sir, Sjc, V, false, opn, P, beta, stream);
+}
+
+API int bidmat_dds_plan_stored(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc,
+                               int opn, float* P, void* stream) {
+    return dds_through_plan(plan, k, A, B, Sir, Sjc, nullptr, true, opn, P, 0, stream);
 }
 
 API int bidmat_plan_set_values(bidmat_plan* plan, const float* Sdata, void* stream) {

@@ -99,7 +99,7 @@ __device__ __forceinline__ float dds_round(const float* __restrict__ A, int k, i
 template <int W, int V, int LPN, bool EXACT, bool FULL, bool LDSROWS = false>
 __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, int myrow, float* o, int rem, int g,
                                           int l, const int (&eld)[V], const bool (&ev)[V],
-                                          const Vec<W> (&b)[V], bool accumulate, const float* vq, int opn) {
+                                          const Vec<W> (&b)[V], bool accumulate, bool apply, float vval, int opn) {
     constexpr int NG = 64 / LPN;
     constexpr int U = Unroll<V, LPN>::U;
     const int q = l * NG + g;            // the nonzero of this chunk whose result this lane keeps
@@ -122,7 +122,7 @@ __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, in
     }
     if (FULL || q < rem) {                                        // o: where this lane's nonzero goes
         if (accumulate) res += *o;
-        if (vq != nullptr) res = binop_rt(opn, *vq, res);         // only on the last pass over k
+        if (apply) res = binop_rt(opn, vval, res);               // only on the last pass over k
         *o = res;
     }
 }
@@ -178,9 +178,11 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
         while (rem > 0) {
             const int nrow = (q < rem - 64) ? a.ir[j0 + 64 + q] : 0;
             float* o = a.P + j0 + q;
-            const float* vq = (a.V != nullptr && k0 + KT >= a.k) ? a.V + j0 + q : nullptr;
-            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, vq, a.opn);
-            else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, vq, a.opn);
+            // the epilogue's operand is requested before the gathers, so that it is there when they are done
+            const bool apply = a.V != nullptr && k0 + KT >= a.k;
+            const float vval = (apply && q < rem) ? a.V[j0 + q] : 0.f;
+            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
+            else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
             crow = nrow;
             j0 += 64;
             rem -= 64;
@@ -208,6 +210,7 @@ struct DdsClassedArgs {
     const float* A;
     const float* B;
     const float* V;
+    int v_classed;       // V is in class order (indexed like cir), not in stored order (indexed through cperm)
     const int* cir;
     const int* cperm;
     const int* cptr;
@@ -226,9 +229,10 @@ __device__ __forceinline__ void dds_classed_run(const DdsClassedArgs& a, int jst
         int nrow = 0, npos = 0;
         if (q < rem - 64) { nrow = a.cir[j0 + 64 + q]; npos = a.cperm[j0 + 64 + q]; }
         float* o = a.P + cpos;
-        const float* vq = (a.V != nullptr && last) ? a.V + cpos : nullptr;
-        if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true, LDSROWS>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, vq, a.opn);
-        else dds_chunk<W, V, LPN, EXACT, false, LDSROWS>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, vq, a.opn);
+        const bool apply = a.V != nullptr && last;
+        const float vval = (apply && q < rem) ? (a.v_classed ? a.V[j0 + q] : a.V[cpos]) : 0.f;     // requested before the gathers
+        if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true, LDSROWS>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
+        else dds_chunk<W, V, LPN, EXACT, false, LDSROWS>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
         crow = nrow; cpos = npos;
         j0 += 64;
         rem -= 64;
@@ -404,7 +408,7 @@ size_t dds_classed_lds_budget() { return CL_LDS_MAX; }
 
 hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const int* cir, const int* cperm,
                        const int* cptr, int hcap, const int* hotrows, float* P, int beta, hipStream_t s,
-                       const float* V, int opn) {
+                       const float* V, int opn, bool v_classed) {
     if (ncols <= 0 || k <= 0) return hipErrorInvalidValue;          // callers route those cases to dds_csc
     if (V != nullptr && (beta != 0 || opn < 0 || opn > 14)) return hipErrorInvalidValue;
     const size_t lds_bytes = (size_t)hcap * (size_t)k * sizeof(float);
@@ -415,7 +419,7 @@ hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const i
     DdsClassedArgs a;
     a.k = k; a.ncols = ncols; a.beta = beta; a.opn = opn; a.hcap = hcap;
     a.strip = (int)opt_class_strip();
-    a.A = A; a.B = B; a.V = V; a.cir = cir; a.cperm = cperm; a.cptr = cptr; a.hotrows = hotrows; a.P = P;
+    a.A = A; a.B = B; a.V = V; a.v_classed = v_classed ? 1 : 0; a.cir = cir; a.cperm = cperm; a.cptr = cptr; a.hotrows = hotrows; a.P = P;
     return launch_dds_classed(sh, exact, a, lds_bytes, s);
 }
 

@@ -97,6 +97,11 @@ JFN(jint, ddsPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong B, jlong 
                             P(const float, V), opn, P(float, Pv), beta, nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
+JFN(jint, ddsPlanStored)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong B, jlong Sir, jlong Sjc, jint opn, jlong Pv) {
+    int e = bidmat_dds_plan_stored(P(bidmat_plan, plan), k, P(const float, A), P(const float, B), P(const int, Sir), P(const int, Sjc),
+                                   opn, P(float, Pv), nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
 JFN(jint, planSetValues)(JNIEnv*, jclass, jlong plan, jlong Sdata) {
     int e = bidmat_plan_set_values(P(bidmat_plan, plan), P(const float, Sdata), nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);

@@ -12,7 +12,7 @@ int opt_heavy_min();   // a row is cut by panels when it averages at least this 
 int opt_class_threads(); // workgroup size of the class-ordered DDS kernel when it keeps hot rows in LDS (256, 512, 1024)
 int opt_class_phases(); // passes of A*S over a class-ordered pattern (1, 2, 4, 8), 0 = plain kernel
 int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..64)
-int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: 0 = none (default), -1 = what 128 KiB hold
+int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: -1 = by k_hint (default), 0 = none
 int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always
 
 // ---- CSC utilities (csc_util.hip)
@@ -82,12 +82,12 @@ hipError_t dds_csc(int k, int ncols, int nnz, const float* A, const float* B, co
                    const int* jc, float* P, int beta, hipStream_t s, const float* V = nullptr, int opn = 0,
                    const ColTable* tab = nullptr);
 // DDS over a row-class ordered pattern (a plan's cir / cperm / cptr); same results, bit for bit.
-// hcap / hotrows: the hot rows per class the ordering was built with. Fails with hipErrorInvalidValue
+// hcap / hotrows: the hot rows per class the ordering was built with. v_classed: V is in class order. Fails with hipErrorInvalidValue
 // when hcap rows of k floats do not fit the kernel's LDS budget (callers then use dds_csc).
 size_t dds_classed_lds_budget();
 hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const int* cir, const int* cperm,
                        const int* cptr, int hcap, const int* hotrows, float* P, int beta, hipStream_t s,
-                       const float* V = nullptr, int opn = 0);
+                       const float* V = nullptr, int opn = 0, bool v_classed = false);
 // The same with no allocation at all: the overflow table lives in a fixed device array of the
 // library (one copy per device). ncols may not exceed dds_static_max_cols().
 int dds_static_max_cols();

@@ -260,7 +260,7 @@ inline int bits_for(unsigned long long maxval) {
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
     hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals, p->cir, p->cperm, p->cptr, p->hotrows};
+    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals, p->cir, p->cperm, p->cptr, p->hotrows, p->cvals, p->svals};
     for (void* b : bufs)
         if (b && (f = hipFree(b)) != hipSuccess) e = f;
     delete p;
@@ -323,6 +323,23 @@ hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s) {
     }
     hipLaunchKernelGGL(k_permute_values, dim3(grid_for(((long long)p->nnz + 3) / 4, 8192)), dim3(BM_BLOCK), 0, s,
                        (long long)p->nnz, data, p->perm, p->pvals);
+    if (p->ncls == 8) {
+        // A*S in passes over row classes and the fused step of DDS read their values in class order
+        if (!p->cvals) {
+            hipError_t e = hipMalloc((void**)&p->cvals, sizeof(float) * (size_t)p->nnz);
+            if (e != hipSuccess) { (void)hipGetLastError(); p->cvals = nullptr; return e; }
+        }
+        hipLaunchKernelGGL(k_permute_values, dim3(grid_for(((long long)p->nnz + 3) / 4, 8192)), dim3(BM_BLOCK), 0, s,
+                           (long long)p->nnz, data, p->cperm, p->cvals);
+    } else {
+        // without a class ordering the fused step of DDS reads them in stored order: a plain copy
+        if (!p->svals) {
+            hipError_t e = hipMalloc((void**)&p->svals, sizeof(float) * (size_t)p->nnz);
+            if (e != hipSuccess) { (void)hipGetLastError(); p->svals = nullptr; return e; }
+        }
+        hipError_t e = hipMemcpyAsync(p->svals, data, sizeof(float) * (size_t)p->nnz, hipMemcpyDeviceToDevice, s);
+        if (e != hipSuccess) return e;
+    }
     return hipGetLastError();
 }
 
@@ -488,10 +505,11 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     {
         const int mode = opt_col_classes();              // -1 auto, 0 never, 1 always
         bool want = mode == 1;
-        // Measured (100 M nonzeros, Zipf(1.1) rows, k = 256): 5.53 -> 4.78 ms. With rows of 512 bytes
-        // (k = 128, 400 M nonzeros, Zipf(1.05)) the class-ordered kernel is bound by its instruction
-        // stream, not by the memory path, and loses (14.8 -> 16.1 ms): full-wave rows only.
-        const bool candidate = mode == 1 || (mode < 0 && ncols > 0 && nnz / ncols >= 64 && k_hint >= 256 &&
+        // Measured: 100 M nonzeros, Zipf(1.1) rows, k = 256: 5.53 -> 4.78 ms. With rows of 512 bytes
+        // (k = 128, 400 M nonzeros, Zipf(1.05)) the class-ordered kernel alone is bound by its
+        // instruction stream and loses (14.8 -> 16.1 ms), but wins with each class's most frequent rows
+        // in LDS (13.75 ms): below k = 256 the hot rows are switched on with the classes.
+        const bool candidate = mode == 1 || (mode < 0 && ncols > 0 && nnz / ncols >= 64 &&
                                              (long long)nrows * 4 * k_hint > (8LL << 20));
         int* hotrank = nullptr;
         if (candidate && (size_t)nrows <= (size_t)nnz) {
@@ -513,12 +531,12 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
                 PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
                 // at least a tenth of all gathers must move from "misses L2" to "hits L2"
                 if (mode < 0) want = (double)(h[1] - h[0]) >= 0.10 * (double)nnz;
-                // hot rows per class kept in LDS: off unless asked for (-1: what 128 KiB hold at k_hint).
-                // Measured: no gain at k = 256 (4.78 ms without, 4.85 ms with 128 rows per class: the
-                // 1024-thread persistent workgroups that share the LDS rows cost what the rows save);
-                // at k = 128 they recover the class-ordered kernel's loss (16.1 -> 14.1 ms, plain 14.8).
+                // hot rows per class kept in LDS. -1 (default): what 128 KiB hold when k_hint < 256, none
+                // from k = 256 on, where they were measured to change nothing (4.78 ms without, 4.85 ms with
+                // 128 rows per class: the 1024-thread persistent workgroups that share the LDS rows cost
+                // what the rows save).
                 long long hcap = opt_class_hot();
-                if (hcap < 0) hcap = (128LL << 10) / (4LL * k_hint);     // one workgroup of 1024 threads per CU
+                if (hcap < 0) hcap = k_hint < 256 ? (128LL << 10) / (4LL * k_hint) : 0;
                 if (hcap > 1024) hcap = 1024;
                 if (want && hcap > 0) {
                     const int ntop = (int)(8 * hcap < nrows ? 8 * hcap : nrows);

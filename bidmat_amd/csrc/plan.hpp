@@ -60,6 +60,8 @@ struct bidmat_plan {
     // Values in plan order (optional, bidmat_plan_set_values): pvals[p] = data[perm[p]], so that
     // A*^S and row sums stream their values instead of fetching each one through perm.
     float* pvals = nullptr;
+    float* cvals = nullptr;      // the same in class order (with a class ordering): cvals[p] = data[cperm[p]]
+    float* svals = nullptr;      // the same in stored (CSC) order (without a class ordering): a plain copy
 };
 
 namespace bm {

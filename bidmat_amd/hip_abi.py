@@ -37,6 +37,7 @@ SIGNATURES = {
     "bidmat_plan_set_values": (C.c_int, [vp, vp, vp]),
     "bidmat_dsmult_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp]),
     "bidmat_dds_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp, C.c_int, vp]),
+    "bidmat_dds_plan_stored": (C.c_int, [vp, C.c_int, vp, vp, vp, vp, C.c_int, vp, vp]),
     "bidmat_plan_overflow_segments": (C.c_int, [vp]),
     "bidmat_plan_create": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, C.POINTER(vp)]),
     "bidmat_plan_destroy": (C.c_int, [vp]),

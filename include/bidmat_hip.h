@@ -178,8 +178,10 @@ int bidmat_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *S
 
 /* The values of the pattern in plan order, stored in the plan (nnz floats): afterwards
  * bidmat_dsmultT_plan, bidmat_sdmult_plan and bidmat_spsum_rows_plan accept Sdata == NULL and stream
- * the stored values instead of fetching every value through the plan's permutation.  For callers
- * whose values stay the same over several calls (a data minibatch); call it again when they change. */
+ * the stored values instead of fetching every value through the plan's permutation; so does
+ * bidmat_dsmult_plan when the plan carries a row-class ordering of its columns (otherwise it needs
+ * Sdata).  For callers whose values stay the same over several calls (a data minibatch); call it
+ * again when they change. */
 int bidmat_plan_set_values(bidmat_plan *plan, const float *Sdata, void *stream);
 
 /* A*S and DDS through a plan: the plan holds what is a function of the pattern alone (whether any
@@ -195,6 +197,12 @@ int bidmat_dsmult_plan(bidmat_plan *plan, int k, const float *A, const float *Sd
                        const int *Sjc, float *C, int beta, void *stream);
 int bidmat_dds_plan(bidmat_plan *plan, int k, const float *A, const float *B, const int *Sir,
                     const int *Sjc, const float *V, int opn, float *P, int beta, void *stream);
+/* P = op(v, DDS) where v are the values stored in the plan by bidmat_plan_set_values (the data
+ * matrix of an NMF / LDA update stays the same over all iterations): like bidmat_dds_plan with V, but
+ * the kernel streams its copy of the values in the order it walks the nonzeros.
+ * hipErrorInvalidValue when no values are stored. */
+int bidmat_dds_plan_stored(bidmat_plan *plan, int k, const float *A, const float *B, const int *Sir,
+                           const int *Sjc, int opn, float *P, void *stream);
 /* Number of extra wave segments of the plan's long columns (0: every column fits one segment). */
 int bidmat_plan_overflow_segments(const bidmat_plan *plan);
 
@@ -336,9 +344,10 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *              per panel (default 8)
  *   "col_classes" row-class ordering of the columns inside a plan, used by bidmat_dds_plan so that the
  *              eight L2s of the device cache disjoint rows: -1 = decide from the pattern and k_hint
- *              (default; needs k_hint >= 256), 0 = never, 1 = always
- *   "class_hot" most frequent rows per class that the class-ordered DDS kernel keeps in LDS: 0 = none
- *              (default), -1 = as many as 128 KiB hold at the plan's k_hint, otherwise the number
+ *              (default), 0 = never, 1 = always
+ *   "class_hot" most frequent rows per class that the class-ordered DDS kernel keeps in LDS: -1 = as
+ *              many as 128 KiB hold when the plan's k_hint is below 256, none from 256 on (default),
+ *              0 = none, otherwise the number
  *   "class_threads" workgroup size of that kernel when it keeps rows in LDS (256, 512 or 1024; default 1024)
  *   "class_phases" passes of bidmat_dsmult_plan over a class-ordered pattern, each pass gathering a
  *              disjoint share of the row classes so that the L2s hold more of the rows that matter

@@ -344,10 +344,16 @@ def test_dds_with_fused_elementwise_step(hip, k):
             hip_abi.check(hip.bidmat_applyop_flat(d.V.ptr, R.ptr, two.ptr, nnz, opn, None))
             hip_abi.check(hip.bidmat_dds_csc_op(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, opn, one.ptr, None))
             hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, opn, viaplan.ptr, 0, None))
+            stored = DeviceArray.zeros(nnz)
+            if opn == 0:
+                assert hip.bidmat_dds_plan_stored(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, opn, stored.ptr, None) == 1   # nothing stored yet
+                hip_abi.check(hip.bidmat_plan_set_values(plan, d.V.ptr, None))
+            hip_abi.check(hip.bidmat_dds_plan_stored(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, opn, stored.ptr, None))
             hip_abi.check(hip.bidmat_synchronize())
             a, b, c = two.numpy(), one.numpy(), viaplan.numpy()
             assert np.array_equal(a, b, equal_nan=True), "op %d" % opn
             assert np.array_equal(a, c, equal_nan=True), "op %d (plan form)" % opn
+            assert np.array_equal(a, stored.numpy(), equal_nan=True), "op %d (values stored in the plan)" % opn
             if opn == 3:
                 r32, _, _ = oracle.dds(A, B, k, ir, jc)
                 r64, _ = oracle.dds_f64(A, B, k, ir, jc)
@@ -403,8 +409,12 @@ def test_class_ordered_dds_equals_plain_dds(hip, k):
                 q1, q2 = DeviceArray.zeros(nnz), DeviceArray.zeros(nnz)
                 hip_abi.check(hip.bidmat_dds_csc_op(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, 3, q1.ptr, None))
                 hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.V.ptr, 3, q2.ptr, 0, None))
+                q3 = DeviceArray.zeros(nnz)
+                hip_abi.check(hip.bidmat_plan_set_values(plan, d.V.ptr, None))
+                hip_abi.check(hip.bidmat_dds_plan_stored(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, 3, q3.ptr, None))
                 hip_abi.check(hip.bidmat_synchronize())
                 assert np.array_equal(q1.numpy(), q2.numpy(), equal_nan=True), (variant, strip)
+                assert np.array_equal(q1.numpy(), q3.numpy(), equal_nan=True), (variant, strip)
             # A*S through the same plan: passes over disjoint row classes (only without hot-row ranks)
             if hot == 0:
                 vals = (1.0 - rng.random(nnz)).astype(np.float32)
@@ -421,6 +431,12 @@ def test_class_ordered_dds_equals_plain_dds(hip, k):
                             hip_abi.check(hip.bidmat_dsmult_plan(plan, k, d.A.ptr, dv.ptr, d.ir.ptr, d.jc.ptr, c2.ptr, beta, None))
                             hip_abi.check(hip.bidmat_synchronize())
                             assert np.array_equal(c1.numpy(), c2.numpy())           # same bits run to run
+                            if phases > 0:      # values stored in the plan (class order): same bits as values passed in
+                                hip_abi.check(hip.bidmat_plan_set_values(plan, dv.ptr, None))
+                                c3 = DeviceArray.from_numpy(C0)
+                                hip_abi.check(hip.bidmat_dsmult_plan(plan, k, d.A.ptr, None, d.ir.ptr, d.jc.ptr, c3.ptr, beta, None))
+                                hip_abi.check(hip.bidmat_synchronize())
+                                assert np.array_equal(c1.numpy(), c3.numpy())
                             r, s_ = (ref64 + C0, sa + np.abs(C0)) if beta else (ref64, sa)
                             close(c1.numpy(), r, s_, "A*S in %d passes, k=%d %s beta=%d" % (phases, k, variant, beta))
                 finally:
