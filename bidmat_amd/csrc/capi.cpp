@@ -101,7 +101,8 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     if (!jc) return err;
     if ((err = bm::coo_compress_cols(ncols, nnz, ic, jc, s)) != hipSuccess) return err;
     bidmat_plan* p = nullptr;
-    if ((err = bm::plan_build(nrows, ncols, nnz, ir, jc, k_hint, &p)) != hipSuccess) return err;
+    // the reference-shaped entries only ever use the row side of a cached plan
+    if ((err = bm::plan_build(nrows, ncols, nnz, ir, jc, k_hint, &p, false)) != hipSuccess) return err;
     while (g_cache.size() >= kMaxCachedPlans) g_cache.pop_back();   // freed when its last user lets go
     g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, ir, ic, h[0], h[1], own(p)});
     *out = g_cache.front().plan;
@@ -383,6 +384,7 @@ API int bidmat_dsmultT_plan(bidmat_plan* plan, int k, const float* A, const floa
 
 namespace {
 // the plan's column table as the kernels take it
+// (plans made by bidmat_plan_create always carry the column side)
 bm::ColTable col_table(bidmat_plan* plan) {
     return bm::ColTable{plan->col_seglen, plan->ovf, (long long)plan->novf, plan->ovf_partial};
 }

@@ -372,7 +372,7 @@ static hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int
     } while (0)
 
 hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,
-                      bidmat_plan** out) {
+                      bidmat_plan** out, bool column_side) {
     *out = nullptr;
     // builds share the workspace arena of their device: one at a time
     static std::mutex build_mu;
@@ -429,7 +429,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     // column side: the overflow-segment table of the columns, kept only when a column is longer
     // than seglen
     plan->col_seglen = opt_seglen();
-    {
+    if (column_side) {
         int* tbl = nullptr;
         PB_CHECK(build_overflow_table(ncols, nnz, jc, plan->col_seglen, &tbl, s));
         if (tbl) {
@@ -503,7 +503,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     // and the nonzeros of the top n1 and top 8*n1 rows compared, n1 = rows of the operand per L2. The
     // same ranking names every class's hot rows, the ones the DDS kernel keeps in LDS.
     {
-        const int mode = opt_col_classes();              // -1 auto, 0 never, 1 always
+        const int mode = column_side ? opt_col_classes() : 0;       // -1 auto, 0 never, 1 always
         bool want = mode == 1;
         // Measured: 100 M nonzeros, Zipf(1.1) rows, k = 256: 5.53 -> 4.78 ms. With rows of 512 bytes
         // (k = 128, 400 M nonzeros, Zipf(1.05)) the class-ordered kernel alone is bound by its

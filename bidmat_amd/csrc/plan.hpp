@@ -65,8 +65,10 @@ struct bidmat_plan {
 };
 
 namespace bm {
+// column_side == false: only the row side (A*^S, row sums) is built - no column overflow table, no
+// class ordering - for callers that will never run A*S or DDS through the plan.
 hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,
-                      bidmat_plan** out);
+                      bidmat_plan** out, bool column_side = true);
 hipError_t plan_free(bidmat_plan* p);
 // Makes sure the plan's partial buffer holds nseg*k floats.
 hipError_t plan_reserve_partial(bidmat_plan* p, int k);
