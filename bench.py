@@ -42,9 +42,9 @@ HBM_PEAK_GBS = 8000.0
 # was taken on; it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dds", 100003320): (41.8e9, "bidmat_amd/csrc/dds.hip", "@DDS_SHA@",
+    ("headline", "dds", 100003320): (25.47e9, "bidmat_amd/csrc/dds.hip", "14e5b6251a964ba4",
                                      "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "@SPMM_SHA@",
+    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "11b833e92f55259c",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 
@@ -107,6 +107,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs (baseline timing and verification)")
     ap.add_argument("--cpu-sample", type=float, default=1.0,
                     help="fraction of the columns timed on the CPU (1.0 = the whole workload)")
+    ap.add_argument("--sections", default="probe,shaped,graph,stored",
+                    help="side measurements around the timed steps, comma-separated: probe (L2-resident and streaming "
+                         "rates for the bounded roofline), shaped (reference-shaped entries), graph (HIP-graph replay), "
+                         "stored (values stored in the plan); 'none' runs the timed steps only, which keeps a profiler's "
+                         "per-kernel averages clean")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain streaming kernel of known size (C = A + B on 3 x 1 GiB) "
                          "before the steps: the scale for rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
@@ -130,6 +135,7 @@ def main():
     mem = C.c_longlong(0)
     hip_abi.check(lib.bidmat_device_info(arch, 64, C.byref(cus), C.byref(mem)))
 
+    sections = set() if args.sections == "none" else set(args.sections.split(","))
     if args.workload == "footprint":
         return footprint_sweep(lib, args)
     if args.workload == "next":
@@ -187,7 +193,7 @@ def main():
         ]
         workload = "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), step = DDS, A*S, A*^S"
         metric = "algorithmic GB/s (gathered operand charged once per nonzero) and nnz/s for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
-        roof_op, roof_kernel = "dds", "k_dds<W=4,V=1,LPN=64> (one launch = DDS over the whole pattern)"
+        roof_op, roof_kernel = "dds", "k_dds_classed<W=4,V=1,LPN=64> (one launch = DDS over the whole pattern, class-ordered columns)"
     elif args.workload in ("C1", "C4"):
         d_A = up(cfg["A"])
         d_C = DeviceArray(k * ncols, np.float32)
@@ -213,7 +219,7 @@ def main():
         ]
         workload = "configs[4]: NMF update chain Q = V ./ DDS(W,H,V) (one fused launch), G = H *^ Q (dense row sums timed apart)"
         metric = "algorithmic GB/s (gathered operand charged once per nonzero) for the NMF update chain at k=128, ~400M nnz"
-        roof_op, roof_kernel = "dsmultT", "k_gather_axpy<W=4,V=1,LPN=32,plan>"
+        roof_op, roof_kernel = "dsmultT", "k_gather_axpy<W=4,V=1,LPN=32,plan> (stage 1 of A*^S)"
 
     def ev():
         e = C.c_void_p()
@@ -277,11 +283,13 @@ def main():
     # ---- what bounds the roofline kernel, measured on this device in this run: the rate of the
     # same gather kernel when the gathered rows fit in L2 (the ceiling of a kernel whose every gather
     # is served by L2), and the plain streaming rate of the device.
-    live = live_rates(lib, stream, k, "dds" if roof_op in ("dds", "dds_op") else "dsmult")
+    live = live_rates(lib, stream, k, "dds" if roof_op in ("dds", "dds_op") else "dsmult") if "probe" in sections else \
+        {"l2_resident_gather_GBps": None, "stream_GBps": None, "probe": None}
     r_avg, r_bytes = per_op[roof_op]["ms_avg"], alg_bytes(roof_op, k, nnz, nrows, ncols)
     r_comp = compulsory_bytes(roof_op, k, nnz, nrows, ncols)
     gathered = nnz * 4 * k
-    bound_ms = max(r_comp / (HBM_PEAK_GBS * 1e9), gathered / (live["l2_resident_gather_GBps"] * 1e9)) * 1e3
+    bound_ms = max(r_comp / (HBM_PEAK_GBS * 1e9), gathered / (live["l2_resident_gather_GBps"] * 1e9)) * 1e3 \
+        if live["l2_resident_gather_GBps"] else None
     traffic, traffic_src = measured_traffic(args.workload, roof_op, nnz)
     roofline = {
         "kernel": roof_kernel, "bound": "hbm", "achieved": round(r_bytes / r_avg / 1e6, 1), "peak": HBM_PEAK_GBS,
@@ -293,7 +301,7 @@ def main():
         "compulsory_bytes": r_comp, "gathered_bytes": gathered,
         "l2_resident_gather_GBps": live["l2_resident_gather_GBps"], "l2_resident_probe": live["probe"],
         "stream_GBps": live["stream_GBps"],
-        "bound_ms": round(bound_ms, 4), "frac_of_bound": round(bound_ms / r_avg, 4),
+        "bound_ms": round(bound_ms, 4) if bound_ms else None, "frac_of_bound": round(bound_ms / r_avg, 4) if bound_ms else None,
         "bound_basis": "max(compulsory bytes / 8 TB/s, gathered bytes / rate of the same kernel with an L2-resident operand)",
     }
     if traffic:
@@ -338,7 +346,7 @@ def main():
     # the outputs of the timed steps, checked below
     results = {name: d.numpy() for name, d in outputs.items()} if not args.no_cpu else {}
 
-    if args.workload == "headline":
+    if args.workload == "headline" and "shaped" in sections:
         # What unchanged call sites get: the blocking entries with the reference's argument lists
         # (per-nonzero column array, no column pointer, no plan handle), each preceded by the clear
         # of its output that GSMult / GSMultT / DDS do; wall clock around clear + call.
@@ -361,7 +369,7 @@ def main():
             shaped[name] = round(float(np.median(ts[1:])), 3)
         out["reference_shaped_ms_incl_clear"] = shaped
 
-    if args.workload == "headline":
+    if args.workload == "headline" and "stored" in sections:
         # Callers whose values stay fixed over several calls (the data matrix of an LDA minibatch) can
         # store them in the plan, in plan order: A*^S, A*S and the sparse row sums then stream them.
         d_rs = DeviceArray(nrows, np.float32)
@@ -374,7 +382,7 @@ def main():
             sv["dsmult_ms"] = round(_timed(lib, lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, None, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream), stream, 5), 4)
         out["values_stored_in_plan"] = sv
 
-    if args.workload in ("C1", "headline"):
+    if args.workload in ("C1", "headline") and "graph" in sections:
         # the same step recorded once into a HIP graph and replayed with one launch per step
         gx = C.c_void_p()
         hip_abi.check(lib.bidmat_graph_begin_capture(stream))
