@@ -103,6 +103,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="headline", choices=["headline", "C1", "C4", "C5", "next", "footprint"])
+    ap.add_argument("--footprint-k", type=int, default=256, help="k of the footprint sweep")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows/columns of the pattern (testing)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs (baseline timing and verification)")
     ap.add_argument("--cpu-sample", type=float, default=1.0,
@@ -467,22 +468,25 @@ def _timed(lib, fn, stream, reps, warm=2):
 
 
 def footprint_sweep(lib, args):
-    """DDS and A*S at k=256 on 100 000 columns x 200 nonzeros whose rows are uniform over R rows:
+    """DDS and A*S at k = --footprint-k (256) on 100 000 columns x 200 nonzeros whose rows are uniform over R rows:
     R KiB of gathered footprint, so the sweep shows what L1, L2, the Infinity Cache and HBM deliver."""
     from bidmat_amd import hip_abi
     from bidmat_amd.device import DeviceArray
-    k, ncols, L = 256, 100000, 200
+    k, ncols, L = args.footprint_k, 100000, 200
     nnz = ncols * L
     rng = np.random.default_rng(0)
     stream = C.c_void_p()
     hip_abi.check(lib.bidmat_stream_create(C.byref(stream)))
-    d_A = DeviceArray.from_numpy(rng.random(k * (1 << 20), dtype=np.float32))
+    k_rows_max = 1 << 20                      # A holds 2^20 rows of 256 floats: fewer rows fit when k is larger
+    d_A = DeviceArray.from_numpy(rng.random(256 * k_rows_max, dtype=np.float32))
     d_B = DeviceArray.from_numpy(rng.random(k * ncols, dtype=np.float32))
     d_v = DeviceArray.from_numpy(rng.random(nnz, dtype=np.float32))
     d_jc = DeviceArray.from_numpy((np.arange(ncols + 1) * L).astype(np.int32))
     d_P, d_C = DeviceArray(nnz, np.float32), DeviceArray(k * ncols, np.float32)
     rows = []
     for R in (16, 64, 256, 1024, 2048, 4096, 8192, 16384, 65536, 262144, 1048576):
+        if R * k > k_rows_max * 256:
+            break
         d_ir = DeviceArray.from_numpy(rng.integers(0, R, size=nnz).astype(np.int32))
         t_dds = _timed(lib, lambda: lib.bidmat_dds_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_P.ptr, 0, stream), stream, 5)
         t_as = _timed(lib, lambda: lib.bidmat_dsmult_csc(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream), stream, 5)
@@ -491,7 +495,7 @@ def footprint_sweep(lib, args):
                      "dds_TBps": round(b / t_dds / 1e9, 2), "dsmult_ms": round(t_as, 3),
                      "dsmult_TBps": round(b / t_as / 1e9, 2)})
         d_ir.free()
-    print(json.dumps({"metric": "gather throughput vs gathered footprint (algorithmic TB/s), k=256, 20M nnz",
+    print(json.dumps({"metric": "gather throughput vs gathered footprint (algorithmic TB/s), k=%d, 20M nnz" % k,
                       "unit": "TB/s", "n_gpus": 1, "sweep": rows}))
 
 
