@@ -26,8 +26,10 @@ std::atomic<int> g_class_strip{16};
 std::atomic<int> g_class_hot{-1};
 std::atomic<int> g_class_threads{1024};
 std::atomic<int> g_class_phases{2};
+std::atomic<int> g_plan_keep_mb{4096};
 }  // namespace
 int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
+int opt_plan_keep_mb() { return g_plan_keep_mb.load(std::memory_order_relaxed); }
 int opt_class_phases() { return g_class_phases.load(std::memory_order_relaxed); }
 int opt_class_hot() { return g_class_hot.load(std::memory_order_relaxed); }
 int opt_class_strip() { return g_class_strip.load(std::memory_order_relaxed); }
@@ -784,6 +786,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_class_phases.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "plan_keep_mb")) {
+        if (value < 0 || value > (1 << 20)) return kInvalid;
+        bm::g_plan_keep_mb.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "class_threads")) {
         if (value != 256 && value != 512 && value != 1024) return kInvalid;
         bm::g_class_threads.store((int)value);
@@ -817,6 +824,7 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "class_hot")) return bm::opt_class_hot();
     if (!strcmp(name, "class_threads")) return bm::opt_class_threads();
     if (!strcmp(name, "class_phases")) return bm::opt_class_phases();
+    if (!strcmp(name, "plan_keep_mb")) return bm::opt_plan_keep_mb();
     return -2;
 }
 

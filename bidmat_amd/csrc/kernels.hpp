@@ -12,6 +12,7 @@ int opt_heavy_min();   // a row is cut by panels when it averages at least this 
 int opt_class_threads(); // workgroup size of the class-ordered DDS kernel when it keeps hot rows in LDS (256, 512, 1024)
 int opt_class_phases(); // passes of A*S over a class-ordered pattern (1, 2, 4, 8), 0 = plain kernel
 int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..64)
+int opt_plan_keep_mb(); // plan-build temporaries up to this many MiB stay allocated for the next build
 int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: -1 = by k_hint (default), 0 = none
 int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always
 

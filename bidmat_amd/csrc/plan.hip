@@ -8,6 +8,9 @@
 #include "workspace.hpp"
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
+#include <rocprim/iterator/transform_iterator.hpp>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -27,23 +30,33 @@ struct Arena {
     }
 };
 
-// Build temporaries up to this size stay in the library's workspace for the next build;
-// larger ones are given back at once.
-constexpr size_t kKeepArenaBytes = size_t(512) << 20;
+// Build temporaries up to option "plan_keep_mb" (4096 MiB: what a 100 M-nonzero pattern needs) stay in the
+// library's workspace for the next build - a caller that meets a new pattern with every minibatch builds a plan
+// per call, and allocating and freeing 3.7 GB each time costs 0.9 of its 6.5 ms; larger ones are given back at
+// once. bidmat_release_caches frees the kept area.
 
 // Row histogram. The first HIST_LDS_ROWS rows are counted in a per-workgroup LDS copy that is
 // flushed once at the end (popular rows tend to carry small indices in count-sorted vocabularies,
 // and even when they do not this only costs the flush); all other rows go straight to global
 // integer atomics. The counts do not depend on the order of the increments.
+// The counts only steer choices that do not change any result (which rows are cut by panels, whether
+// the columns get a class ordering, which rows count as hot), so large patterns are counted on a
+// fixed pseudo-random eighth of their 256-nonzero chunks: sample = 8 keeps chunk ch when the top three
+// bits of ch * 0x9E3779B1 are zero, and every count is then about an eighth of the true one.
+// Row indices are checked here only as far as they are seen; k_make_keys checks every one.
 constexpr int HIST_LDS_ROWS = 16384;
-__global__ __launch_bounds__(BM_BLOCK) void k_row_hist(int nnz, int nrows, const int* __restrict__ ir,
+constexpr int HIST_SAMPLE = 8;
+constexpr long long HIST_SAMPLE_FROM = 16LL << 20;        // nonzeros from which the histogram is sampled
+__global__ __launch_bounds__(BM_BLOCK) void k_row_hist(int nnz, int nrows, int sample, const int* __restrict__ ir,
                                                        int* __restrict__ cnt, int* __restrict__ bad) {
     __shared__ int local[HIST_LDS_ROWS];
     for (int i = threadIdx.x; i < HIST_LDS_ROWS; i += BM_BLOCK) local[i] = 0;
     __syncthreads();
-    long long j = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    const long long stride = (long long)gridDim.x * BM_BLOCK;
-    for (; j < nnz; j += stride) {
+    const long long nchunks = ((long long)nnz + BM_BLOCK - 1) / BM_BLOCK;
+    for (long long ch = blockIdx.x; ch < nchunks; ch += gridDim.x) {
+        if (sample > 1 && (((unsigned)ch * 0x9E3779B1u) >> 29) != 0u) continue;
+        const long long j = ch * BM_BLOCK + threadIdx.x;
+        if (j >= nnz) continue;
         const int r = ir[j];
         if (r < 0 || r >= nrows) *bad = 1;
         else if (r < HIST_LDS_ROWS) atomicAdd(&local[r], 1);
@@ -84,7 +97,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_make_keys(int ncols, int nrows, co
                                                         const int* __restrict__ ir, const int* __restrict__ hcode,
                                                         int nheavy, int npanels,
                                                         int panel_cols, int p8, unsigned* __restrict__ keys,
-                                                        unsigned long long* __restrict__ colpos) {
+                                                        unsigned long long* __restrict__ colpos, int* __restrict__ bad) {
     const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long c = t >> 4;
     const int l = (int)(t & 15);
@@ -95,28 +108,47 @@ __global__ __launch_bounds__(BM_BLOCK) void k_make_keys(int ncols, int nrows, co
     const unsigned panel = (praw & 7u) * (unsigned)p8 + (praw >> 3);
     const unsigned light_base = 8u * (unsigned)p8 * (unsigned)nheavy;
     (void)npanels;
-    for (int j = s + l; j < e; j += 16) {
-        int r = ir[j];
-        r = r < 0 ? 0 : (r >= nrows ? nrows - 1 : r);
-        const int h = hcode[r];                         // heavy rank, or -1
-        keys[j] = h >= 0 ? panel * (unsigned)nheavy + (unsigned)h : light_base + (unsigned)r;
-        colpos[j] = ((unsigned long long)(unsigned)c << 32) | (unsigned)j;   // travels with the key
+    // four nonzeros per lane and step: the row loads, then the dependent code lookups, then the stores
+    constexpr int UN = 4;
+    for (int j0 = s + l; j0 < e; j0 += 16 * UN) {
+        int r[UN], h[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int j = j0 + 16 * u;
+            r[u] = j < e ? ir[j] : 0;
+            if ((unsigned)r[u] >= (unsigned)nrows) { *bad = 1; r[u] = 0; }
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) h[u] = hcode[r[u]];             // heavy rank, or -1
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int j = j0 + 16 * u;
+            if (j < e) {
+                keys[j] = h[u] >= 0 ? panel * (unsigned)nheavy + (unsigned)h[u] : light_base + (unsigned)r[u];
+                colpos[j] = ((unsigned long long)(unsigned)c << 32) | (unsigned)j;   // travels with the key
+            }
+        }
     }
 }
 
-__global__ __launch_bounds__(BM_BLOCK) void k_boundaries(int nnz, int seglen, const unsigned* __restrict__ keys,
-                                                         int* __restrict__ flag) {
-    long long p = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    const long long stride = (long long)gridDim.x * BM_BLOCK;
-    for (; p < nnz; p += stride)
-        flag[p] = (p == 0 || keys[p] != keys[p - 1] || (p % seglen) == 0) ? 1 : 0;
-}
+// 1 where a segment starts in the sorted key sequence: at a new key and every seglen positions.
+// Position n (one past the end) counts as 0, so an exclusive scan over n+1 positions ends with the
+// number of segments.
+struct SegmentStart {
+    const unsigned* keys;
+    unsigned n;
+    unsigned seglen;
+    __device__ __forceinline__ bool at(unsigned p) const {
+        return p == 0 || keys[p] != keys[p - 1] || (p % seglen) == 0;
+    }
+    __device__ __forceinline__ int operator()(unsigned p) const { return (p < n && at(p)) ? 1 : 0; }
+};
 
 // Column and original position of every nonzero in plan order; segment tables at the flagged
 // positions.
 __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __restrict__ keys,
                                                    const unsigned long long* __restrict__ colpos,
-                                                   const int* __restrict__ flag, const int* __restrict__ segidx,
+                                                   SegmentStart starts, const int* __restrict__ segidx,
                                                    const int* __restrict__ hrow, int nheavy, int p8,
                                                    int* __restrict__ pc, int* __restrict__ perm,
                                                    int* __restrict__ segstart,
@@ -130,7 +162,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_emit(int nnz, const unsigned* __re
         const unsigned long long cp = colpos[p];
         pc[p] = (int)(cp >> 32);
         perm[p] = (int)(cp & 0xffffffffULL);
-        if (flag[p]) {
+        if (starts.at((unsigned)p)) {
             const int sidx = segidx[p];
             const unsigned key = keys[p];
             segstart[sidx] = (int)p;
@@ -156,35 +188,41 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_bounds(int nseg, const unsig
 // row is one of its class's hot rows, else 1), then writes them out bucket by bucket, keeping the
 // stored order inside a bucket. cptr[16*c + b] = start of bucket b of column c; the last entry closes
 // the last column. For a hot row cir holds its rank among the hot rows of its class, otherwise the row.
-__global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, const int* __restrict__ ir,
+// HOT == false: no hot rows, the even buckets stay empty and only the eight classes are counted.
+template <bool HOT>
+__global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nrows, const int* __restrict__ ir,
                                                               const int* __restrict__ jc,
                                                               const int* __restrict__ hotrank,
                                                               int* __restrict__ cir,
                                                               int* __restrict__ cperm, int* __restrict__ cptr,
                                                               int* __restrict__ maxlen) {
+    constexpr int NB = HOT ? 16 : 8;
     const int lane = threadIdx.x & 63;
     const long long c = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
     if (c >= ncols) return;
     const int s = jc[c], e = jc[c + 1];
-    int cnt[16];
+    int cnt[NB];
 #pragma unroll
-    for (int x = 0; x < 16; ++x) cnt[x] = 0;
+    for (int x = 0; x < NB; ++x) cnt[x] = 0;
     for (int j0 = s; j0 < e; j0 += 64) {
         const int j = j0 + lane;
         const bool valid = j < e;
         const int r = valid ? ir[j] : 0;
-        const int hr = (valid && hotrank != nullptr) ? hotrank[r] : -1;
-        const int bucket = 2 * (r & 7) + (hr < 0 ? 1 : 0);
+        const int hr = (HOT && valid && (unsigned)r < (unsigned)nrows) ? hotrank[r] : -1;
+        const int bucket = HOT ? 2 * (r & 7) + (hr < 0 ? 1 : 0) : (r & 7);
 #pragma unroll
-        for (int x = 0; x < 16; ++x) cnt[x] += __popcll(__ballot(valid && bucket == x));
+        for (int x = 0; x < NB; ++x) cnt[x] += __popcll(__ballot(valid && bucket == x));
     }
-    int base[16], run = 0;
+    int base[NB], run = 0;
 #pragma unroll
-    for (int x = 0; x < 16; ++x) { base[x] = run; run += cnt[x]; }
+    for (int x = 0; x < NB; ++x) { base[x] = run; run += cnt[x]; }
     if (lane < 16) {
+        // table entry `lane` = start of bucket `lane` of the 16; without hot rows bucket 2x is empty and starts
+        // where bucket 2x+1 (class x) does
+        const int which = HOT ? lane : lane >> 1;
         int bb = 0;
 #pragma unroll
-        for (int x = 0; x < 16; ++x) bb = (lane == x) ? base[x] : bb;
+        for (int x = 0; x < NB; ++x) bb = (which == x) ? base[x] : bb;
         cptr[c * 16 + lane] = s + bb;
     }
     if (c == ncols - 1 && lane == 0) cptr[(long long)ncols * 16] = e;
@@ -196,11 +234,11 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, const i
         const int j = j0 + lane;
         const bool valid = j < e;
         const int r = valid ? ir[j] : 0;
-        const int hr = (valid && hotrank != nullptr) ? hotrank[r] : -1;
-        const int bucket = 2 * (r & 7) + (hr < 0 ? 1 : 0);
+        const int hr = (HOT && valid && (unsigned)r < (unsigned)nrows) ? hotrank[r] : -1;
+        const int bucket = HOT ? 2 * (r & 7) + (hr < 0 ? 1 : 0) : (r & 7);
         int dest = -1;
 #pragma unroll
-        for (int x = 0; x < 16; ++x) {
+        for (int x = 0; x < NB; ++x) {
             const bool mine = valid && bucket == x;
             const unsigned long long m = __ballot(mine);
             if (mine) dest = s + base[x] + __popcll(m & below);
@@ -356,8 +394,12 @@ static hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int
     int* d_maxlen = plan->cptr + nsub;                   // one spare int behind the table
     if ((e = fill_i32(d_maxlen, 1, 0, s)) != hipSuccess) return e;
     const long long nblk = ((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
-    hipLaunchKernelGGL(k_class_partition, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, ir, jc, hotrank, plan->cir,
-                       plan->cperm, plan->cptr, d_maxlen);
+    if (hotrank != nullptr)
+        hipLaunchKernelGGL(k_class_partition<true>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank,
+                           plan->cir, plan->cperm, plan->cptr, d_maxlen);
+    else
+        hipLaunchKernelGGL(k_class_partition<false>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank,
+                           plan->cir, plan->cperm, plan->cptr, d_maxlen);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if ((e = hipMemcpy(&plan->maxlen, d_maxlen, sizeof(int), hipMemcpyDeviceToHost)) != hipSuccess) return e;
     plan->ncls = 8;
@@ -457,11 +499,18 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
                                            (unsigned long long*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
         PB_CHECK(rocprim::radix_sort_pairs(nullptr, b2, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
                                            (int*)nullptr, (size_t)nnz, 0, rbits, s));
+        size_t b3 = 0;                                   // the scan over the segment starts
+        {
+            auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u),
+                                                       SegmentStart{nullptr, (unsigned)nnz, 1u});
+            PB_CHECK(rocprim::exclusive_scan(nullptr, b3, in, (int*)nullptr, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        }
         sort_bytes = b1 > b2 ? b1 : b2;
+        if (b3 > sort_bytes) sort_bytes = b3;
     }
     Arena tmp;
     int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *crank = nullptr, *scantmp = nullptr, *class_count = nullptr;
-    int *flag = nullptr, *segidx = nullptr;
+    int* segidx = nullptr;
     unsigned *keys_in = nullptr, *keys_out = nullptr;
     unsigned long long *colpos_in = nullptr, *colpos_out = nullptr;
     unsigned char* segclass = nullptr;
@@ -479,7 +528,6 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         keys_out = tmp.take<unsigned>((size_t)nnz);
         colpos_in = tmp.take<unsigned long long>((size_t)nnz);   // later: segment rows in sorted order
         colpos_out = tmp.take<unsigned long long>((size_t)nnz);
-        flag = tmp.take<int>((size_t)nnz);
         segidx = tmp.take<int>((size_t)nnz + 1);
         segclass = tmp.take<unsigned char>((size_t)nnz);
         sorttmp = tmp.take<char>(sort_bytes);
@@ -496,7 +544,8 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     PB_CHECK(fill_i32(cnt, nrows, 0, s));
     PB_CHECK(fill_i32(hrank + nrows, 2, 0, s));
     // few, long-lived workgroups: every one flushes its LDS histogram once at the end
-    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, ir, cnt, bad);
+    const int sample = (long long)nnz >= HIST_SAMPLE_FROM ? HIST_SAMPLE : 1;     // cnt[r] ~ (nonzeros of row r) / sample
+    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, sample, ir, cnt, bad);
 
     // 1b. column classes for DDS: worth it when one L2 (4 MiB) holds clearly fewer of the gathered
     // rows' nonzeros than eight L2s with disjoint rows would. The rows are sorted by count (descending)
@@ -530,7 +579,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
                 unsigned long long h[2] = {0, 0};
                 PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
                 // at least a tenth of all gathers must move from "misses L2" to "hits L2"
-                if (mode < 0) want = (double)(h[1] - h[0]) >= 0.10 * (double)nnz;
+                if (mode < 0) want = (double)(h[1] - h[0]) * sample >= 0.10 * (double)nnz;
                 // hot rows per class kept in LDS. -1 (default): what 128 KiB hold when k_hint < 256, none
                 // from k = 256 on, where they were measured to change nothing (4.78 ms without, 4.85 ms with
                 // 128 rows per class: the 1024-thread persistent workgroups that share the LDS rows cost
@@ -579,6 +628,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     if (plan->npanels >= 2) {
         long long thresh = (long long)plan->npanels * opt_heavy_min();
         if (thresh > 0x7fffffffLL) thresh = 0x7fffffffLL;
+        thresh = (thresh + sample - 1) / sample;
         hipLaunchKernelGGL(k_heavy_flag, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, cnt, (int)thresh, hflag);
         // the scan writes hrank[0..nrows]; the bad-index flag sits behind it
         PB_CHECK(scan_exclusive_i32(hflag, hrank, nrows, scantmp, s));
@@ -601,7 +651,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     {
         long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
         hipLaunchKernelGGL(k_make_keys, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nrows, jc, ir,
-                           hflag, nheavy, plan->npanels, plan->panel_cols, p8, keys_in, colpos_in);
+                           hflag, nheavy, plan->npanels, plan->panel_cols, p8, keys_in, colpos_in, bad);
     }
     const unsigned long long maxkey = 8ULL * (unsigned long long)p8 * nheavy + (unsigned long long)nrows;
     const int end_bit = bits_for(maxkey);
@@ -613,10 +663,21 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     }
 
     // 4. segment boundaries
-    hipLaunchKernelGGL(k_boundaries, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, plan->seglen, keys_out, flag);
-    PB_CHECK(scan_exclusive_i32(flag, segidx, nnz, scantmp, s));
+    const SegmentStart starts{keys_out, (unsigned)nnz, (unsigned)plan->seglen};
+    {
+        auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u), starts);
+        size_t tmp_bytes = 0;
+        PB_CHECK(rocprim::exclusive_scan(nullptr, tmp_bytes, in, segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        if (tmp_bytes > sort_bytes) { (void)plan_free(plan); return hipErrorOutOfMemory; }
+        PB_CHECK(rocprim::exclusive_scan(sorttmp, tmp_bytes, in, segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+    }
     int nseg = 0;
     PB_CHECK(hipMemcpy(&nseg, segidx + nnz, sizeof(int), hipMemcpyDeviceToHost));
+    {
+        int badv = 0;                                    // k_make_keys has seen every row index by now
+        PB_CHECK(hipMemcpy(&badv, bad, sizeof(int), hipMemcpyDeviceToHost));
+        if (badv) { (void)plan_free(plan); return hipErrorInvalidValue; }
+    }
     plan->nseg = nseg;
 
     // memory the plan keeps, part 2: the segment tables
@@ -640,7 +701,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
     unsigned* const segrow_u = reinterpret_cast<unsigned*>(plan->segrow);
     PB_CHECK(fill_i32(class_count, 9, nseg, s));
     hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out, colpos_out,
-                       flag, segidx, hrow, nheavy > 0 ? nheavy : 1,
+                       starts, segidx, hrow, nheavy > 0 ? nheavy : 1,
                        nheavy > 0 ? p8 : 0, plan->pc, plan->perm, plan->segstart, segrow_u, segid, segclass);
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
     hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg, segclass, class_count);
@@ -656,7 +717,7 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
         PB_CHECK(hipStreamSynchronize(s));
     }
     PB_CHECK(hipGetLastError());
-    if (arena_bytes > kKeepArenaBytes) PB_CHECK(ws_drop(WS_PLAN));
+    if (arena_bytes > ((size_t)opt_plan_keep_mb() << 20)) PB_CHECK(ws_drop(WS_PLAN));
     *out = plan;
     return hipSuccess;
 }

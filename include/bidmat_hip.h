@@ -353,6 +353,9 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *              disjoint share of the row classes so that the L2s hold more of the rows that matter
  *              (1, 2, 4 or 8; default 2; 0 = always the plain one-pass kernel)
  *   "class_strip" columns per wavefront in the class-ordered DDS kernel (default 16, 1..64)
+ *   "plan_keep_mb" temporaries of a plan build up to this many MiB stay allocated on the device for the
+ *              next build (default 4096: a 100 M-nonzero pattern needs 3.7 GB; 0 = always give them
+ *              back); bidmat_release_caches frees them
  * Returns 0, or hipErrorInvalidValue for an unknown name / bad value; bidmat_get_option returns -2
  * for an unknown name. */
 int bidmat_set_option(const char *name, long long value);

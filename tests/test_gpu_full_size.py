@@ -183,3 +183,35 @@ def test_config5_nmf_step(hip):
     ref = H.reshape(ncols, k).astype(np.float64).sum(axis=0)
     np.testing.assert_allclose(drs.numpy(), ref, rtol=1e-5)
     hip_abi.check(hip.bidmat_plan_destroy(plan))
+
+
+@pytest.mark.timeout(300)
+def test_large_pattern_with_one_bad_row_index_is_refused(hip):
+    """From 16 M nonzeros on the plan build counts rows on a sample of the nonzeros (the counts only
+    steer performance choices), but every row index is still checked: one index outside the matrix,
+    placed where the sampled histogram does not look (chunk 1 of 256 nonzeros: the top three bits of
+    1 * 0x9E3779B1 are not zero), must make bidmat_plan_create fail, and the sound pattern must build."""
+    nrows, ncols = 50000, 100000
+    ir, jc = gen.pattern(nrows, ncols, ("const", 200), ("zipf", 1.1), 77)
+    nnz = int(ir.size)
+    assert nnz >= (16 << 20)
+    assert ((1 * 0x9E3779B1) & 0xFFFFFFFF) >> 29 != 0
+    djc = DeviceArray.from_numpy(jc)
+    for bad in (nrows, -1):
+        broken = ir.copy()
+        broken[300] = bad
+        dbad = DeviceArray.from_numpy(broken)
+        plan = C.c_void_p()
+        rc = hip.bidmat_plan_create(nrows, ncols, nnz, dbad.ptr, djc.ptr, 256, C.byref(plan))
+        assert rc == 1 and not plan.value, "bad row index %d accepted (rc %d)" % (bad, rc)
+        dbad.free()
+    dir_ = DeviceArray.from_numpy(ir)
+    plan = make_plan(hip, nrows, ncols, nnz, dir_, djc, 256)
+    # the sampled counts still find the heavy rows: row sums through the plan equal the oracle's
+    vals = gen.uniform_open0(nnz, 5)
+    dv, dout = DeviceArray.from_numpy(vals), DeviceArray(nrows, np.float32)
+    hip_abi.check(hip.bidmat_spsum_rows_plan(plan, dv.ptr, dout.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    ref = np.bincount(ir, weights=vals.astype(np.float64), minlength=nrows)
+    assert np.allclose(dout.numpy(), ref, rtol=RTOL, atol=0)
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
