@@ -84,20 +84,22 @@ FMat::FMat(int nr, int nc, const float* src) : nrows(nr), ncols(nc), data(src, s
 SMat::SMat(int nr, int nc, int nnz) : nrows(nr), ncols(nc), ir((size_t)nnz), jc((size_t)nc + 1, Mat::ioneBased),
                                       data((size_t)nnz), GUID(Mat::newGUID()) {}
 
-void SMat::check() const {
+void SMat::check() const { checkArrays(nrows, ncols, nnz(), ir.data(), jc.data()); }
+
+void SMat::checkArrays(int nrows, int ncols, int nnz, const int* ir, const int* jc) {
     const int ioff = Mat::ioneBased;
     if (jc[0] != ioff) fail(fmt("jc(0) should be %d", ioff));
     for (int i = 0; i < ncols; ++i) {
         int j = jc[i] - ioff;
         if (jc[i] > jc[i + 1]) fail(fmt("jc(i) out of order %d %d %d", i, jc[i], jc[i + 1]));
-        while (j < jc[i + 1] - ioff - 1 && j + 1 < nnz()) {    // never read past the arrays
+        while (j < jc[i + 1] - ioff - 1 && j + 1 < nnz) {      // never read past the arrays
             if (ir[j + 1] <= ir[j]) fail(fmt("ir(j) out of order %d %d %d", j, ir[j], ir[j + 1]));
             if (ir[j] < ioff) fail(fmt("ir(%d)=%d too small", j, ir[j]));
             if (ir[j + 1] >= nrows + ioff) fail(fmt("ir(%d)=%d out of range %d", j + 1, ir[j + 1], nrows + ioff));
             ++j;
         }
     }
-    if (jc[ncols] != nnz() + ioff) fail(fmt("jc(ncols) should be %d", nnz()));
+    if (jc[ncols] != nnz + ioff) fail(fmt("jc(ncols) should be %d", nnz));
 }
 
 FMat SMat::full() const {
@@ -469,12 +471,16 @@ GSMatP GSMat::fromHost(int nr, int nc, int n, const float* data, const int* ir, 
 // smaller, so that is what crosses PCIe. The index base is added while the staging buffers are drained.
 SMat GSMat::toSMat() const {
     SMat out(nrows, ncols, nnz0);
+    toHost(out.data.data(), out.ir.data(), out.jc.data());
+    return out;
+}
+
+void GSMat::toHost(float* data, int* ir, int* jc) const {
     const int ioff = Mat::ioneBased;
     Staging st;
-    st.download(out.jc.data(), pjc, sizeof(int) * ((size_t)ncols + 1), ioff);
-    st.download(out.ir.data(), pir, sizeof(int) * (size_t)nnz0, ioff);
-    st.download(out.data.data(), pdata, sizeof(float) * (size_t)nnz0);
-    return out;
+    st.download(jc, pjc, sizeof(int) * ((size_t)ncols + 1), ioff);
+    st.download(ir, pir, sizeof(int) * (size_t)nnz0, ioff);
+    st.download(data, pdata, sizeof(float) * (size_t)nnz0);
 }
 
 GMatP GSMat::contents() {

@@ -61,6 +61,8 @@ public:
     int nnz() const { return (int)data.size(); }
     // SparseMat.check (SparseMat.scala:710-740): throws with the reference's messages
     void check() const;
+    // the same on caller-owned arrays (index base Mat::ioneBased)
+    static void checkArrays(int nrows, int ncols, int nnz, const int* ir, const int* jc);
     FMat full() const;
     std::string mytype() const { return "SMat"; }
 };
@@ -171,6 +173,8 @@ public:
     // ncats0 == 0: rows = largest category + 1  (GSMat.scala:686-720)
     static GSMatP nHot(const std::vector<int>& cats, int n, int ncols, int ncats0);
     SMat toSMat() const;                                         // GSMat.scala:108-127
+    // the same into caller-owned arrays (nnz values, nnz rows, ncols+1 column pointers, base Mat::ioneBased)
+    void toHost(float* data, int* ir, int* jc) const;
     GMatP contents();                                            // GSMat.scala:21-25
     GSMat& clear();
     void free();

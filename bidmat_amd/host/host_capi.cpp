@@ -59,11 +59,8 @@ API int bmh_gsmat_dims(void* h, int* nr, int* nc, int* nnz) {
 // copies the matrix back as a host SMat and runs SparseMat.check on it
 API int bmh_gsmat_to_host(void* h, float* data, int* ir, int* jc) {
     return guard_int([&] {
-        SMat a = S(h)->toSMat();
-        a.check();
-        memcpy(data, a.data.data(), sizeof(float) * a.data.size());
-        memcpy(ir, a.ir.data(), sizeof(int) * a.ir.size());
-        memcpy(jc, a.jc.data(), sizeof(int) * a.jc.size());
+        S(h)->toHost(data, ir, jc);
+        SMat::checkArrays(S(h)->nrows, S(h)->ncols, S(h)->nnz(), ir, jc);
     });
 }
 // the device column pointer, 0-based (to check that DDS results carry it)
