@@ -56,6 +56,16 @@ def test_no_compute_without_gpu_helpers_work():
     assert lib.bidmat_get_option(b"seglen") >= 64
     assert lib.bidmat_set_option(b"seglen", 1) == 1            # rejected, unchanged
     assert lib.bidmat_set_option(b"nonsense", 5) == 1
+    assert lib.bidmat_get_option(b"nonsense") == -2
+    # every documented option: default inside its range, a set/get round trip, out-of-range values refused
+    for name, good, bad in ((b"seglen", 512, 0), (b"panel_kb", 1024, 1), (b"heavy_min", 4, 0), (b"col_classes", 1, 2),
+                            (b"class_hot", 16, 5000), (b"class_threads", 512, 300), (b"class_strip", 8, 65),
+                            (b"class_phases", 4, 3), (b"plan_keep_mb", 0, -1)):
+        old = lib.bidmat_get_option(name)
+        assert old != -2, name
+        assert lib.bidmat_set_option(name, bad) == 1 and lib.bidmat_get_option(name) == old, name
+        assert lib.bidmat_set_option(name, good) == 0 and lib.bidmat_get_option(name) == good, name
+        assert lib.bidmat_set_option(name, old) == 0
     assert lib.bidmat_error_string(0)
     # argument validation happens before any device work
     assert lib.bidmat_dsmult(-1, 1, 1, None, None, None, None, None) == 1
