@@ -42,9 +42,9 @@ HBM_PEAK_GBS = 8000.0
 # was taken on; it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dds", 100003320): (25.47e9, "bidmat_amd/csrc/dds.hip", "14e5b6251a964ba4",
+    ("headline", "dds", 100003320): (25.46e9, "bidmat_amd/csrc/dds.hip", "2b6c7d772c9cbfcf",
                                      "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "11b833e92f55259c",
+    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "4df7d618119c5dec",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 

@@ -111,25 +111,33 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     return hipSuccess;
 }
 
+// The nseg*k partial sums of one call through a plan: scratch of the stream the call runs on, so a plan holds
+// pattern data only and calls on different streams do not meet.
+float* row_partial(const bidmat_plan* plan, int k, hipStream_t s, hipError_t* err) {
+    return (float*)bm::ws_get(bm::WS_ROWPARTIAL, sizeof(float) * (size_t)plan->nseg * (size_t)k, err, s);
+}
+
 // vals == nullptr: the values stored in the plan by bidmat_plan_set_values (already in plan order)
 hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* vals, float* C, int beta,
                        hipStream_t s) {
     hipError_t err;
     if (!vals && !plan->pvals && plan->nnz > 0) return hipErrorInvalidValue;
-    if ((err = bm::plan_reserve_partial(plan, k)) != hipSuccess) return err;
+    float* partial = row_partial(plan, k, s, &err);
+    if (!partial) return err;
     if ((err = bm::gather_segments(k, plan->nseg, plan->xcd_start, A, vals ? vals : plan->pvals, plan->pc,
-                                   vals ? plan->perm : nullptr, plan->segstart, plan->partial, s)) != hipSuccess) return err;
-    return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, C, beta, s);
+                                   vals ? plan->perm : nullptr, plan->segstart, partial, s)) != hipSuccess) return err;
+    return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, partial, C, beta, s);
 }
 
 hipError_t run_spsum_rows(bidmat_plan* plan, const float* vals, float* out, int beta, hipStream_t s) {
     hipError_t err;
     if (!vals && !plan->pvals && plan->nnz > 0) return hipErrorInvalidValue;
-    if ((err = bm::plan_reserve_partial(plan, 1)) != hipSuccess) return err;
+    float* partial = row_partial(plan, 1, s, &err);
+    if (!partial) return err;
     if ((err = bm::spsum_segments(plan->nseg, plan->xcd_start, vals ? vals : plan->pvals, vals ? plan->perm : nullptr,
-                                  plan->segstart, plan->partial, s)) != hipSuccess)
+                                  plan->segstart, partial, s)) != hipSuccess)
         return err;
-    return bm::reduce_segments(1, plan->nrows, plan->rowptr, plan->rowseg, plan->partial, out, beta, s);
+    return bm::reduce_segments(1, plan->nrows, plan->rowptr, plan->rowseg, partial, out, beta, s);
 }
 
 bool plan_on_current_device(const bidmat_plan* p) {
@@ -204,13 +212,13 @@ API int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float* A, int 
     if (err != hipSuccess) return finish_blocking(err);
     if (broff >= plan->nrows) return 0;                  // the tile holds no stored row
     const int nrows_eff = nc < plan->nrows - broff ? nc : plan->nrows - broff;
-    err = bm::plan_reserve_partial(plan.get(), nr);
-    if (err == hipSuccess)
+    float* partial = row_partial(plan.get(), nr, nullptr, &err);
+    if (partial)
         err = bm::gather_segments_ex(nr, lda, plan->nseg, plan->xcd_start, A, Bdata, plan->pc, plan->perm,
-                                     plan->segstart, plan->partial, bm::Window{1, bcoff, kk}, plan->segrow,
+                                     plan->segstart, partial, bm::Window{1, bcoff, kk}, plan->segrow,
                                      bm::Window{1, broff, nrows_eff}, nullptr);
-    if (err == hipSuccess)
-        err = bm::reduce_segments_ex(nr, ldc, broff, nrows_eff, plan->rowptr, plan->rowseg, plan->partial, C, 1, nullptr);
+    if (partial && err == hipSuccess)
+        err = bm::reduce_segments_ex(nr, ldc, broff, nrows_eff, plan->rowptr, plan->rowseg, partial, C, 1, nullptr);
     return finish_blocking(err);
 }
 
@@ -368,7 +376,7 @@ API int bidmat_plan_destroy(bidmat_plan* plan) {
 
 API long long bidmat_plan_bytes(const bidmat_plan* plan) {
     if (!plan) return 0;
-    return (long long)(plan->index_bytes + (plan->partial_floats + plan->ovf_partial_floats) * sizeof(float) +
+    return (long long)(plan->index_bytes +
                        ((plan->pvals ? 1 : 0) + (plan->cvals ? 1 : 0) + (plan->svals ? 1 : 0)) * (size_t)plan->nnz * sizeof(float));
 }
 
@@ -388,7 +396,7 @@ namespace {
 // the plan's column table as the kernels take it
 // (plans made by bidmat_plan_create always carry the column side)
 bm::ColTable col_table(bidmat_plan* plan) {
-    return bm::ColTable{plan->col_seglen, plan->ovf, (long long)plan->novf, plan->ovf_partial};
+    return bm::ColTable{plan->col_seglen, plan->ovf, (long long)plan->novf};
 }
 }  // namespace
 
@@ -406,10 +414,6 @@ API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float
     if (phased)
         return (int)bm::dsmult_phased(k, plan->ncols, A, Sdata ? Sdata : plan->cvals, plan->cir, Sdata ? plan->cperm : nullptr,
                                       plan->cptr, nphase, C, beta, as_stream(stream));
-    if (plan->novf > 0) {
-        hipError_t err = bm::plan_reserve_ovf_partial(plan, k);
-        if (err != hipSuccess) return (int)err;
-    }
     const bm::ColTable tab = col_table(plan);
     return (int)bm::dsmult_csc(k, plan->ncols, plan->nnz, A, Sdata, Sir, Sjc, C, beta, as_stream(stream), &tab);
 }

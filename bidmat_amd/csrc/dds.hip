@@ -505,7 +505,7 @@ hipError_t dds_csc_static(int k, int ncols, int nnz, const float* A, const float
     // every entry of the table that the kernels read is written by this build: nothing to clear
     err = build_overflow_table_in(ncols, nnz, jc, seglen, buf, &ovf, s);
     if (err != hipSuccess) return err;
-    const ColTable tab{seglen, ovf, ovf ? (long long)(nnz / seglen) : 0, nullptr};
+    const ColTable tab{seglen, ovf, ovf ? (long long)(nnz / seglen) : 0};
     return dds_csc(k, ncols, nnz, A, B, ir, jc, P, beta, s, nullptr, 0, &tab);
 }
 

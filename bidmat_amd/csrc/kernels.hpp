@@ -58,8 +58,8 @@ hipError_t build_overflow_table_in(int ncols, int nnz, const int* jc, int seglen
                                    hipStream_t s);
 // A column overflow table that the caller already holds (a plan builds it once per pattern):
 // seglen it was built with, table (ncols+1 ints; unused when novf == 0), number of overflow
-// segments, and for A*S a buffer of novf*k floats for their partial sums.
-struct ColTable { int seglen; const int* ovf; long long novf; float* partial; };
+// segments. (A*S keeps the novf*k partial sums of those segments in the stream's scratch.)
+struct ColTable { int seglen; const int* ovf; long long novf; };
 
 // A window [off, off+len) on the gather index of the nonzeros (tile variants); on == 0: no filter.
 struct Window { int on, off, len; };

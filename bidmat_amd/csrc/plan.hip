@@ -298,39 +298,11 @@ inline int bits_for(unsigned long long maxval) {
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
     hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->block_nnz, p->block_seg, p->partial, p->ovf, p->ovf_partial, p->pvals, p->cir, p->cperm, p->cptr, p->hotrows, p->cvals, p->svals};
+    void* bufs[] = {p->block_nnz, p->block_seg, p->ovf, p->pvals, p->cir, p->cperm, p->cptr, p->hotrows, p->cvals, p->svals};
     for (void* b : bufs)
         if (b && (f = hipFree(b)) != hipSuccess) e = f;
     delete p;
     return e;
-}
-
-hipError_t plan_reserve_partial(bidmat_plan* p, int k) {
-    size_t need = (size_t)p->nseg * (size_t)k;
-    if (need <= p->partial_floats) return hipSuccess;
-    if (p->partial) {
-        hipError_t e = hipFree(p->partial);
-        p->partial = nullptr; p->partial_floats = 0;
-        if (e != hipSuccess) return e;
-    }
-    hipError_t e = hipMalloc((void**)&p->partial, need * sizeof(float));
-    if (e != hipSuccess) { (void)hipGetLastError(); return e; }
-    p->partial_floats = need;
-    return hipSuccess;
-}
-
-hipError_t plan_reserve_ovf_partial(bidmat_plan* p, int k) {
-    size_t need = (size_t)p->novf * (size_t)k;
-    if (need <= p->ovf_partial_floats) return hipSuccess;
-    if (p->ovf_partial) {
-        hipError_t e = hipFree(p->ovf_partial);
-        p->ovf_partial = nullptr; p->ovf_partial_floats = 0;
-        if (e != hipSuccess) return e;
-    }
-    hipError_t e = hipMalloc((void**)&p->ovf_partial, need * sizeof(float));
-    if (e != hipSuccess) { (void)hipGetLastError(); return e; }
-    p->ovf_partial_floats = need;
-    return hipSuccess;
 }
 
 namespace {

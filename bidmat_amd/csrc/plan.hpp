@@ -31,16 +31,13 @@ struct bidmat_plan {
     int* rowseg = nullptr;   // [nseg]   segment ids grouped by row, ascending within a row
     void* block_nnz = nullptr;   // owns pc, perm, rowptr
     void* block_seg = nullptr;   // owns segstart, segrow, rowseg
-    float* partial = nullptr;
-    size_t partial_floats = 0;
+    // (the nseg*k partial sums of a call live in the scratch of the stream it runs on, not here)
     size_t index_bytes = 0;
     // Column side (A*S and DDS through the plan): the overflow-segment table of the columns is a
     // function of jc and seglen only, so it is built once here instead of on every call.
     int col_seglen = 0;          // seglen in force when the plan was built
     int novf = 0;                // overflow segments of all columns (0: no column is longer than col_seglen)
     int* ovf = nullptr;          // [ncols+1] exclusive scan of extra segments per column (only when novf > 0)
-    float* ovf_partial = nullptr;        // A*S: partial sums of the overflow segments (novf*k floats)
-    size_t ovf_partial_floats = 0;
     // Row-class ordering of every column (DDS through the plan). The eight XCDs have one L2 each;
     // when each of them gathers from the whole dense operand, all eight L2s end up holding the same
     // popular rows. Rows are dealt to eight classes (row & 7) and the nonzeros of every column are
@@ -70,10 +67,6 @@ namespace bm {
 hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,
                       bidmat_plan** out, bool column_side = true);
 hipError_t plan_free(bidmat_plan* p);
-// Makes sure the plan's partial buffer holds nseg*k floats.
-hipError_t plan_reserve_partial(bidmat_plan* p, int k);
-// Makes sure the buffer for the overflow partials of A*S holds novf*k floats.
-hipError_t plan_reserve_ovf_partial(bidmat_plan* p, int k);
 // pvals[p] = data[perm[p]] (allocates pvals on first use).
 hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s);
 }  // namespace bm

@@ -428,7 +428,12 @@ hipError_t dsmult_csc_ex(int k, int lda, int ldc, int ncols, int nnz, const floa
     if (tab) {
         // the caller knows the pattern's overflow segments: nothing to build, nothing to allocate
         seglen = tab->seglen;
-        if (tab->novf > 0) { ovf = const_cast<int*>(tab->ovf); novf_max = tab->novf; partial = tab->partial; }
+        if (tab->novf > 0) {
+            ovf = const_cast<int*>(tab->ovf);
+            novf_max = tab->novf;
+            partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err, s);
+            if (!partial) return err;
+        }
     } else {
         err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
         if (err != hipSuccess) return err;

@@ -12,6 +12,7 @@ enum WsSlot {
     WS_JC = 0,        // int[ncols+1]  column pointer derived from ic (reference-shaped entries)
     WS_OVF,           // int[ncols+1]  exclusive scan of extra segments per column
     WS_PARTIAL,       // float[novf*k] partial sums of overflow segments
+    WS_ROWPARTIAL,    // float[nseg*k] partial sums of a plan's row segments (A*^S, row sums)
     WS_SCAN,          // int[...]      block sums of the scan
     WS_MISC,          // small scalars (max row, fingerprints)
     WS_REDUCE,        // float[...]    partials of the dense reductions

@@ -17,17 +17,17 @@
  *   - entry points WITHOUT a stream argument block until the result is complete, like the
  *     reference's launchers (cudaStreamSynchronize, MatKernel.hpp:15).  Entry points WITH
  *     a `stream` argument (a hipStream_t passed as void*, NULL = default stream) only
- *     enqueue work.  The library's scratch buffers are kept per (device, stream): calls on
- *     different streams may overlap; calls that use the same plan handle share its
- *     partial-sum buffer and must be ordered with each other.
+ *     enqueue work.  The library's scratch buffers (including the partial sums of the calls that
+ *     go through a plan) are kept per (device, stream): calls on different streams may overlap,
+ *     also when they use the same plan handle, which holds data of the pattern only.
  *   - results are deterministic: no floating-point atomics anywhere.
  *   - threads: every entry point may be called from any host thread. Calls that take library
  *     scratch or a cached plan (all product, sum and reduction entries) hold a per-device lock
  *     while they look up / build their scratch and enqueue their kernels (the blocking entries:
  *     until their result is complete), so two threads that drive one device through the blocking
  *     entries or share a stream never see each other's scratch. What stays with the caller:
- *     one plan handle must not be used by two calls at the same time (its partial-sum buffer
- *     is one), and option changes (bidmat_set_option) are process-wide.
+ *     bidmat_plan_set_values and bidmat_plan_destroy must not run while another call uses the same
+ *     plan, and option changes (bidmat_set_option) are process-wide.
  */
 #ifndef BIDMAT_HIP_H
 #define BIDMAT_HIP_H
@@ -311,7 +311,7 @@ int bidmat_host_free(void *hptr);
  * calls issued on `stream` between begin and end, then replay them with one launch per step.
  * Only kernels are recorded (the library clears memory with fill kernels, never memset nodes).
  * Nothing may allocate while recording: run the same calls once on the same stream beforehand,
- * so that the stream's scratch buffers and any plan's partial-sum buffer have their size.  The
+ * so that the stream's scratch buffers (partial sums of plan calls included) have their size.  The
  * recorded pointers and sizes are fixed; the data they point to may change between replays.
  * A recording also holds the addresses of the stream's scratch buffers and of any plan it used:
  * destroy it (and record again) before a larger problem is run on that stream (scratch grows by

@@ -260,6 +260,51 @@ def test_two_threads_share_a_device_through_the_blocking_entries(hip):
     hip_abi.check(hip.bidmat_release_caches())
 
 
+def test_one_plan_serves_two_streams_at_once(hip):
+    """A plan holds pattern data only: the partial sums of a call live in the scratch of the stream it runs on.
+    A*^S and sparse row sums through ONE plan are enqueued on two streams without any ordering between them,
+    many times, with different dense operands and values; every result must equal the one computed alone."""
+    rng = np.random.default_rng(45)
+    k, nrows, ncols = 128, 3000, 40000
+    data, ir, jc = random_csc(rng, nrows, ncols, lengths=rng.integers(0, 60, size=ncols))
+    nnz = int(ir.size)
+    d = Dev(ir=ir, jc=jc)
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    streams, jobs = [], []
+    for t in range(2):
+        st = C.c_void_p()
+        hip_abi.check(hip.bidmat_stream_create(C.byref(st)))
+        streams.append(st)
+        A = rng.standard_normal(k * ncols).astype(np.float32)
+        v = rng.standard_normal(nnz).astype(np.float32)
+        jobs.append(dict(A=DeviceArray.from_numpy(A), v=DeviceArray.from_numpy(v), C=DeviceArray.zeros(k * nrows),
+                         rs=DeviceArray.zeros(nrows)))
+    want = []
+    for j, st in zip(jobs, streams):                       # each alone
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, j["A"].ptr, j["v"].ptr, j["C"].ptr, 0, st))
+        hip_abi.check(hip.bidmat_spsum_rows_plan(plan, j["v"].ptr, j["rs"].ptr, 0, st))
+        hip_abi.check(hip.bidmat_synchronize())
+        want.append((j["C"].numpy(), j["rs"].numpy()))
+    for _ in range(20):                                    # interleaved, unordered
+        for j, st in zip(jobs, streams):
+            hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, j["A"].ptr, j["v"].ptr, j["C"].ptr, 0, st))
+            hip_abi.check(hip.bidmat_spsum_rows_plan(plan, j["v"].ptr, j["rs"].ptr, 0, st))
+    hip_abi.check(hip.bidmat_synchronize())
+    for j, w in zip(jobs, want):
+        assert np.array_equal(j["C"].numpy(), w[0]) and np.array_equal(j["rs"].numpy(), w[1])
+    # the plan's own footprint no longer depends on k: no partial-sum buffer inside
+    before = hip.bidmat_plan_bytes(plan)
+    big = DeviceArray.zeros(512 * nrows)
+    A512 = DeviceArray.from_numpy(rng.standard_normal(512 * ncols).astype(np.float32))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, 512, A512.ptr, jobs[0]["v"].ptr, big.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert hip.bidmat_plan_bytes(plan) == before
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    for st in streams:
+        hip_abi.check(hip.bidmat_stream_destroy(st))
+    d.free()
+
+
 # ---------------------------------------------------------------- plan-taking and fused forms
 @pytest.mark.parametrize("k", [32, 100, 256])
 def test_plan_forms_equal_the_plain_entries_bit_for_bit(hip, k):
