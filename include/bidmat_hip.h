@@ -165,7 +165,8 @@ typedef struct bidmat_plan bidmat_plan;
 int bidmat_plan_create(int nrows, int ncols, int nnz, const int *Sir, const int *Sjc, int k_hint,
                        bidmat_plan **plan);
 int bidmat_plan_destroy(bidmat_plan *plan);
-/* Device bytes held by the plan (index arrays + partial-sum workspace). */
+/* Device bytes held by the plan: index arrays and, after bidmat_plan_set_values, the stored values.
+ * (The nseg*k partial sums of a call through the plan are scratch of the stream it runs on.) */
 long long bidmat_plan_bytes(const bidmat_plan *plan);
 /* Number of row segments of the plan (each yields one k-vector partial sum). */
 int bidmat_plan_segments(const bidmat_plan *plan);
