@@ -100,8 +100,8 @@ def flops(op, k, nnz, ncols):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="headline", choices=["headline", "C1", "C4", "C5", "next", "footprint"])
     ap.add_argument("--footprint-k", type=int, default=256, help="k of the footprint sweep")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows/columns of the pattern (testing)")
