@@ -42,7 +42,7 @@ HBM_PEAK_GBS = 8000.0
 # was taken on; it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dds", 100003320): (25.46e9, "bidmat_amd/csrc/dds.hip", "2b6c7d772c9cbfcf",
+    ("headline", "dds", 100003320): (25.45e9, "bidmat_amd/csrc/dds.hip", "f7e2c97e0cc1236f",
                                      "profiles/headline_kernel_trace_and_hbm_counters.txt"),
     ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "4df7d618119c5dec",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
@@ -194,7 +194,7 @@ def main():
         ]
         workload = "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), step = DDS, A*S, A*^S"
         metric = "algorithmic GB/s (gathered operand charged once per nonzero) and nnz/s for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
-        roof_op, roof_kernel = "dds", "k_dds_classed<W=4,V=1,LPN=64> (one launch = DDS over the whole pattern, class-ordered columns)"
+        roof_op, roof_kernel = "dds", "k_dds_classed_nolds_k256 = the class-ordered DDS kernel at W=4,V=1,LPN=64 without LDS rows (one launch = DDS over the whole pattern)"
     elif args.workload in ("C1", "C4"):
         d_A = up(cfg["A"])
         d_C = DeviceArray(k * ncols, np.float32)

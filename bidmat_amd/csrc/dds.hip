@@ -248,12 +248,12 @@ struct ColumnAhead {
     Vec<W> b[V];
 };
 
-template <int W, int V, int LPN>
+template <int W, int V, int LPN, bool HOTLDS>
 __device__ __forceinline__ void load_column_ahead(const DdsClassedArgs& a, long long c, int js, int jm, int je, int q,
                                                   int l, ColumnAhead<W, V>& n) {
     n.js = js; n.jm = jm; n.je = je;
     n.hrow = n.hpos = n.trow = n.tpos = 0;
-    if (q < jm - js) { n.hrow = a.cir[js + q]; n.hpos = a.cperm[js + q]; }
+    if (HOTLDS && q < jm - js) { n.hrow = a.cir[js + q]; n.hpos = a.cperm[js + q]; }
     if (q < je - jm) { n.trow = a.cir[jm + q]; n.tpos = a.cperm[jm + q]; }
     const float* bp = a.B + (size_t)c * (size_t)a.k;
 #pragma unroll
@@ -263,15 +263,17 @@ __device__ __forceinline__ void load_column_ahead(const DdsClassedArgs& a, long 
     }
 }
 
-template <int W, int V, int LPN, bool EXACT>
-__global__ __launch_bounds__(CL_MAX_THREADS) void k_dds_classed(DdsClassedArgs a) {
+// HOTLDS == false: no hot rows (hcap == 0): no LDS, no hot-row runs, workgroups of BM_BLOCK threads, and the
+// registers this saves buy occupancy (the kernel waits on L2 misses: the more waves, the more gathers in flight).
+template <int W, int V, int LPN, bool EXACT, bool HOTLDS>
+__device__ __forceinline__ void dds_classed_body(const DdsClassedArgs& a) {
     constexpr int KT = W * V * LPN;
     const int lane = threadIdx.x & 63;
     const int wave = wave_uniform(threadIdx.x >> 6);
     const int nwaves = blockDim.x >> 6;
     const int x = blockIdx.x & 7;
     // ---- this class's hot rows into LDS, row h at hot_lds[h*k ..]
-    if (a.hcap > 0) {
+    if (HOTLDS && a.hcap > 0) {
         const int vpr = (a.k + W - 1) / W;                // vectors per row (W == 4 implies k % 4 == 0)
         const int total = a.hcap * vpr;
         for (int i = threadIdx.x; i < total; i += blockDim.x) {
@@ -298,13 +300,13 @@ __global__ __launch_bounds__(CL_MAX_THREADS) void k_dds_classed(DdsClassedArgs a
             pe = a.cptr[sc + 2];
         }
         ColumnAhead<W, V> nx;
-        load_column_ahead<W, V, LPN>(a, c0, __builtin_amdgcn_readlane(ps, 0), __builtin_amdgcn_readlane(pm, 0),
+        load_column_ahead<W, V, LPN, HOTLDS>(a, c0, __builtin_amdgcn_readlane(ps, 0), __builtin_amdgcn_readlane(pm, 0),
                                      __builtin_amdgcn_readlane(pe, 0), q, l, nx);
         for (int ci = 0; ci < nc; ++ci) {
             const ColumnAhead<W, V> cur = nx;
             // the next column's index chunks and its column of B are requested before this column's gathers
             if (ci + 1 < nc)
-                load_column_ahead<W, V, LPN>(a, c0 + ci + 1, __builtin_amdgcn_readlane(ps, ci + 1),
+                load_column_ahead<W, V, LPN, HOTLDS>(a, c0 + ci + 1, __builtin_amdgcn_readlane(ps, ci + 1),
                                              __builtin_amdgcn_readlane(pm, ci + 1), __builtin_amdgcn_readlane(pe, ci + 1), q, l, nx);
             if (cur.js >= cur.je) continue;
             const float* bp = a.B + (size_t)(c0 + ci) * (size_t)a.k;
@@ -322,11 +324,29 @@ __global__ __launch_bounds__(CL_MAX_THREADS) void k_dds_classed(DdsClassedArgs a
                 }
                 const bool accumulate = (a.beta != 0) || (k0 > 0);
                 const bool last = k0 + KT >= a.k;
-                dds_classed_run<W, V, LPN, EXACT, true>(a, cur.js, cur.jm, cur.hrow, cur.hpos, q, g, l, eld, ev, b, accumulate, last);
+                if constexpr (HOTLDS)
+                    dds_classed_run<W, V, LPN, EXACT, true>(a, cur.js, cur.jm, cur.hrow, cur.hpos, q, g, l, eld, ev, b, accumulate, last);
                 dds_classed_run<W, V, LPN, EXACT, false>(a, cur.jm, cur.je, cur.trow, cur.tpos, q, g, l, eld, ev, b, accumulate, last);
             }
         }
     }
+}
+
+template <int W, int V, int LPN, bool EXACT>
+__global__ __launch_bounds__(CL_MAX_THREADS) void k_dds_classed(DdsClassedArgs a) {
+    dds_classed_body<W, V, LPN, EXACT, true>(a);
+}
+template <int W, int V, int LPN, bool EXACT>
+__global__ __launch_bounds__(BM_BLOCK) void k_dds_classed_nolds(DdsClassedArgs a) {
+    dds_classed_body<W, V, LPN, EXACT, false>(a);
+}
+// The shape of k in (128, 256] fits six waves per SIMD (80 registers) without spilling, one more than the
+// compiler settles on by itself (4.78 against 4.84 ms at the headline); asked for seven or eight it spills inside
+// the gather loop and loses a fifth (5.85 ms), and the other shapes spill already at six.
+template <bool EXACT>
+__global__ __launch_bounds__(BM_BLOCK) __attribute__((amdgpu_waves_per_eu(6, 6)))
+void k_dds_classed_nolds_k256(DdsClassedArgs a) {
+    dds_classed_body<4, 1, 64, EXACT, false>(a);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -382,6 +402,13 @@ hipError_t launch_dds_classed(const Shape& sh, bool exact, const DdsClassedArgs&
     dim3 grid((unsigned)nblk), block((unsigned)threads);
 #define BM_CASE(W_, V_, L_, E_)                                                          \
     if (sh.W == W_ && sh.V == V_ && sh.LPN == L_ && exact == E_) {                       \
+        if (lds_bytes == 0) {                                                            \
+            if (W_ == 4 && V_ == 1 && L_ == 64)                                          \
+                hipLaunchKernelGGL((k_dds_classed_nolds_k256<E_>), grid, block, 0, s, a); \
+            else                                                                         \
+                hipLaunchKernelGGL((k_dds_classed_nolds<W_, V_, L_, E_>), grid, block, 0, s, a); \
+            return hipGetLastError();                                                    \
+        }                                                                                \
         auto kern = k_dds_classed<W_, V_, L_, E_>;                                       \
         if (lds_bytes > (48u << 10)) {                                                   \
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); \
