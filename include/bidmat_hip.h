@@ -180,8 +180,8 @@ int bidmat_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *S
 /* The values of the pattern in plan order, stored in the plan (nnz floats): afterwards
  * bidmat_dsmultT_plan, bidmat_sdmult_plan and bidmat_spsum_rows_plan accept Sdata == NULL and stream
  * the stored values instead of fetching every value through the plan's permutation; so does
- * bidmat_dsmult_plan when the plan carries a row-class ordering of its columns (otherwise it needs
- * Sdata).  For callers whose values stay the same over several calls (a data minibatch); call it
+ * bidmat_dsmult_plan when the plan carries a row-class ordering of its columns and no column is longer
+ * than 8192 nonzeros (otherwise it needs Sdata: hipErrorInvalidValue without).  For callers whose values stay the same over several calls (a data minibatch); call it
  * again when they change. */
 int bidmat_plan_set_values(bidmat_plan *plan, const float *Sdata, void *stream);
 
