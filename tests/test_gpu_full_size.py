@@ -215,3 +215,45 @@ def test_large_pattern_with_one_bad_row_index_is_refused(hip):
     ref = np.bincount(ir, weights=vals.astype(np.float64), minlength=nrows)
     assert np.allclose(dout.numpy(), ref, rtol=RTOL, atol=0)
     hip_abi.check(hip.bidmat_plan_destroy(plan))
+
+
+@pytest.mark.timeout(300)
+def test_very_long_columns_keep_their_accuracy_through_the_plan(hip):
+    """Pareto column lengths up to 60 000 nonzeros on Zipf rows, all terms positive: A*S through the plan must stay as
+    close to the fp64 result as the plain entry (columns this long are never added up in one running sum), DDS through
+    the plan must equal the plain entry bit for bit, and A*^S must meet the same bound."""
+    k, nrows, ncols = 512, 300000, 60000
+    ir, jc = gen.pattern(nrows, ncols, ("pareto", 20.0, 1.1, 1, 60000), ("zipf", 1.2), 107)
+    nnz = int(ir.size)
+    assert int(np.diff(jc).max()) > 30000
+    A, B, vals = gen.uniform(k * nrows, 8), gen.uniform(k * ncols, 9), gen.uniform_open0(nnz, 10)
+    dA, dB, dv = DeviceArray.from_numpy(A), DeviceArray.from_numpy(B), DeviceArray.from_numpy(vals)
+    dir_, djc = DeviceArray.from_numpy(ir), DeviceArray.from_numpy(jc)
+    old = hip.bidmat_get_option(b"col_classes")
+    hip_abi.check(hip.bidmat_set_option(b"col_classes", 1))          # force the class ordering onto the plan
+    try:
+        plan = make_plan(hip, nrows, ncols, nnz, dir_, djc, k)
+    finally:
+        hip_abi.check(hip.bidmat_set_option(b"col_classes", old))
+    C1, C2 = DeviceArray(k * ncols, np.float32), DeviceArray(k * ncols, np.float32)
+    hip_abi.check(hip.bidmat_dsmult_csc(k, ncols, nnz, dA.ptr, dv.ptr, dir_.ptr, djc.ptr, C1.ptr, 0, None))
+    hip_abi.check(hip.bidmat_dsmult_plan(plan, k, dA.ptr, dv.ptr, dir_.ptr, djc.ptr, C2.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    ref64, _ = oracle.fsmult_f64(A, k, vals, ir, jc, nthreads=oracle.max_threads())
+    nz = ref64 > 0
+    e_plain = float(np.max(np.abs(C1.numpy()[nz] - ref64[nz]) / ref64[nz]))
+    e_plan = float(np.max(np.abs(C2.numpy()[nz] - ref64[nz]) / ref64[nz]))
+    assert e_plain <= 5e-6 and e_plan <= 5e-6, (e_plain, e_plan)
+    C1.free(); C2.free()
+    P1, P2 = DeviceArray(nnz, np.float32), DeviceArray(nnz, np.float32)
+    hip_abi.check(hip.bidmat_dds_csc(k, ncols, nnz, dA.ptr, dB.ptr, dir_.ptr, djc.ptr, P1.ptr, 0, None))
+    hip_abi.check(hip.bidmat_dds_plan(plan, k, dA.ptr, dB.ptr, dir_.ptr, djc.ptr, None, 0, P2.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert np.array_equal(P1.numpy(), P2.numpy())
+    G = DeviceArray(k * nrows, np.float32)
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, dB.ptr, dv.ptr, G.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    ref64, _ = oracle.fsmultT_f64(B, k, nrows, vals, ir, jc, nthreads=oracle.max_threads())
+    nz = ref64 > 0
+    assert float(np.max(np.abs(G.numpy()[nz] - ref64[nz]) / ref64[nz])) <= 5e-6
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
