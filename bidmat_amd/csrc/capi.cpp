@@ -6,6 +6,7 @@
 #include "kernels.hpp"
 #include "plan.hpp"
 #include "workspace.hpp"
+#include <algorithm>
 #include <atomic>
 #include <cstring>
 #include <cstdio>
@@ -27,7 +28,11 @@ std::atomic<int> g_class_hot{-1};
 std::atomic<int> g_class_threads{1024};
 std::atomic<int> g_class_phases{2};
 std::atomic<int> g_plan_keep_mb{4096};
+std::atomic<int> g_cache_cols_after{2};
+std::atomic<int> g_cache_plans{4};
+std::atomic<int> g_check_plan{0};
 }  // namespace
+int opt_check_plan() { return g_check_plan.load(std::memory_order_relaxed); }
 int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
 int opt_plan_keep_mb() { return g_plan_keep_mb.load(std::memory_order_relaxed); }
 int opt_class_phases() { return g_class_phases.load(std::memory_order_relaxed); }
@@ -55,19 +60,21 @@ inline int finish_blocking(hipError_t launch_err) {
 
 // ---- plan cache for entries that only receive (ir, ic): keyed by a fingerprint of both index
 // arrays, so a caller that refills the same device buffers with another pattern never meets a
-// stale plan.
+// stale plan. An entry starts without a plan; A*^S / row sums build the row side at once (they cannot
+// run without it), A*S / DDS build the column side from their "cache_cols_after"-th call on the
+// pattern (default: the second), so a pattern that is used once costs no build.
 struct CacheEntry {
     int device;
     int ncols, nnz, nrows, k_hint;
-    const int *ir, *ic;                     // where the pattern lay when the plan was built
+    const int *ir, *ic;                     // where the pattern lay when the entry was made
     unsigned long long fa, fb;
-    std::shared_ptr<bidmat_plan> plan;      // callers hold a reference while they use the plan
+    int col_uses;                           // A*S / DDS calls that met this pattern
+    std::shared_ptr<bidmat_plan> plan;      // callers hold a reference while they use the plan (may be empty)
 };
 using PlanRef = std::shared_ptr<bidmat_plan>;
 PlanRef own(bidmat_plan* p) { return PlanRef(p, [](bidmat_plan* q) { (void)bm::plan_free(q); }); }
 std::mutex g_cache_mu;
 std::list<CacheEntry> g_cache;          // most recently used first
-constexpr size_t kMaxCachedPlans = 4;
 // the class-ordered DDS kernel walks a column's class in one wave: very long columns stay with the
 // segment-splitting kernel
 constexpr int kMaxClassedColumn = 1 << 16;
@@ -76,7 +83,14 @@ constexpr int kMaxClassedColumn = 1 << 16;
 // kernel that cuts columns into segments); longer ones stay with the segment-splitting kernel
 constexpr int kMaxPhasedColumn = 1 << 13;
 
-hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_hint, PlanRef* out) {
+enum Need { NEED_ROWS, NEED_COLS };
+
+// Finds (or makes) the cache entry of the pattern (ir, ic) and returns its plan with the side `need`
+// built when that side is due; *out stays empty when A*S / DDS should run without a plan. *jc_out
+// (nullable) receives the pattern's column pointer, built in the same pass over ic into the default
+// stream's scratch: valid until the caller's next scratch request for WS_JC.
+hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_hint, Need need, PlanRef* out,
+                       int** jc_out = nullptr) {
     out->reset();
     hipError_t err;
     int dev = 0;
@@ -84,8 +98,11 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     hipStream_t s = nullptr;
     unsigned long long* d_misc = (unsigned long long*)bm::ws_get(bm::WS_MISC, 64, &err);
     if (!d_misc) return err;
+    int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
+    if (!jc) return err;
+    if (jc_out) *jc_out = jc;
     // misc layout: [0..1] digests of ir and ic, [2] (as int) max row
-    if ((err = bm::pattern_digest(ir, ic, nnz, d_misc, s)) != hipSuccess) return err;
+    if ((err = bm::pattern_digest(ir, ic, nnz, d_misc, s, ncols, jc)) != hipSuccess) return err;
     unsigned long long h[3];
     if ((err = hipMemcpy(h, d_misc, sizeof(h), hipMemcpyDeviceToHost)) != hipSuccess) return err;
     int maxrow;
@@ -93,25 +110,43 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     const int nrows = maxrow + 1;
 
     std::lock_guard<std::mutex> lock(g_cache_mu);
+    auto hit = g_cache.end();
     for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
         // panels are sized for k_hint: a request that names k only takes a plan built for that k
         const bool k_ok = k_hint <= 0 || (it->k_hint > 0 ? it->k_hint : 256) == k_hint;
         if (k_ok && it->device == dev && it->ncols == ncols && it->nnz == nnz && it->nrows == nrows &&
             it->ir == ir && it->ic == ic && it->fa == h[0] && it->fb == h[1]) {
-            g_cache.splice(g_cache.begin(), g_cache, it);
-            *out = g_cache.front().plan;
+            hit = it;
+            break;
+        }
+    }
+    if (hit == g_cache.end()) {
+        const size_t cap = (size_t)std::max(1, bm::g_cache_plans.load());
+        while (g_cache.size() >= cap) g_cache.pop_back();           // its plan is freed when its last user lets go
+        g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, ir, ic, h[0], h[1], 0, PlanRef()});
+    } else {
+        g_cache.splice(g_cache.begin(), g_cache, hit);
+    }
+    CacheEntry& e = g_cache.front();
+    int side = bm::PLAN_ROWS;
+    if (need == NEED_COLS) {
+        side = bm::PLAN_COLS;
+        const int after = bm::g_cache_cols_after.load();
+        if (e.col_uses < 0x7fffffff) ++e.col_uses;
+        if (after <= 0 || e.col_uses < after) {
+            // not due yet: use the column side only if an earlier call has built it
+            if (e.plan && (e.plan->sides & bm::PLAN_COLS)) *out = e.plan;
             return hipSuccess;
         }
     }
-    int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
-    if (!jc) return err;
-    if ((err = bm::coo_compress_cols(ncols, nnz, ic, jc, s)) != hipSuccess) return err;
-    bidmat_plan* p = nullptr;
-    // the reference-shaped entries only ever use the row side of a cached plan
-    if ((err = bm::plan_build(nrows, ncols, nnz, ir, jc, k_hint, &p, false)) != hipSuccess) return err;
-    while (g_cache.size() >= kMaxCachedPlans) g_cache.pop_back();   // freed when its last user lets go
-    g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, ir, ic, h[0], h[1], own(p)});
-    *out = g_cache.front().plan;
+    if (!e.plan) {
+        bidmat_plan* p = nullptr;
+        if ((err = bm::plan_build(nrows, ncols, nnz, ir, jc, k_hint, &p, side)) != hipSuccess) return err;
+        e.plan = own(p);
+    } else if (!(e.plan->sides & side)) {
+        if ((err = bm::plan_extend(e.plan.get(), ir, jc, side)) != hipSuccess) return err;
+    }
+    *out = e.plan;
     return hipSuccess;
 }
 
@@ -149,6 +184,84 @@ bool plan_on_current_device(const bidmat_plan* p) {
     return p && hipGetDevice(&dev) == hipSuccess && dev == p->device;
 }
 
+// the plan's column table as the kernels take it
+bm::ColTable col_table(const bidmat_plan* plan) {
+    return bm::ColTable{plan->col_seglen, plan->ovf, (long long)plan->novf};
+}
+
+inline bool ranges_overlap(const float* a, const float* b, long long n) {
+    const uintptr_t x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
+    const uintptr_t len = (uintptr_t)n * sizeof(float);
+    return x < y + len && y < x + len;
+}
+
+// The fused step reads V[j] and writes P[j] from the same lane, so P == V (the in-place update) is sound
+// as long as k is covered in one pass; wider k keeps running sums in P between passes, and a V that
+// overlaps P at another offset is read by other lanes than the ones that write it.
+bool fused_operand_ok(int k, long long nnz, const float* A, const float* B, const float* V, const float* P) {
+    if (!V || !ranges_overlap(V, P, nnz)) return true;
+    if (V != P) return false;
+    const bool al = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
+    const bm::Shape sh = bm::pick_shape(k, al);
+    return k <= sh.W * (sh.V > 4 ? 4 : sh.V) * sh.LPN;
+}
+
+// Checked mode (option "check_plan"): the pattern handed to a plan-taking call must be the one the plan
+// was built from. Compares a digest of (Sir, Sjc) with the one taken at build time; plans built while
+// the option was off carry no digest and pass.
+int plan_pattern_ok(const bidmat_plan* plan, const int* Sir, const int* Sjc) {
+    if (!bm::opt_check_plan() || !plan->has_digest) return 0;
+    unsigned long long d[2];
+    hipError_t e = bm::plan_digest(plan->nnz, plan->ncols, Sir, Sjc, d);
+    if (e != hipSuccess) return (int)e;
+    return (d[0] == plan->digest[0] && d[1] == plan->digest[1]) ? 0 : kInvalid;
+}
+
+// C = beta*C + A*S through the column side of a plan.
+int dsmult_through_plan(bidmat_plan* plan, int k, const float* A, const float* Sdata, const int* Sir, const int* Sjc,
+                        float* C, int beta, hipStream_t s) {
+    if (!(plan->sides & bm::PLAN_COLS)) return kInvalid;
+    const int nphase = bm::opt_class_phases();
+    const bool phased = plan->ncls == 8 && plan->hcap == 0 && nphase > 0 && plan->maxlen <= kMaxPhasedColumn && plan->nnz > 0;
+    if (!Sdata && !phased) return kInvalid;
+    // Sdata == NULL: the values stored by bidmat_plan_set_values, which exist in class order only
+    if (!Sjc || !C || (plan->nnz > 0 && (!A || !Sir || (!Sdata && !(phased && plan->cvals))))) return kInvalid;
+    if (int bad = plan_pattern_ok(plan, Sir, Sjc)) return bad;
+    if (phased)
+        return (int)bm::dsmult_phased(k, plan->ncols, A, Sdata ? Sdata : plan->cvals, plan->cir, Sdata ? plan->cperm : nullptr,
+                                      plan->cptr, nphase, C, beta, s);
+    const bm::ColTable tab = col_table(plan);
+    return (int)bm::dsmult_csc(k, plan->ncols, plan->nnz, A, Sdata, Sir, Sjc, C, beta, s, &tab);
+}
+
+// DDS through the column side of a plan. stored: the epilogue operand is the plan's stored values (V ignored).
+int dds_through_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc, const float* V,
+                     bool stored, int opn, float* P, int beta, hipStream_t s) {
+    if (!(plan->sides & bm::PLAN_COLS)) return kInvalid;
+    if ((V || stored) && (beta != 0 || opn < 0 || opn > 14)) return kInvalid;
+    if (plan->ncols == 0 || plan->nnz == 0) return 0;
+    if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
+    if (!stored && !fused_operand_ok(k, plan->nnz, A, B, V, P)) return kInvalid;
+    if (int bad = plan_pattern_ok(plan, Sir, Sjc)) return bad;
+    const bool classed = plan->ncls == 8 && k > 0 && plan->maxlen <= kMaxClassedColumn &&
+                         (size_t)plan->hcap * (size_t)k * sizeof(float) <= bm::dds_classed_lds_budget();
+    if (stored) {
+        V = plan->ncls == 8 ? (classed ? plan->cvals : nullptr) : plan->svals;
+        if (!V) return kInvalid;              // bidmat_plan_set_values has not been called (or k does not fit the ordering)
+    }
+    if (classed) {
+        const hipError_t e = bm::dds_classed(k, plan->ncols, A, B, plan->cir, plan->cperm, plan->cptr, plan->hcap, plan->hotrows,
+                                             P, beta, s, V, opn, stored);
+        // A launch that the device refuses (e.g. less LDS per workgroup than the ordering was built for)
+        // leaves nothing enqueued: the plain kernel gives the same bits. Stored values exist in class
+        // order only, so that form reports the error.
+        if (e == hipSuccess || stored) return (int)e;
+        (void)hipGetLastError();
+    }
+    const bm::ColTable tab = col_table(plan);
+    return (int)bm::dds_csc(k, plan->ncols, plan->nnz, A, B, Sir, Sjc, P, beta, s, V, opn, &tab);
+}
+
 }  // namespace
 
 // ======================================================================== reference-shaped
@@ -160,6 +273,15 @@ API int bidmat_dsmult(int nrows, int ncols, int nnz, const float* A, const float
     if (nrows == 0 || ncols == 0 || nnz == 0) return 0;           // C += 0
     if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
     hipError_t err;
+    if (bm::g_cache_cols_after.load() > 0) {
+        // a pattern met before runs through the column side of its cached plan
+        PlanRef plan;
+        int* jc = nullptr;
+        err = cached_plan(ncols, nnz, Bir, Bic, nrows, NEED_COLS, &plan, &jc);
+        if (err != hipSuccess) return finish_blocking(err);
+        if (plan) return finish_blocking((hipError_t)dsmult_through_plan(plan.get(), nrows, A, Bdata, Bir, jc, C, 1, nullptr));
+        return finish_blocking(bm::dsmult_csc(nrows, ncols, nnz, A, Bdata, Bir, jc, C, 1, nullptr));
+    }
     int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
     if (!jc) return (int)err;
     err = bm::coo_compress_cols(ncols, nnz, Bic, jc, nullptr);
@@ -174,7 +296,7 @@ API int bidmat_dsmultT(int nrows, int ncols, int nnz, const float* A, const floa
     if (nrows == 0 || ncols == 0 || nnz == 0) return 0;
     if (!A || !Bdata || !Bir || !Bic || !C) return kInvalid;
     PlanRef plan;
-    hipError_t err = cached_plan(ncols, nnz, Bir, Bic, nrows, &plan);
+    hipError_t err = cached_plan(ncols, nnz, Bir, Bic, nrows, NEED_ROWS, &plan);
     if (err == hipSuccess) err = run_dsmultT(plan.get(), nrows, A, Bdata, C, 1, nullptr);
     return finish_blocking(err);
 }
@@ -212,7 +334,7 @@ API int bidmat_dsmultTileT(int nr, int nc, int kk, int nnz, const float* A, int 
     if (err != hipSuccess) return (int)err;
     if (last < 0 || last == 0x7fffffff) return kInvalid;
     PlanRef plan;
-    err = cached_plan(last + 1, nnz, Bir, Bic, nr, &plan);
+    err = cached_plan(last + 1, nnz, Bir, Bic, nr, NEED_ROWS, &plan);
     if (err != hipSuccess) return finish_blocking(err);
     if (broff >= plan->nrows) return 0;                  // the tile holds no stored row
     const int nrows_eff = nc < plan->nrows - broff ? nc : plan->nrows - broff;
@@ -254,6 +376,15 @@ API int bidmat_dds(int nrows, int nnz, const float* A, const float* B, const int
     if (err != hipSuccess) return (int)err;
     if (last < 0 || last == 0x7fffffff) return kInvalid;
     const int ncols = last + 1;
+    if (bm::g_cache_cols_after.load() > 0 && nrows > 0) {
+        // a pattern met before runs through the column side of its cached plan
+        PlanRef plan;
+        int* jc = nullptr;
+        err = cached_plan(ncols, nnz, Cir, Cic, nrows, NEED_COLS, &plan, &jc);
+        if (err != hipSuccess) return finish_blocking(err);
+        if (plan) return finish_blocking((hipError_t)dds_through_plan(plan.get(), nrows, A, B, Cir, jc, nullptr, false, 0, P, 1, nullptr));
+        return finish_blocking(bm::dds_csc(nrows, ncols, nnz, A, B, Cir, jc, P, 1, nullptr));
+    }
     int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
     if (!jc) return (int)err;
     err = bm::coo_compress_cols(ncols, nnz, Cic, jc, nullptr);
@@ -275,7 +406,7 @@ API int bidmat_spsum(int nrows, int ncols, int nnz, const int* Air, const int* A
         if (err == hipSuccess) err = bm::spsum_cols(ncols, nnz, P, jc, B, 1, nullptr);
     } else {
         PlanRef plan;
-        err = cached_plan(ncols, nnz, Air, Aic, 0, &plan);
+        err = cached_plan(ncols, nnz, Air, Aic, 0, NEED_ROWS, &plan);
         if (err == hipSuccess && plan->nrows > nrows) err = hipErrorInvalidValue;   // row index outside B
         if (err == hipSuccess) err = run_spsum_rows(plan.get(), P, B, 1, nullptr);
     }
@@ -329,6 +460,9 @@ API int bidmat_dds_csc(int k, int ncols, int nnz, const float* A, const float* B
 
 API int bidmat_dds_csc_static(int k, int ncols, int nnz, const float* A, const float* B, const int* Sir,
                               const int* Sjc, float* P, int beta, void* stream) {
+    // a mutex allocates nothing: host threads that share a stream cannot interleave "table built" and
+    // "kernel enqueued" on the one scratch array (calls on different streams of a device still race on it)
+    auto lock = bm::device_lock();
     if (k < 0 || ncols < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
     if (ncols > bm::dds_static_max_cols()) return kInvalid;      // beyond the fixed scratch array
     if (ncols == 0 || nnz == 0) return 0;
@@ -344,6 +478,7 @@ API int bidmat_dds_csc_op(int k, int ncols, int nnz, const float* A, const float
     if (k < 0 || ncols < 0 || nnz < 0 || opn < 0 || opn > 14) return kInvalid;
     if (ncols == 0 || nnz == 0) return 0;
     if (!Sjc || !Sir || !P || !V || (k > 0 && (!A || !B))) return kInvalid;
+    if (!fused_operand_ok(k, nnz, A, B, V, P)) return kInvalid;
     return (int)bm::dds_csc(k, ncols, nnz, A, B, Sir, Sjc, P, 0, as_stream(stream), V, opn);
 }
 
@@ -375,12 +510,13 @@ API int bidmat_plan_create(int nrows, int ncols, int nnz, const int* Sir, const 
 
 API int bidmat_plan_destroy(bidmat_plan* plan) {
     if (!plan) return 0;
+    auto lock = bm::device_lock();          // no call of another thread is between its scratch lookup and its launch
     return (int)bm::plan_free(plan);
 }
 
 API long long bidmat_plan_bytes(const bidmat_plan* plan) {
     if (!plan) return 0;
-    return (long long)(plan->index_bytes +
+    return (long long)(plan->row_bytes + plan->col_bytes +
                        ((plan->pvals ? 1 : 0) + (plan->cvals ? 1 : 0) + (plan->svals ? 1 : 0)) * (size_t)plan->nnz * sizeof(float));
 }
 
@@ -391,18 +527,11 @@ API int bidmat_dsmultT_plan(bidmat_plan* plan, int k, const float* A, const floa
     auto lock = bm::device_lock();
     if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (!(plan->sides & bm::PLAN_ROWS)) return kInvalid;
     if (k == 0 || plan->nrows == 0) return 0;
     if (!C || (plan->nnz > 0 && (!A || (!Sdata && !plan->pvals)))) return kInvalid;
     return (int)run_dsmultT(plan, k, A, Sdata, C, beta, as_stream(stream));
 }
-
-namespace {
-// the plan's column table as the kernels take it
-// (plans made by bidmat_plan_create always carry the column side)
-bm::ColTable col_table(bidmat_plan* plan) {
-    return bm::ColTable{plan->col_seglen, plan->ovf, (long long)plan->novf};
-}
-}  // namespace
 
 API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float* Sdata, const int* Sir,
                            const int* Sjc, float* C, int beta, void* stream) {
@@ -410,54 +539,32 @@ API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float
     if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (k == 0 || plan->ncols == 0) return 0;
-    const int nphase = bm::opt_class_phases();
-    const bool phased = plan->ncls == 8 && plan->hcap == 0 && nphase > 0 && plan->maxlen <= kMaxPhasedColumn && plan->nnz > 0;
-    if (!Sdata && !phased) return kInvalid;
-    // Sdata == NULL: the values stored by bidmat_plan_set_values, which exist in class order only
-    if (!Sjc || !C || (plan->nnz > 0 && (!A || !Sir || (!Sdata && !(phased && plan->cvals))))) return kInvalid;
-    if (phased)
-        return (int)bm::dsmult_phased(k, plan->ncols, A, Sdata ? Sdata : plan->cvals, plan->cir, Sdata ? plan->cperm : nullptr,
-                                      plan->cptr, nphase, C, beta, as_stream(stream));
-    const bm::ColTable tab = col_table(plan);
-    return (int)bm::dsmult_csc(k, plan->ncols, plan->nnz, A, Sdata, Sir, Sjc, C, beta, as_stream(stream), &tab);
+    return dsmult_through_plan(plan, k, A, Sdata, Sir, Sjc, C, beta, as_stream(stream));
 }
 
 namespace {
-// DDS through a plan. stored: the epilogue operand is the plan's stored values (V ignored).
-int dds_through_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc, const float* V,
-                     bool stored, int opn, float* P, int beta, void* stream) {
+int dds_plan_entry(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc, const float* V,
+                   bool stored, int opn, float* P, int beta, void* stream) {
     auto lock = bm::device_lock();
     if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
-    if ((V || stored) && (beta != 0 || opn < 0 || opn > 14)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
-    if (plan->ncols == 0 || plan->nnz == 0) return 0;
-    if (!Sjc || !Sir || !P || (k > 0 && (!A || !B))) return kInvalid;
-    const bool classed = plan->ncls == 8 && k > 0 && plan->maxlen <= kMaxClassedColumn &&
-                         (size_t)plan->hcap * (size_t)k * sizeof(float) <= bm::dds_classed_lds_budget();
-    if (stored) {
-        V = plan->ncls == 8 ? (classed ? plan->cvals : nullptr) : plan->svals;
-        if (!V) return kInvalid;              // bidmat_plan_set_values has not been called (or k does not fit the ordering)
-    }
-    if (classed)
-        return (int)bm::dds_classed(k, plan->ncols, A, B, plan->cir, plan->cperm, plan->cptr, plan->hcap, plan->hotrows, P, beta,
-                                    as_stream(stream), V, opn, stored);
-    const bm::ColTable tab = col_table(plan);
-    return (int)bm::dds_csc(k, plan->ncols, plan->nnz, A, B, Sir, Sjc, P, beta, as_stream(stream), V, opn, &tab);
+    return dds_through_plan(plan, k, A, B, Sir, Sjc, V, stored, opn, P, beta, as_stream(stream));
 }
 }  // namespace
 
 API int bidmat_dds_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc,
                         const float* V, int opn, float* P, int beta, void* stream) {
-    return dds_through_plan(plan, k, A, B, Sir, Sjc, V, false, opn, P, beta, stream);
+    return dds_plan_entry(plan, k, A, B, Sir, Sjc, V, false, opn, P, beta, stream);
 }
 
 API int bidmat_dds_plan_stored(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc,
                                int opn, float* P, void* stream) {
-    return dds_through_plan(plan, k, A, B, Sir, Sjc, nullptr, true, opn, P, 0, stream);
+    return dds_plan_entry(plan, k, A, B, Sir, Sjc, nullptr, true, opn, P, 0, stream);
 }
 
 API int bidmat_plan_set_values(bidmat_plan* plan, const float* Sdata, void* stream) {
     if (!plan) return kInvalid;
+    auto lock = bm::device_lock();
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
     if (plan->nnz == 0) return 0;
     if (!Sdata) return kInvalid;
@@ -478,6 +585,7 @@ API int bidmat_spsum_rows_plan(bidmat_plan* plan, const float* Sdata, float* out
     auto lock = bm::device_lock();
     if (!plan || (beta != 0 && beta != 1)) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (!(plan->sides & bm::PLAN_ROWS)) return kInvalid;
     if (plan->nrows == 0) return 0;
     if (!out || (plan->nnz > 0 && !Sdata && !plan->pvals)) return kInvalid;
     return (int)run_spsum_rows(plan, Sdata, out, beta, as_stream(stream));
@@ -513,7 +621,7 @@ API int bidmat_sdmult_plan(bidmat_plan* plan, int p, const float* Sdata, const f
     auto lock = bm::device_lock();
     if (!plan || p < 0) return kInvalid;
     if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
-    if (lda < plan->ncols || ldc < plan->nrows) return kInvalid;
+    if (lda < plan->ncols || ldc < plan->nrows || !(plan->sides & bm::PLAN_ROWS)) return kInvalid;
     if (plan->nrows == 0 || p == 0) return 0;
     if (!C || (plan->nnz > 0 && (!Sdata || !A))) return kInvalid;
     hipStream_t s = as_stream(stream);
@@ -799,6 +907,21 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_plan_keep_mb.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "cache_cols_after")) {
+        if (value < 0 || value > (1 << 20)) return kInvalid;
+        bm::g_cache_cols_after.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "cache_plans")) {
+        if (value < 1 || value > 1024) return kInvalid;
+        bm::g_cache_plans.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "check_plan")) {
+        if (value != 0 && value != 1) return kInvalid;
+        bm::g_check_plan.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "class_threads")) {
         if (value != 256 && value != 512 && value != 1024) return kInvalid;
         bm::g_class_threads.store((int)value);
@@ -833,6 +956,9 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "class_threads")) return bm::opt_class_threads();
     if (!strcmp(name, "class_phases")) return bm::opt_class_phases();
     if (!strcmp(name, "plan_keep_mb")) return bm::opt_plan_keep_mb();
+    if (!strcmp(name, "cache_cols_after")) return bm::g_cache_cols_after.load();
+    if (!strcmp(name, "cache_plans")) return bm::g_cache_plans.load();
+    if (!strcmp(name, "check_plan")) return bm::opt_check_plan();
     return -2;
 }
 

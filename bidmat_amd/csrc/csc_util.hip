@@ -83,20 +83,40 @@ __device__ __forceinline__ unsigned long long digest_term(unsigned long long i, 
 // (64-bit integer sums: position-sensitive, independent of the order in which threads contribute)
 // and the largest row index. A workgroup walks tiles of 4 x 256 positions with four
 // loads per array in flight per thread. out: [0] digest of ir, [1] digest of ic, [2] (int) max.
+// jc != nullptr: the column pointer of the pattern is written in the same pass (what k_compress_cols
+// does): position j closes the columns ic[j-1]+1 .. ic[j], the last position also those behind ic[n-1].
 __global__ __launch_bounds__(BM_BLOCK) void k_pattern_digest(const int* __restrict__ ir, const int* __restrict__ ic,
-                                                             long long n, unsigned long long* out) {
+                                                             long long n, unsigned long long* out, int ncols,
+                                                             int* __restrict__ jc) {
     constexpr int UN = 4;
     long long i = (long long)blockIdx.x * (UN * BM_BLOCK) + threadIdx.x;
     const long long stride = (long long)gridDim.x * (UN * BM_BLOCK);
     unsigned long long ha = 0, hb = 0;
     int m = -1;
     for (; i < n; i += stride) {
-        int r[UN], c[UN];
+        int r[UN], c[UN], cp[UN];
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const long long j = i + u * BM_BLOCK;
             r[u] = j < n ? ir[j] : -1;
             c[u] = j < n ? ic[j] : -1;
+            cp[u] = (jc != nullptr && j > 0 && j < n) ? ic[j - 1] : -1;      // the neighbour's line: a cache hit
+        }
+        if (jc != nullptr) {
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const long long j = i + u * BM_BLOCK;
+                if (j < n) {
+                    // malformed input: stay inside jc
+                    int prev = cp[u] < -1 ? -1 : (cp[u] >= ncols ? ncols - 1 : cp[u]);
+                    int cur = c[u] > ncols ? ncols : c[u];
+                    for (int q = prev + 1; q <= cur; ++q) jc[q] = (int)j;
+                    if (j == n - 1) {
+                        prev = cur < -1 ? -1 : (cur >= ncols ? ncols - 1 : cur);
+                        for (int q = prev + 1; q <= ncols; ++q) jc[q] = (int)n;
+                    }
+                }
+            }
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
@@ -283,10 +303,14 @@ hipError_t index_shift(int* p, long long n, int delta, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s) {
+hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s,
+                          int ncols, int* jc) {
     hipLaunchKernelGGL(k_digest_init, dim3(1), dim3(64), 0, s, d_out);
     if (nnz > 0)
-        hipLaunchKernelGGL(k_pattern_digest, dim3(grid_for((nnz + 3) / 4, 2048)), dim3(BM_BLOCK), 0, s, ir, ic, nnz, d_out);
+        hipLaunchKernelGGL(k_pattern_digest, dim3(grid_for((nnz + 3) / 4, 2048)), dim3(BM_BLOCK), 0, s, ir, ic, nnz, d_out,
+                           ncols, jc);
+    else if (jc != nullptr)
+        return fill_i32(jc, (long long)ncols + 1, 0, s);
     return hipGetLastError();
 }
 

@@ -431,7 +431,21 @@ hipError_t launch_dds_classed(const Shape& sh, bool exact, const DdsClassedArgs&
 
 }  // namespace
 
-size_t dds_classed_lds_budget() { return CL_LDS_MAX; }
+// Most LDS the class-ordered kernel may ask for on the current device: what the device grants one
+// workgroup, and never more than CL_LDS_MAX.
+size_t dds_classed_lds_budget() {
+    static std::mutex mu;
+    static size_t per_device[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 48u << 10;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[dev]) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || v <= 0) v = 48 << 10;
+        per_device[dev] = (size_t)v < CL_LDS_MAX ? (size_t)v : CL_LDS_MAX;
+    }
+    return per_device[dev];
+}
 
 hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const int* cir, const int* cperm,
                        const int* cptr, int hcap, const int* hotrows, float* P, int beta, hipStream_t s,
@@ -439,7 +453,7 @@ hipError_t dds_classed(int k, int ncols, const float* A, const float* B, const i
     if (ncols <= 0 || k <= 0) return hipErrorInvalidValue;          // callers route those cases to dds_csc
     if (V != nullptr && (beta != 0 || opn < 0 || opn > 14)) return hipErrorInvalidValue;
     const size_t lds_bytes = (size_t)hcap * (size_t)k * sizeof(float);
-    if (lds_bytes > CL_LDS_MAX || (hcap > 0 && !hotrows)) return hipErrorInvalidValue;
+    if (lds_bytes > dds_classed_lds_budget() || (hcap > 0 && !hotrows)) return hipErrorInvalidValue;
     Shape sh = pick_shape(k, aligned16(A) && aligned16(B));
     if (sh.V > 4) sh.V = 4;
     const bool exact = (sh.W == 4) && (k % (sh.W * sh.V * sh.LPN) == 0);

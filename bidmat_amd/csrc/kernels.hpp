@@ -14,6 +14,7 @@ int opt_class_phases(); // passes of A*S over a class-ordered pattern (1, 2, 4, 
 int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..64)
 int opt_plan_keep_mb(); // plan-build temporaries up to this many MiB stay allocated for the next build
 int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: -1 = by k_hint (default), 0 = none
+int opt_check_plan();  // 1: plans keep a digest of their pattern and the plan-taking calls compare it
 int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always
 
 // ---- CSC utilities (csc_util.hip)
@@ -45,7 +46,9 @@ hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
 hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);
 // One pass over the two index arrays of a pattern (device result, 3 x uint64): [0], [1] order- and
 // position-sensitive 64-bit digests of ir and ic, [2] (as int) the largest entry of ir (-1: empty).
-hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s);
+// jc != nullptr: also writes the column pointer jc[ncols+1] that ic implies (ic non-decreasing), in the same pass.
+hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s,
+                          int ncols = 0, int* jc = nullptr);
 
 // ---- overflow-segment table shared by dsmult and dds (spmm.hip)
 // Returns in *d_ovf a device table int[ncols+1] (exclusive scan of the number of extra

@@ -12,6 +12,7 @@
 #include <rocprim/iterator/counting_iterator.hpp>
 #include <rocprim/iterator/transform_iterator.hpp>
 #include <mutex>
+#include <initializer_list>
 #include <new>
 #include <vector>
 
@@ -195,7 +196,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nro
                                                               const int* __restrict__ hotrank,
                                                               int* __restrict__ cir,
                                                               int* __restrict__ cperm, int* __restrict__ cptr,
-                                                              int* __restrict__ maxlen) {
+                                                              int* __restrict__ maxlen, int* __restrict__ bad) {
     constexpr int NB = HOT ? 16 : 8;
     const int lane = threadIdx.x & 63;
     const long long c = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
@@ -208,6 +209,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nro
         const int j = j0 + lane;
         const bool valid = j < e;
         const int r = valid ? ir[j] : 0;
+        if ((unsigned)r >= (unsigned)nrows) *bad = 1;           // a row outside the matrix: the build fails
         const int hr = (HOT && valid && (unsigned)r < (unsigned)nrows) ? hotrank[r] : -1;
         const int bucket = HOT ? 2 * (r & 7) + (hr < 0 ? 1 : 0) : (r & 7);
 #pragma unroll
@@ -295,14 +297,43 @@ inline int bits_for(unsigned long long maxval) {
 
 }  // namespace
 
+namespace {
+void free_all(std::initializer_list<void**> bufs, hipError_t* e) {
+    for (void** b : bufs) {
+        if (*b) {
+            hipError_t f = hipFree(*b);
+            if (f != hipSuccess) *e = f;
+            *b = nullptr;
+        }
+    }
+}
+// Frees one half of a plan and marks it absent.
+hipError_t drop_rows(bidmat_plan* p) {
+    hipError_t e = hipSuccess;
+    free_all({&p->block_nnz, &p->block_seg, (void**)&p->pvals}, &e);
+    p->pc = p->perm = p->rowptr = p->segstart = p->segrow = p->rowseg = nullptr;
+    p->nseg = p->nheavy = 0;
+    for (int& x : p->xcd_start) x = 0;
+    p->row_bytes = 0;
+    p->sides &= ~PLAN_ROWS;
+    return e;
+}
+hipError_t drop_cols(bidmat_plan* p) {
+    hipError_t e = hipSuccess;
+    free_all({(void**)&p->ovf, (void**)&p->cir, (void**)&p->cperm, (void**)&p->cptr, (void**)&p->hotrows,
+              (void**)&p->cvals, (void**)&p->svals}, &e);
+    p->novf = p->ncls = p->hcap = p->maxlen = 0;
+    p->col_bytes = 0;
+    p->sides &= ~PLAN_COLS;
+    return e;
+}
+}  // namespace
+
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
-    hipError_t e = hipSuccess, f;
-    void* bufs[] = {p->block_nnz, p->block_seg, p->ovf, p->pvals, p->cir, p->cperm, p->cptr, p->hotrows, p->cvals, p->svals};
-    for (void* b : bufs)
-        if (b && (f = hipFree(b)) != hipSuccess) e = f;
+    hipError_t e = drop_rows(p), f = drop_cols(p);
     delete p;
-    return e;
+    return e != hipSuccess ? e : f;
 }
 
 namespace {
@@ -323,39 +354,42 @@ __global__ __launch_bounds__(BM_BLOCK) void k_permute_values(long long n, const 
         for (int u = 0; u < UN; ++u) { const long long j = i + u * BM_BLOCK; if (j < n) out[j] = v[u]; }
     }
 }
+
+hipError_t value_buffer(float** buf, int nnz) {
+    if (*buf) return hipSuccess;
+    hipError_t e = hipMalloc((void**)buf, sizeof(float) * (size_t)nnz);
+    if (e != hipSuccess) { (void)hipGetLastError(); *buf = nullptr; }
+    return e;
+}
 }  // namespace
 
+// Stores the values in the orders the built halves walk: plan order (row side), class order or stored
+// order (column side with / without a class ordering).
 hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s) {
     if (p->nnz <= 0) return hipSuccess;
-    if (!p->pvals) {
-        hipError_t e = hipMalloc((void**)&p->pvals, sizeof(float) * (size_t)p->nnz);
-        if (e != hipSuccess) { (void)hipGetLastError(); p->pvals = nullptr; return e; }
+    hipError_t e;
+    const dim3 grid(grid_for(((long long)p->nnz + 3) / 4, 8192)), block(BM_BLOCK);
+    if (p->sides & PLAN_ROWS) {
+        if ((e = value_buffer(&p->pvals, p->nnz)) != hipSuccess) return e;
+        hipLaunchKernelGGL(k_permute_values, grid, block, 0, s, (long long)p->nnz, data, p->perm, p->pvals);
     }
-    hipLaunchKernelGGL(k_permute_values, dim3(grid_for(((long long)p->nnz + 3) / 4, 8192)), dim3(BM_BLOCK), 0, s,
-                       (long long)p->nnz, data, p->perm, p->pvals);
-    if (p->ncls == 8) {
+    if ((p->sides & PLAN_COLS) && p->ncls == 8) {
         // A*S in passes over row classes and the fused step of DDS read their values in class order
-        if (!p->cvals) {
-            hipError_t e = hipMalloc((void**)&p->cvals, sizeof(float) * (size_t)p->nnz);
-            if (e != hipSuccess) { (void)hipGetLastError(); p->cvals = nullptr; return e; }
-        }
-        hipLaunchKernelGGL(k_permute_values, dim3(grid_for(((long long)p->nnz + 3) / 4, 8192)), dim3(BM_BLOCK), 0, s,
-                           (long long)p->nnz, data, p->cperm, p->cvals);
-    } else {
+        if ((e = value_buffer(&p->cvals, p->nnz)) != hipSuccess) return e;
+        hipLaunchKernelGGL(k_permute_values, grid, block, 0, s, (long long)p->nnz, data, p->cperm, p->cvals);
+    } else if (p->sides & PLAN_COLS) {
         // without a class ordering the fused step of DDS reads them in stored order: a plain copy
-        if (!p->svals) {
-            hipError_t e = hipMalloc((void**)&p->svals, sizeof(float) * (size_t)p->nnz);
-            if (e != hipSuccess) { (void)hipGetLastError(); p->svals = nullptr; return e; }
-        }
-        hipError_t e = hipMemcpyAsync(p->svals, data, sizeof(float) * (size_t)p->nnz, hipMemcpyDeviceToDevice, s);
-        if (e != hipSuccess) return e;
+        if ((e = value_buffer(&p->svals, p->nnz)) != hipSuccess) return e;
+        if ((e = hipMemcpyAsync(p->svals, data, sizeof(float) * (size_t)p->nnz, hipMemcpyDeviceToDevice, s)) != hipSuccess) return e;
     }
     return hipGetLastError();
 }
 
-// Builds the row-class ordering of the columns (see plan.hpp). Row indices must be valid (the row
-// histogram has checked them, or does so right after).
-static hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, const int* hotrank, hipStream_t s) {
+namespace {
+
+// Builds the row-class ordering of the columns (see plan.hpp). `bad` is set when a row index lies
+// outside the matrix.
+hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, const int* hotrank, int* bad, hipStream_t s) {
     const int ncols = plan->ncols, nnz = plan->nnz;
     if (ncols <= 0 || nnz <= 0 || (long long)ncols * 16 + 1 > 0x7fffffffLL) return hipSuccess;
     hipError_t e;
@@ -368,82 +402,42 @@ static hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int
     const long long nblk = ((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
     if (hotrank != nullptr)
         hipLaunchKernelGGL(k_class_partition<true>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank,
-                           plan->cir, plan->cperm, plan->cptr, d_maxlen);
+                           plan->cir, plan->cperm, plan->cptr, d_maxlen, bad);
     else
         hipLaunchKernelGGL(k_class_partition<false>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank,
-                           plan->cir, plan->cperm, plan->cptr, d_maxlen);
+                           plan->cir, plan->cperm, plan->cptr, d_maxlen, bad);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if ((e = hipMemcpy(&plan->maxlen, d_maxlen, sizeof(int), hipMemcpyDeviceToHost)) != hipSuccess) return e;
     plan->ncls = 8;
-    plan->index_bytes += sizeof(int) * (nsub + 1 + 2 * (size_t)nnz);
+    plan->col_bytes += sizeof(int) * (nsub + 1 + 2 * (size_t)nnz);
     return hipSuccess;
 }
 
 #define PB_CHECK(expr)                                          \
     do {                                                        \
         hipError_t _e = (expr);                                 \
-        if (_e != hipSuccess) { (void)plan_free(plan); return _e; }   \
+        if (_e != hipSuccess) return _e;                        \
     } while (0)
 
-hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,
-                      bidmat_plan** out, bool column_side) {
-    *out = nullptr;
-    // builds share the workspace arena of their device: one at a time
-    static std::mutex build_mu;
-    std::lock_guard<std::mutex> build_lock(build_mu);
-    bidmat_plan* plan = new (std::nothrow) bidmat_plan();
-    if (!plan) return hipErrorOutOfMemory;
-    hipStream_t s = nullptr;
-    PB_CHECK(hipGetDevice(&plan->device));
-    plan->nrows = nrows; plan->ncols = ncols; plan->nnz = nnz;
-    plan->seglen = opt_seglen();
-    {
-        // small patterns: shorter segments, so that the gather stage still has a few waves for
-        // every wave slot of the device
-        long long want = ((long long)nnz / 32768 / 64) * 64;
-        if (want < 64) want = 64;
-        if (want < plan->seglen) plan->seglen = (int)want;
-    }
-    if (k_hint <= 0) k_hint = 256;
-    long long pcols = (long long)opt_panel_kb() * 1024 / (4LL * k_hint);
-    if (pcols < 64) pcols = 64;
-    if (pcols > ncols) pcols = ncols > 0 ? ncols : 1;
-    if (ncols >= 8 * 64) {
-        // panels are dealt to the 8 XCDs round-robin: a multiple of 8 keeps them all equally busy
-        long long np = (ncols + pcols - 1) / pcols;
-        np = ((np + 7) / 8) * 8;
-        pcols = (ncols + np - 1) / np;
-    }
-    plan->panel_cols = (int)pcols;
-    plan->npanels = ncols > 0 ? (int)(((long long)ncols + pcols - 1) / pcols) : 1;
-    const int p8 = (plan->npanels + 7) / 8;          // panels per XCD group
+// Temporaries of one build, carved out of the library's workspace.
+struct BuildTmp {
+    int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *crank = nullptr, *scantmp = nullptr,
+        *class_count = nullptr, *segidx = nullptr, *bad = nullptr;
+    unsigned *keys_in = nullptr, *keys_out = nullptr;
+    unsigned long long *colpos_in = nullptr, *colpos_out = nullptr;
+    unsigned char* segclass = nullptr;
+    char* sorttmp = nullptr;
+    size_t sort_bytes = 0, arena_bytes = 0;
+    int sample = 1;
+};
 
-    // memory the plan keeps, part 1: everything whose size is known now
-    {
-        Arena own;
-        for (int pass = 0; pass < 2; ++pass) {
-            own.used = 0;
-            plan->rowptr = own.take<int>((size_t)nrows + 1);
-            plan->perm = own.take<int>((size_t)nnz);
-            plan->pc = own.take<int>((size_t)nnz);
-            if (pass == 0) {
-                PB_CHECK(hipMalloc(&plan->block_nnz, own.used));
-                own.base = static_cast<char*>(plan->block_nnz);
-                plan->index_bytes += own.used;
-            }
-        }
-    }
-    if (nnz == 0 || nrows == 0 || ncols == 0) {
-        PB_CHECK(fill_i32(plan->rowptr, (long long)nrows + 1, 0, s));
-        PB_CHECK(hipStreamSynchronize(s));
-        *out = plan;
-        return hipSuccess;
-    }
-
-    // column side: the overflow-segment table of the columns, kept only when a column is longer
-    // than seglen
+// Column side: the overflow-segment table of the columns (kept only when a column is longer than
+// seglen) and, where the pattern promises a gain, the row-class ordering. cnt: the row histogram.
+hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const BuildTmp& t, hipStream_t s) {
+    const int nrows = plan->nrows, ncols = plan->ncols, nnz = plan->nnz;
+    const int k_hint = plan->k_hint;
     plan->col_seglen = opt_seglen();
-    if (column_side) {
+    {
         int* tbl = nullptr;
         PB_CHECK(build_overflow_table(ncols, nnz, jc, plan->col_seglen, &tbl, s));
         if (tbl) {
@@ -453,202 +447,144 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
                 PB_CHECK(hipMalloc((void**)&plan->ovf, sizeof(int) * ((size_t)ncols + 1)));
                 PB_CHECK(hipMemcpy(plan->ovf, tbl, sizeof(int) * ((size_t)ncols + 1), hipMemcpyDeviceToDevice));
                 plan->novf = n;
-                plan->index_bytes += sizeof(int) * ((size_t)ncols + 1);
+                plan->col_bytes += sizeof(int) * ((size_t)ncols + 1);
             }
         }
     }
-
-    // temporaries: one arena out of the library's workspace
-    const size_t scan_n = (size_t)(nnz > nrows ? nnz : nrows);
-    const unsigned long long maxkey_bound = 8ULL * (unsigned long long)p8 * (unsigned long long)nrows + (unsigned long long)nrows;
-    const int rbits = bits_for((unsigned long long)nrows);
-    size_t sort_bytes = 0;
-    {
-        // both sorts share one scratch area, sized for the larger request (the second sort has
-        // at most nnz items)
-        size_t b1 = 0, b2 = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b1, (unsigned*)nullptr, (unsigned*)nullptr, (unsigned long long*)nullptr,
-                                           (unsigned long long*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b2, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
-                                           (int*)nullptr, (size_t)nnz, 0, rbits, s));
-        size_t b3 = 0;                                   // the scan over the segment starts
-        {
-            auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u),
-                                                       SegmentStart{nullptr, (unsigned)nnz, 1u});
-            PB_CHECK(rocprim::exclusive_scan(nullptr, b3, in, (int*)nullptr, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
-        }
-        sort_bytes = b1 > b2 ? b1 : b2;
-        if (b3 > sort_bytes) sort_bytes = b3;
-    }
-    Arena tmp;
-    int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *crank = nullptr, *scantmp = nullptr, *class_count = nullptr;
-    int* segidx = nullptr;
-    unsigned *keys_in = nullptr, *keys_out = nullptr;
-    unsigned long long *colpos_in = nullptr, *colpos_out = nullptr;
-    unsigned char* segclass = nullptr;
-    char* sorttmp = nullptr;
-    for (int pass = 0; pass < 2; ++pass) {
-        tmp.used = 0;
-        cnt = tmp.take<int>((size_t)nrows);
-        hflag = tmp.take<int>((size_t)nrows);
-        hrank = tmp.take<int>((size_t)nrows + 2);        // [nrows] = number of heavy rows, [nrows+1] = bad-index flag
-        hrow = tmp.take<int>((size_t)nrows);
-        crank = tmp.take<int>((size_t)nrows);            // rank of a row among its class's hot rows, or -1
-        scantmp = tmp.take<int>(scan_tmp_ints((long long)scan_n));
-        class_count = tmp.take<int>(9);
-        keys_in = tmp.take<unsigned>((size_t)nnz);       // later: ids of the segments
-        keys_out = tmp.take<unsigned>((size_t)nnz);
-        colpos_in = tmp.take<unsigned long long>((size_t)nnz);   // later: segment rows in sorted order
-        colpos_out = tmp.take<unsigned long long>((size_t)nnz);
-        segidx = tmp.take<int>((size_t)nnz + 1);
-        segclass = tmp.take<unsigned char>((size_t)nnz);
-        sorttmp = tmp.take<char>(sort_bytes);
-        if (pass == 0) {
-            hipError_t werr;
-            tmp.base = static_cast<char*>(ws_get(WS_PLAN, tmp.used, &werr));
-            if (!tmp.base) { (void)plan_free(plan); return werr; }
-        }
-    }
-    const size_t arena_bytes = tmp.used;
-    int* const bad = hrank + nrows + 1;
-
-    // 1. row histogram (integer atomics: the counts do not depend on the order)
-    PB_CHECK(fill_i32(cnt, nrows, 0, s));
-    PB_CHECK(fill_i32(hrank + nrows, 2, 0, s));
-    // few, long-lived workgroups: every one flushes its LDS histogram once at the end
-    const int sample = (long long)nnz >= HIST_SAMPLE_FROM ? HIST_SAMPLE : 1;     // cnt[r] ~ (nonzeros of row r) / sample
-    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, sample, ir, cnt, bad);
-
-    // 1b. column classes for DDS: worth it when one L2 (4 MiB) holds clearly fewer of the gathered
+    // Column classes for DDS and A*S: worth it when one L2 (4 MiB) holds clearly fewer of the gathered
     // rows' nonzeros than eight L2s with disjoint rows would. The rows are sorted by count (descending)
     // and the nonzeros of the top n1 and top 8*n1 rows compared, n1 = rows of the operand per L2. The
     // same ranking names every class's hot rows, the ones the DDS kernel keeps in LDS.
-    {
-        const int mode = column_side ? opt_col_classes() : 0;       // -1 auto, 0 never, 1 always
-        bool want = mode == 1;
-        // Measured: 100 M nonzeros, Zipf(1.1) rows, k = 256: 5.53 -> 4.78 ms. With rows of 512 bytes
-        // (k = 128, 400 M nonzeros, Zipf(1.05)) the class-ordered kernel alone is bound by its
-        // instruction stream and loses (14.8 -> 16.1 ms), but wins with each class's most frequent rows
-        // in LDS (13.75 ms): below k = 256 the hot rows are switched on with the classes.
-        const bool candidate = mode == 1 || (mode < 0 && ncols > 0 && nnz / ncols >= 64 &&
-                                             (long long)nrows * 4 * k_hint > (8LL << 20));
-        int* hotrank = nullptr;
-        if (candidate && (size_t)nrows <= (size_t)nnz) {
-            const long long n1 = (4LL << 20) / (4LL * k_hint);
-            int* iota = reinterpret_cast<int*>(keys_in);             // all free until the key sort
-            unsigned* cnt_sorted = keys_out;
-            int* rows_sorted = reinterpret_cast<int*>(colpos_in);
-            unsigned long long* cov = reinterpret_cast<unsigned long long*>(colpos_out);
-            size_t tb = 0;
-            PB_CHECK(rocprim::radix_sort_pairs_desc(nullptr, tb, reinterpret_cast<unsigned*>(cnt), cnt_sorted, iota, rows_sorted,
+    const int mode = opt_col_classes();       // -1 auto, 0 never, 1 always
+    bool want = mode == 1;
+    // Measured: 100 M nonzeros, Zipf(1.1) rows, k = 256: 5.53 -> 4.78 ms. With rows of 512 bytes
+    // (k = 128, 400 M nonzeros, Zipf(1.05)) the class-ordered kernel alone is bound by its
+    // instruction stream and loses (14.8 -> 16.1 ms), but wins with each class's most frequent rows
+    // in LDS (13.75 ms): below k = 256 the hot rows are switched on with the classes.
+    const bool candidate = mode == 1 || (mode < 0 && ncols > 0 && nnz / ncols >= 64 &&
+                                         (long long)nrows * 4 * k_hint > (8LL << 20));
+    int* hotrank = nullptr;
+    if (candidate && (size_t)nrows <= (size_t)nnz) {
+        const long long n1 = (4LL << 20) / (4LL * k_hint);
+        int* iota = reinterpret_cast<int*>(t.keys_in);             // all free until the key sort
+        unsigned* cnt_sorted = t.keys_out;
+        int* rows_sorted = reinterpret_cast<int*>(t.colpos_in);
+        unsigned long long* cov = reinterpret_cast<unsigned long long*>(t.colpos_out);
+        size_t tb = 0;
+        PB_CHECK(rocprim::radix_sort_pairs_desc(nullptr, tb, reinterpret_cast<unsigned*>(t.cnt), cnt_sorted, iota, rows_sorted,
+                                                (size_t)nrows, 0, 32, s));
+        if (tb <= t.sort_bytes) {
+            hipLaunchKernelGGL(k_iota, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, iota);
+            PB_CHECK(rocprim::radix_sort_pairs_desc(t.sorttmp, tb, reinterpret_cast<unsigned*>(t.cnt), cnt_sorted, iota, rows_sorted,
                                                     (size_t)nrows, 0, 32, s));
-            if (tb <= sort_bytes) {
-                hipLaunchKernelGGL(k_iota, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, iota);
-                PB_CHECK(rocprim::radix_sort_pairs_desc(sorttmp, tb, reinterpret_cast<unsigned*>(cnt), cnt_sorted, iota, rows_sorted,
-                                                        (size_t)nrows, 0, 32, s));
-                hipLaunchKernelGGL(k_top_coverage, dim3(1), dim3(BM_BLOCK), 0, s, nrows, reinterpret_cast<const int*>(cnt_sorted),
-                                   (int)(n1 < nrows ? n1 : nrows), (int)(8 * n1 < nrows ? 8 * n1 : nrows), cov);
-                unsigned long long h[2] = {0, 0};
-                PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
-                // at least a tenth of all gathers must move from "misses L2" to "hits L2"
-                if (mode < 0) want = (double)(h[1] - h[0]) * sample >= 0.10 * (double)nnz;
-                // hot rows per class kept in LDS. -1 (default): what 128 KiB hold when k_hint < 256, none
-                // from k = 256 on, where they were measured to change nothing (4.78 ms without, 4.85 ms with
-                // 128 rows per class: the 1024-thread persistent workgroups that share the LDS rows cost
-                // what the rows save).
-                long long hcap = opt_class_hot();
-                if (hcap < 0) hcap = k_hint < 256 ? (128LL << 10) / (4LL * k_hint) : 0;
-                if (hcap > 1024) hcap = 1024;
-                if (want && hcap > 0) {
-                    const int ntop = (int)(8 * hcap < nrows ? 8 * hcap : nrows);
-                    std::vector<int> top((size_t)ntop), cnts((size_t)ntop);
-                    PB_CHECK(hipMemcpy(top.data(), rows_sorted, sizeof(int) * (size_t)ntop, hipMemcpyDeviceToHost));
-                    PB_CHECK(hipMemcpy(cnts.data(), cnt_sorted, sizeof(int) * (size_t)ntop, hipMemcpyDeviceToHost));
-                    std::vector<int> hotrows((size_t)(8 * hcap), -1), rows, ranks;
-                    int filled[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                    for (int i = 0; i < ntop; ++i) {
-                        const int r = top[i], x = r & 7;
-                        if (cnts[i] < 2 || filled[x] >= hcap) continue;      // a row used once gains nothing
-                        hotrows[(size_t)x * hcap + filled[x]] = r;
-                        rows.push_back(r);
-                        ranks.push_back(filled[x]++);
-                    }
-                    if (!rows.empty()) {
-                        PB_CHECK(hipMalloc((void**)&plan->hotrows, sizeof(int) * hotrows.size()));
-                        PB_CHECK(hipMemcpy(plan->hotrows, hotrows.data(), sizeof(int) * hotrows.size(), hipMemcpyHostToDevice));
-                        plan->hcap = (int)hcap;
-                        plan->index_bytes += sizeof(int) * hotrows.size();
-                        hotrank = crank;
-                        PB_CHECK(fill_i32(hotrank, nrows, -1, s));
-                        // the two small lists ride in the (still free) coverage area
-                        int* d_rows = reinterpret_cast<int*>(colpos_out);
-                        int* d_ranks = d_rows + rows.size();
-                        PB_CHECK(hipMemcpy(d_rows, rows.data(), sizeof(int) * rows.size(), hipMemcpyHostToDevice));
-                        PB_CHECK(hipMemcpy(d_ranks, ranks.data(), sizeof(int) * ranks.size(), hipMemcpyHostToDevice));
-                        hipLaunchKernelGGL(k_scatter_rank, dim3(grid_for((long long)rows.size(), 1 << 30)), dim3(BM_BLOCK), 0, s,
-                                           (int)rows.size(), d_rows, d_ranks, hotrank);
-                    }
+            hipLaunchKernelGGL(k_top_coverage, dim3(1), dim3(BM_BLOCK), 0, s, nrows, reinterpret_cast<const int*>(cnt_sorted),
+                               (int)(n1 < nrows ? n1 : nrows), (int)(8 * n1 < nrows ? 8 * n1 : nrows), cov);
+            unsigned long long h[2] = {0, 0};
+            PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
+            // at least a tenth of all gathers must move from "misses L2" to "hits L2"
+            if (mode < 0) want = (double)(h[1] - h[0]) * t.sample >= 0.10 * (double)nnz;
+            // hot rows per class kept in LDS. -1 (default): what 128 KiB hold when k_hint < 256, none
+            // from k = 256 on, where they were measured to change nothing (4.78 ms without, 4.85 ms with
+            // 128 rows per class: the 1024-thread persistent workgroups that share the LDS rows cost
+            // what the rows save).
+            long long hcap = opt_class_hot();
+            if (hcap < 0) hcap = k_hint < 256 ? (long long)(dds_classed_lds_budget() / (4 * (size_t)k_hint)) : 0;
+            if (hcap > 1024) hcap = 1024;
+            if (want && hcap > 0) {
+                const int ntop = (int)(8 * hcap < nrows ? 8 * hcap : nrows);
+                std::vector<int> top((size_t)ntop), cnts((size_t)ntop);
+                PB_CHECK(hipMemcpy(top.data(), rows_sorted, sizeof(int) * (size_t)ntop, hipMemcpyDeviceToHost));
+                PB_CHECK(hipMemcpy(cnts.data(), cnt_sorted, sizeof(int) * (size_t)ntop, hipMemcpyDeviceToHost));
+                std::vector<int> hotrows((size_t)(8 * hcap), -1), rows, ranks;
+                int filled[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                for (int i = 0; i < ntop; ++i) {
+                    const int r = top[i], x = r & 7;
+                    if (cnts[i] < 2 || filled[x] >= hcap) continue;      // a row used once gains nothing
+                    hotrows[(size_t)x * hcap + filled[x]] = r;
+                    rows.push_back(r);
+                    ranks.push_back(filled[x]++);
+                }
+                if (!rows.empty()) {
+                    PB_CHECK(hipMalloc((void**)&plan->hotrows, sizeof(int) * hotrows.size()));
+                    PB_CHECK(hipMemcpy(plan->hotrows, hotrows.data(), sizeof(int) * hotrows.size(), hipMemcpyHostToDevice));
+                    plan->hcap = (int)hcap;
+                    plan->col_bytes += sizeof(int) * hotrows.size();
+                    hotrank = t.crank;
+                    PB_CHECK(fill_i32(hotrank, nrows, -1, s));
+                    // the two small lists ride in the (still free) coverage area
+                    int* d_rows = reinterpret_cast<int*>(t.colpos_out);
+                    int* d_ranks = d_rows + rows.size();
+                    PB_CHECK(hipMemcpy(d_rows, rows.data(), sizeof(int) * rows.size(), hipMemcpyHostToDevice));
+                    PB_CHECK(hipMemcpy(d_ranks, ranks.data(), sizeof(int) * ranks.size(), hipMemcpyHostToDevice));
+                    hipLaunchKernelGGL(k_scatter_rank, dim3(grid_for((long long)rows.size(), 1 << 30)), dim3(BM_BLOCK), 0, s,
+                                       (int)rows.size(), d_rows, d_ranks, hotrank);
                 }
             }
         }
-        if (want) PB_CHECK(plan_build_classes(plan, ir, jc, hotrank, s));
     }
+    if (want) PB_CHECK(plan_build_classes(plan, ir, jc, hotrank, t.bad, s));
+    return hipGetLastError();
+}
 
-    // 2. heavy rows and their ranks
+// Row side through one stable radix sort (rocPRIM) of (panel,row) keys.
+hipError_t build_rows_sorted(bidmat_plan* plan, const int* ir, const int* jc, const BuildTmp& t, int p8, hipStream_t s) {
+    const int nrows = plan->nrows, ncols = plan->ncols, nnz = plan->nnz;
+    const int rbits = bits_for((unsigned long long)nrows);
+    // heavy rows and their ranks
     int nheavy = 0;
     int h2[2] = {0, 0};                                  // {number of heavy rows, bad-index flag}
     if (plan->npanels >= 2) {
         long long thresh = (long long)plan->npanels * opt_heavy_min();
         if (thresh > 0x7fffffffLL) thresh = 0x7fffffffLL;
-        thresh = (thresh + sample - 1) / sample;
-        hipLaunchKernelGGL(k_heavy_flag, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, cnt, (int)thresh, hflag);
+        thresh = (thresh + t.sample - 1) / t.sample;
+        hipLaunchKernelGGL(k_heavy_flag, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, t.cnt, (int)thresh, t.hflag);
         // the scan writes hrank[0..nrows]; the bad-index flag sits behind it
-        PB_CHECK(scan_exclusive_i32(hflag, hrank, nrows, scantmp, s));
+        PB_CHECK(scan_exclusive_i32(t.hflag, t.hrank, nrows, t.scantmp, s));
     }
-    PB_CHECK(hipMemcpy(h2, hrank + nrows, sizeof(h2), hipMemcpyDeviceToHost));
-    if (h2[1]) { (void)plan_free(plan); return hipErrorInvalidValue; }
+    PB_CHECK(hipMemcpy(h2, t.hrank + nrows, sizeof(h2), hipMemcpyDeviceToHost));
+    if (h2[1]) return hipErrorInvalidValue;
     if (plan->npanels >= 2) {
         nheavy = h2[0];
         // keys must fit 32 bits
         if (8ULL * (unsigned long long)p8 * (unsigned long long)nheavy + (unsigned long long)nrows > 0xffffffffULL) nheavy = 0;
     }
     if (nheavy == 0) {
-        PB_CHECK(fill_i32(hflag, nrows, -1, s));        // every row is light
+        PB_CHECK(fill_i32(t.hflag, nrows, -1, s));        // every row is light
     } else {
-        hipLaunchKernelGGL(k_heavy_rows, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, hflag, hrank, hrow);
+        hipLaunchKernelGGL(k_heavy_rows, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, t.hflag, t.hrank, t.hrow);
     }
     plan->nheavy = nheavy;
 
-    // 3. keys + stable radix sort
+    // keys + stable radix sort
     {
         long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
         hipLaunchKernelGGL(k_make_keys, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nrows, jc, ir,
-                           hflag, nheavy, plan->npanels, plan->panel_cols, p8, keys_in, colpos_in, bad);
+                           t.hflag, nheavy, plan->npanels, plan->panel_cols, p8, t.keys_in, t.colpos_in, t.bad);
     }
     const unsigned long long maxkey = 8ULL * (unsigned long long)p8 * nheavy + (unsigned long long)nrows;
     const int end_bit = bits_for(maxkey);
     {
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in, keys_out, colpos_in, colpos_out, (size_t)nnz, 0, end_bit, s));
-        if (tmp_bytes > sort_bytes) { (void)plan_free(plan); return hipErrorOutOfMemory; }
-        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, keys_in, keys_out, colpos_in, colpos_out, (size_t)nnz, 0, end_bit, s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, t.keys_in, t.keys_out, t.colpos_in, t.colpos_out, (size_t)nnz, 0, end_bit, s));
+        if (tmp_bytes > t.sort_bytes) return hipErrorOutOfMemory;
+        PB_CHECK(rocprim::radix_sort_pairs(t.sorttmp, tmp_bytes, t.keys_in, t.keys_out, t.colpos_in, t.colpos_out, (size_t)nnz, 0, end_bit, s));
     }
 
-    // 4. segment boundaries
-    const SegmentStart starts{keys_out, (unsigned)nnz, (unsigned)plan->seglen};
+    // segment boundaries
+    const SegmentStart starts{t.keys_out, (unsigned)nnz, (unsigned)plan->seglen};
     {
         auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u), starts);
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::exclusive_scan(nullptr, tmp_bytes, in, segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
-        if (tmp_bytes > sort_bytes) { (void)plan_free(plan); return hipErrorOutOfMemory; }
-        PB_CHECK(rocprim::exclusive_scan(sorttmp, tmp_bytes, in, segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        PB_CHECK(rocprim::exclusive_scan(nullptr, tmp_bytes, in, t.segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        if (tmp_bytes > t.sort_bytes) return hipErrorOutOfMemory;
+        PB_CHECK(rocprim::exclusive_scan(t.sorttmp, tmp_bytes, in, t.segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
     }
     int nseg = 0;
-    PB_CHECK(hipMemcpy(&nseg, segidx + nnz, sizeof(int), hipMemcpyDeviceToHost));
+    PB_CHECK(hipMemcpy(&nseg, t.segidx + nnz, sizeof(int), hipMemcpyDeviceToHost));
     {
         int badv = 0;                                    // k_make_keys has seen every row index by now
-        PB_CHECK(hipMemcpy(&badv, bad, sizeof(int), hipMemcpyDeviceToHost));
-        if (badv) { (void)plan_free(plan); return hipErrorInvalidValue; }
+        PB_CHECK(hipMemcpy(&badv, t.bad, sizeof(int), hipMemcpyDeviceToHost));
+        if (badv) return hipErrorInvalidValue;
     }
     plan->nseg = nseg;
 
@@ -663,34 +599,216 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
             if (pass == 0) {
                 PB_CHECK(hipMalloc(&plan->block_seg, own.used));
                 own.base = static_cast<char*>(plan->block_seg);
-                plan->index_bytes += own.used;
+                plan->row_bytes += own.used;
             }
         }
     }
     // the sort's inputs are dead by now: their space holds the segment ids and the sorted rows
-    int* const segid = reinterpret_cast<int*>(keys_in);
-    unsigned* const segrow_sorted = reinterpret_cast<unsigned*>(colpos_in);
+    int* const segid = reinterpret_cast<int*>(t.keys_in);
+    unsigned* const segrow_sorted = reinterpret_cast<unsigned*>(t.colpos_in);
     unsigned* const segrow_u = reinterpret_cast<unsigned*>(plan->segrow);
-    PB_CHECK(fill_i32(class_count, 9, nseg, s));
-    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out, colpos_out,
-                       starts, segidx, hrow, nheavy > 0 ? nheavy : 1,
-                       nheavy > 0 ? p8 : 0, plan->pc, plan->perm, plan->segstart, segrow_u, segid, segclass);
+    PB_CHECK(fill_i32(t.class_count, 9, nseg, s));
+    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, t.keys_out, t.colpos_out,
+                       starts, t.segidx, t.hrow, nheavy > 0 ? nheavy : 1,
+                       nheavy > 0 ? p8 : 0, plan->pc, plan->perm, plan->segstart, segrow_u, segid, t.segclass);
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
-    hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg, segclass, class_count);
-    PB_CHECK(hipMemcpy(plan->xcd_start, class_count, sizeof(int) * 9, hipMemcpyDeviceToHost));
+    hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg, t.segclass, t.class_count);
+    PB_CHECK(hipMemcpy(plan->xcd_start, t.class_count, sizeof(int) * 9, hipMemcpyDeviceToHost));
 
-    // 5. a row's segments, in ascending segment order (stable sort by row)
+    // a row's segments, in ascending segment order (stable sort by row)
     {
         size_t tmp_bytes = 0;
         PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
-        if (tmp_bytes > sort_bytes) { (void)plan_free(plan); return hipErrorOutOfMemory; }
-        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
+        if (tmp_bytes > t.sort_bytes) return hipErrorOutOfMemory;
+        PB_CHECK(rocprim::radix_sort_pairs(t.sorttmp, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
         PB_CHECK(coo_compress_cols(nrows, nseg, reinterpret_cast<const int*>(segrow_sorted), plan->rowptr, s));
         PB_CHECK(hipStreamSynchronize(s));
     }
+    return hipGetLastError();
+}
+
+// Builds the halves named in `sides` into `plan` (whose sizes and k_hint are set). On failure the
+// caller drops what was begun.
+hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int sides) {
+    const bool rows = (sides & PLAN_ROWS) != 0, cols = (sides & PLAN_COLS) != 0;
+    const int nrows = plan->nrows, ncols = plan->ncols, nnz = plan->nnz;
+    const int k_hint = plan->k_hint;
+    hipStream_t s = nullptr;
+    int p8 = 0;
+    if (rows) {
+        plan->seglen = opt_seglen();
+        {
+            // small patterns: shorter segments, so that the gather stage still has a few waves for
+            // every wave slot of the device
+            long long want = ((long long)nnz / 32768 / 64) * 64;
+            if (want < 64) want = 64;
+            if (want < plan->seglen) plan->seglen = (int)want;
+        }
+        long long pcols = (long long)opt_panel_kb() * 1024 / (4LL * k_hint);
+        if (pcols < 64) pcols = 64;
+        if (pcols > ncols) pcols = ncols > 0 ? ncols : 1;
+        if (ncols >= 8 * 64) {
+            // panels are dealt to the 8 XCDs round-robin: a multiple of 8 keeps them all equally busy
+            long long np = (ncols + pcols - 1) / pcols;
+            np = ((np + 7) / 8) * 8;
+            pcols = (ncols + np - 1) / np;
+        }
+        plan->panel_cols = (int)pcols;
+        plan->npanels = ncols > 0 ? (int)(((long long)ncols + pcols - 1) / pcols) : 1;
+        p8 = (plan->npanels + 7) / 8;          // panels per XCD group
+        // memory the plan keeps, part 1: everything whose size is known now
+        Arena own;
+        for (int pass = 0; pass < 2; ++pass) {
+            own.used = 0;
+            plan->rowptr = own.take<int>((size_t)nrows + 1);
+            plan->perm = own.take<int>((size_t)nnz);
+            plan->pc = own.take<int>((size_t)nnz);
+            if (pass == 0) {
+                PB_CHECK(hipMalloc(&plan->block_nnz, own.used));
+                own.base = static_cast<char*>(plan->block_nnz);
+                plan->row_bytes += own.used;
+            }
+        }
+    }
+    if (nnz == 0 || nrows == 0 || ncols == 0) {
+        if (rows) {
+            PB_CHECK(fill_i32(plan->rowptr, (long long)nrows + 1, 0, s));
+            PB_CHECK(hipStreamSynchronize(s));
+        }
+        if (cols) plan->col_seglen = opt_seglen();
+        return hipSuccess;
+    }
+
+    // temporaries: one arena out of the library's workspace. The row side sorts all nonzeros; the
+    // column side alone only ranks the rows.
+    const size_t nitem = rows ? (size_t)nnz : (size_t)(nrows > (1 << 14) ? nrows : (1 << 14));
+    const size_t scan_n = (size_t)(rows && nnz > nrows ? nnz : nrows);
+    const unsigned long long maxkey_bound = 8ULL * (unsigned long long)p8 * (unsigned long long)nrows + (unsigned long long)nrows;
+    const int rbits = bits_for((unsigned long long)nrows);
+    BuildTmp t;
+    {
+        // all sorts and scans share one scratch area, sized for the largest request
+        size_t b1 = 0, b2 = 0, b3 = 0, b4 = 0;
+        if (rows) {
+            PB_CHECK(rocprim::radix_sort_pairs(nullptr, b1, (unsigned*)nullptr, (unsigned*)nullptr, (unsigned long long*)nullptr,
+                                               (unsigned long long*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
+            PB_CHECK(rocprim::radix_sort_pairs(nullptr, b2, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
+                                               (int*)nullptr, (size_t)nnz, 0, rbits, s));
+            auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u),
+                                                       SegmentStart{nullptr, (unsigned)nnz, 1u});
+            PB_CHECK(rocprim::exclusive_scan(nullptr, b3, in, (int*)nullptr, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        } else {
+            PB_CHECK(rocprim::radix_sort_pairs_desc(nullptr, b4, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr, (int*)nullptr,
+                                                    (size_t)nrows, 0, 32, s));
+        }
+        t.sort_bytes = b1 > b2 ? b1 : b2;
+        if (b3 > t.sort_bytes) t.sort_bytes = b3;
+        if (b4 > t.sort_bytes) t.sort_bytes = b4;
+    }
+    Arena tmp;
+    for (int pass = 0; pass < 2; ++pass) {
+        tmp.used = 0;
+        t.cnt = tmp.take<int>((size_t)nrows);
+        t.hflag = tmp.take<int>((size_t)nrows);
+        t.hrank = tmp.take<int>((size_t)nrows + 2);        // [nrows] = number of heavy rows, [nrows+1] = bad-index flag
+        t.hrow = tmp.take<int>((size_t)nrows);
+        t.crank = tmp.take<int>((size_t)nrows);            // rank of a row among its class's hot rows, or -1
+        t.scantmp = tmp.take<int>(scan_tmp_ints((long long)scan_n));
+        t.class_count = tmp.take<int>(9);
+        t.keys_in = tmp.take<unsigned>(nitem);             // later: ids of the segments
+        t.keys_out = tmp.take<unsigned>(nitem);
+        t.colpos_in = tmp.take<unsigned long long>(nitem); // later: segment rows in sorted order
+        t.colpos_out = tmp.take<unsigned long long>(nitem);
+        t.segidx = tmp.take<int>(rows ? (size_t)nnz + 1 : 1);
+        t.segclass = tmp.take<unsigned char>(rows ? (size_t)nnz : 1);
+        t.sorttmp = tmp.take<char>(t.sort_bytes);
+        if (pass == 0) {
+            hipError_t werr;
+            tmp.base = static_cast<char*>(ws_get(WS_PLAN, tmp.used, &werr));
+            if (!tmp.base) return werr;
+        }
+    }
+    t.arena_bytes = tmp.used;
+    t.bad = t.hrank + nrows + 1;
+
+    // row histogram (integer atomics: the counts do not depend on the order)
+    PB_CHECK(fill_i32(t.cnt, nrows, 0, s));
+    PB_CHECK(fill_i32(t.hrank + nrows, 2, 0, s));
+    // few, long-lived workgroups: every one flushes its LDS histogram once at the end
+    t.sample = (long long)nnz >= HIST_SAMPLE_FROM ? HIST_SAMPLE : 1;     // cnt[r] ~ (nonzeros of row r) / sample
+    hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, t.sample, ir, t.cnt, t.bad);
+
+    if (cols) {
+        PB_CHECK(build_cols(plan, ir, jc, t, s));
+        if (!rows) {
+            int badv = 0;                                // set by the histogram (as far as it looked) or the class ordering
+            PB_CHECK(hipMemcpy(&badv, t.bad, sizeof(int), hipMemcpyDeviceToHost));
+            if (badv) return hipErrorInvalidValue;
+        }
+    }
+    if (rows) PB_CHECK(build_rows_sorted(plan, ir, jc, t, p8, s));
     PB_CHECK(hipGetLastError());
-    if (arena_bytes > ((size_t)opt_plan_keep_mb() << 20)) PB_CHECK(ws_drop(WS_PLAN));
+    if (t.arena_bytes > ((size_t)opt_plan_keep_mb() << 20)) PB_CHECK(ws_drop(WS_PLAN));
+    return hipSuccess;
+}
+
+// builds share the workspace arena of their device: one at a time
+std::mutex g_build_mu;
+
+}  // namespace
+
+hipError_t plan_digest(int nnz, int ncols, const int* ir, const int* jc, unsigned long long d[2]) {
+    d[0] = d[1] = 0;
+    hipError_t e;
+    unsigned long long* dm = (unsigned long long*)ws_get(WS_MISC, 64, &e);
+    if (!dm) return e;
+    if ((e = pattern_digest(ir, ir, nnz, dm, nullptr)) != hipSuccess) return e;
+    if ((e = pattern_digest(jc, jc, (long long)ncols + 1, dm + 4, nullptr)) != hipSuccess) return e;
+    unsigned long long h[5];
+    if ((e = hipMemcpy(h, dm, sizeof(h), hipMemcpyDeviceToHost)) != hipSuccess) return e;
+    d[0] = h[0];
+    d[1] = h[4];
+    return hipSuccess;
+}
+
+hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,
+                      bidmat_plan** out, int sides) {
+    *out = nullptr;
+    if ((sides & ~(PLAN_ROWS | PLAN_COLS)) != 0 || sides == 0) return hipErrorInvalidValue;
+    std::lock_guard<std::mutex> build_lock(g_build_mu);
+    bidmat_plan* plan = new (std::nothrow) bidmat_plan();
+    if (!plan) return hipErrorOutOfMemory;
+    hipError_t e = hipGetDevice(&plan->device);
+    plan->nrows = nrows; plan->ncols = ncols; plan->nnz = nnz;
+    plan->k_hint = k_hint > 0 ? k_hint : 256;
+    if (e == hipSuccess) e = build_sides(plan, ir, jc, sides);
+    if (e == hipSuccess && opt_check_plan() && nnz > 0 && ncols > 0) {
+        e = plan_digest(nnz, ncols, ir, jc, plan->digest);
+        plan->has_digest = e == hipSuccess;
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        (void)plan_free(plan);
+        return e;
+    }
+    plan->sides = sides;
     *out = plan;
+    return hipSuccess;
+}
+
+hipError_t plan_extend(bidmat_plan* plan, const int* ir, const int* jc, int sides) {
+    if (!plan || (sides & ~(PLAN_ROWS | PLAN_COLS)) != 0) return hipErrorInvalidValue;
+    const int missing = sides & ~plan->sides;
+    if (missing == 0) return hipSuccess;
+    std::lock_guard<std::mutex> build_lock(g_build_mu);
+    hipError_t e = build_sides(plan, ir, jc, missing);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        if (missing & PLAN_ROWS) (void)drop_rows(plan);
+        if (missing & PLAN_COLS) (void)drop_cols(plan);
+        return e;
+    }
+    plan->sides |= missing;
     return hipSuccess;
 }
 

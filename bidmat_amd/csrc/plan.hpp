@@ -11,9 +11,19 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 
+// A plan has two independent halves. The row side (PLAN_ROWS) serves A*^S, S*A and sparse row sums;
+// the column side (PLAN_COLS) serves A*S and DDS. Either can be built alone and the other added later.
+namespace bm { enum { PLAN_ROWS = 1, PLAN_COLS = 2 }; }
+
 struct bidmat_plan {
     int device = 0;
     int nrows = 0, ncols = 0, nnz = 0;
+    int sides = 0;           // PLAN_ROWS | PLAN_COLS: which halves have been built
+    int k_hint = 0;          // dense leading dimension the plan was sized for
+    // 64-bit digests of the ir and jc arrays the plan was built from, taken when option "check_plan" is on:
+    // the plan-taking calls then refuse a pattern that is not the plan's
+    bool has_digest = false;
+    unsigned long long digest[2] = {0, 0};
     int nseg = 0;            // number of segments
     int nheavy = 0;          // rows cut by column panels
     int npanels = 0;
@@ -32,7 +42,8 @@ struct bidmat_plan {
     void* block_nnz = nullptr;   // owns pc, perm, rowptr
     void* block_seg = nullptr;   // owns segstart, segrow, rowseg
     // (the nseg*k partial sums of a call live in the scratch of the stream it runs on, not here)
-    size_t index_bytes = 0;
+    size_t row_bytes = 0;        // device bytes of the row side's index arrays
+    size_t col_bytes = 0;        // device bytes of the column side's index arrays
     // Column side (A*S and DDS through the plan): the overflow-segment table of the columns is a
     // function of jc and seglen only, so it is built once here instead of on every call.
     int col_seglen = 0;          // seglen in force when the plan was built
@@ -62,11 +73,15 @@ struct bidmat_plan {
 };
 
 namespace bm {
-// column_side == false: only the row side (A*^S, row sums) is built - no column overflow table, no
-// class ordering - for callers that will never run A*S or DDS through the plan.
+// sides: which halves to build now (PLAN_ROWS, PLAN_COLS or both).
 hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,
-                      bidmat_plan** out, bool column_side = true);
+                      bidmat_plan** out, int sides = PLAN_ROWS | PLAN_COLS);
+// Builds the halves named in `sides` that the plan does not hold yet, from the pattern the plan was
+// made from. On failure the plan keeps the halves it had.
+hipError_t plan_extend(bidmat_plan* p, const int* ir, const int* jc, int sides);
 hipError_t plan_free(bidmat_plan* p);
+// d[0], d[1] = digests of ir[nnz] and jc[ncols+1] (blocking; default stream)
+hipError_t plan_digest(int nnz, int ncols, const int* ir, const int* jc, unsigned long long d[2]);
 // pvals[p] = data[perm[p]] (allocates pvals on first use).
 hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s);
 }  // namespace bm

@@ -183,12 +183,21 @@ GMatP GMat::newOrCheckGMat(int nr, int nc, GMatP outmat, long long g1, long long
     return m;
 }
 
+namespace {
+// C = beta*C + A*S: through the plan of S's pattern when it has one (or is due one), else the plain kernel
+int dsmultDispatch(const GMat& A, GSMat& S, float* C, int beta) {
+    if (bidmat_plan* p = S.planIfDue(A.nrows))
+        return bidmat_dsmult_plan(p, A.nrows, A.pdata, S.pdata, S.pir, S.pjc, C, beta, nullptr);
+    return bidmat_dsmult_csc(A.nrows, S.ncols, S.nnz(), A.pdata, S.pdata, S.pir, S.pjc, C, beta, nullptr);
+}
+}  // namespace
+
 GMatP GMat::GSMult(const GSMatP& a, GMatP oldmat) {
     if (ncols != a->nrows) fail(fmt("GSMult dimensions mismatch (%d %d) (%d %d)", nrows, ncols, a->nrows, a->ncols));
     GMatP out = newOrCheckGMat(nrows, a->ncols, oldmat, GUID, a->GUID, opHash("GSMult"));
     // the reference clears `out` and accumulates (GMat.scala:1047-1048); beta = 0 overwrites instead
     Mat::nflops += 2LL * nrows * a->nnz();
-    int err = bidmat_dsmult_csc(nrows, a->ncols, a->nnz(), pdata, a->pdata, a->pir, a->pjc, out->pdata, 0, nullptr);
+    int err = dsmultDispatch(*this, *a, out->pdata, 0);
     if (err == 0) err = bidmat_stream_synchronize(nullptr);
     if (err != 0) fail(std::string("GMult: HIP kernel error in dsmult ") + bidmat_error_string(err));
     return out;
@@ -198,7 +207,7 @@ GMatP GMat::madd(const GSMatP& a, GMatP out) {
     if (ncols != a->nrows || nrows != out->nrows || a->ncols != out->ncols)
         fail(fmt("GSMadd dimensions mismatch (%d %d) (%d %d) (%d %d)", nrows, ncols, a->nrows, a->ncols, out->nrows, out->ncols));
     Mat::nflops += 2LL * nrows * a->nnz();
-    int err = bidmat_dsmult_csc(nrows, a->ncols, a->nnz(), pdata, a->pdata, a->pir, a->pjc, out->pdata, 1, nullptr);
+    int err = dsmultDispatch(*this, *a, out->pdata, 1);
     if (err == 0) err = bidmat_stream_synchronize(nullptr);
     if (err != 0) fail(std::string("GMult: HIP kernel error in dsmult ") + bidmat_error_string(err));
     return out;
@@ -373,15 +382,41 @@ PlanHolder::~PlanHolder() {
     if (plan) bidmat_plan_destroy(plan);
 }
 
-GSMat::GSMat(int nr, int nc, int nnz, int rn)
-    : nrows(nr), ncols(nc), nnz0(nnz), pir(nullptr), pic(nullptr), pjc(nullptr), pdata(nullptr),
-      realnnz(std::max(1, rn)), GUID(Mat::newGUID()), myGPU(getGPU()), planHolder(std::make_shared<PlanHolder>()) {
-    if (Mat::debugMem) fprintf(stderr, "GSMat %d %d %d, %d %f\n", nr, nc, nnz, getGPU(), GPUmem().first);
+Pattern::Pattern(int ncols, int realnnz) {
     void* p = nullptr;
     int err = bidmat_malloc(&p, (long long)sizeof(int) * realnnz); pir = (int*)p;
     if (err == 0) { err = bidmat_malloc(&p, (long long)sizeof(int) * realnnz); pic = (int*)p; }
     if (err == 0) { err = bidmat_malloc(&p, (long long)sizeof(int) * ((long long)ncols + 1)); pjc = (int*)p; }
-    if (err == 0) { err = bidmat_malloc(&p, (long long)sizeof(float) * realnnz); pdata = (float*)p; }
+    if (err != 0) {
+        this->~Pattern();
+        fail(std::string("HIP error in GSMat() ") + bidmat_error_string(err));
+    }
+}
+
+Pattern::~Pattern() {
+    if (pic) bidmat_free(pic);
+    if (pir) bidmat_free(pir);
+    if (pjc) bidmat_free(pjc);
+    pic = pir = pjc = nullptr;
+}
+
+GSMat::GSMat(int nr, int nc, int nnz, int rn)
+    : nrows(nr), ncols(nc), nnz0(nnz), pir(nullptr), pic(nullptr), pjc(nullptr), pdata(nullptr),
+      realnnz(std::max(1, rn)), GUID(Mat::newGUID()), myGPU(getGPU()), planHolder(std::make_shared<PlanHolder>()) {
+    if (Mat::debugMem) fprintf(stderr, "GSMat %d %d %d, %d %f\n", nr, nc, nnz, getGPU(), GPUmem().first);
+    pattern = std::make_shared<Pattern>(ncols, realnnz);
+    pir = pattern->pir; pic = pattern->pic; pjc = pattern->pjc;
+    void* p = nullptr;
+    int err = bidmat_malloc(&p, (long long)sizeof(float) * realnnz); pdata = (float*)p;
+    if (err != 0) { free(); fail(std::string("HIP error in GSMat() ") + bidmat_error_string(err)); }
+}
+
+GSMat::GSMat(int nr, int nc, int nnz, int rn, const GSMat& like)
+    : nrows(nr), ncols(nc), nnz0(nnz), pir(like.pir), pic(like.pic), pjc(like.pjc), pdata(nullptr),
+      realnnz(std::max(1, rn)), GUID(Mat::newGUID()), myGPU(getGPU()), pattern(like.pattern), planHolder(like.planHolder) {
+    if (Mat::debugMem) fprintf(stderr, "GSMat %d %d %d (shared pattern), %d %f\n", nr, nc, nnz, getGPU(), GPUmem().first);
+    void* p = nullptr;
+    int err = bidmat_malloc(&p, (long long)sizeof(float) * realnnz); pdata = (float*)p;
     if (err != 0) { free(); fail(std::string("HIP error in GSMat() ") + bidmat_error_string(err)); }
 }
 
@@ -389,10 +424,23 @@ GSMat::~GSMat() { free(); }
 
 void GSMat::free() {
     if (pdata) bidmat_free(pdata);
-    if (pic) bidmat_free(pic);
-    if (pir) bidmat_free(pir);
-    if (pjc) bidmat_free(pjc);
-    pdata = nullptr; pic = pir = pjc = nullptr;
+    pdata = nullptr;
+    pattern.reset();                       // the arrays go with their last user
+    pic = pir = pjc = nullptr;
+}
+
+void GSMat::ownPattern() {
+    if (pattern.use_count() > 1) {
+        pattern = std::make_shared<Pattern>(ncols, realnnz);
+        pir = pattern->pir; pic = pattern->pic; pjc = pattern->pjc;
+    }
+    planHolder = std::make_shared<PlanHolder>();      // new indices: any older plan is stale
+}
+
+void GSMat::sharePattern(const GSMat& like) {
+    pattern = like.pattern;
+    pir = like.pir; pic = like.pic; pjc = like.pjc;
+    planHolder = like.planHolder;
 }
 
 GSMatP GSMat::make(int nr, int nc, int nnz, int realnnz) { return std::make_shared<GSMat>(nr, nc, nnz, realnnz); }
@@ -402,32 +450,34 @@ GSMat& GSMat::clear() {
     return *this;
 }
 
-GSMatP GSMat::newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP oldmat) {
+// like != nullptr: a matrix that has to be made new takes `like`'s pattern instead of index arrays of its own
+GSMatP GSMat::newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP oldmat, const GSMat* like) {
+    auto fresh = [&](int rn) { return like ? std::make_shared<GSMat>(nr, nc, nnz, rn, *like) : make(nr, nc, nnz, rn); };
     if (!oldmat || (oldmat->nrows == 0 && oldmat->ncols == 0)) {
-        if (Mat::useGPUcache) return make(nr, nc, nnz, std::max((int)(Mat::recycleGrow * nnz), realnnz));
-        return make(nr, nc, nnz, realnnz);
+        if (Mat::useGPUcache) return fresh(std::max((int)(Mat::recycleGrow * nnz), realnnz));
+        return fresh(realnnz);
     }
     if (oldmat->nrows == nr && oldmat->ncols == nc && nnz <= oldmat->realnnz) {
         oldmat->nnz0 = nnz;
         return oldmat;
     }
     // recycle (GSMat.scala:234-248): the column pointer depends on ncols, so a new shape gets new buffers
-    GSMatP m = Mat::useGPUcache ? make(nr, nc, nnz, (int)(Mat::recycleGrow * nnz)) : make(nr, nc, nnz, nnz);
+    GSMatP m = Mat::useGPUcache ? fresh((int)(Mat::recycleGrow * nnz)) : fresh(nnz);
     if (oldmat->nrows == nr && oldmat->ncols == nc) m->GUID = oldmat->GUID;
     return m;
 }
 
 GSMatP GSMat::newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP outmat, long long g1, long long g2,
-                              long long g3, long long oph) {
+                              long long g3, long long oph, const GSMat* like) {
     GSMatP m;
     if (outmat || !Mat::useGPUcache) {
-        m = newOrCheckGSMat(nr, nc, nnz, realnnz, outmat);
+        m = newOrCheckGSMat(nr, nc, nnz, realnnz, outmat, like);
     } else {
         Key key(g1, g2, g3, oph, getGPU());
         std::lock_guard<std::mutex> lock(g_cache_mu);
         auto it = g_scache.find(key);
         GSMatP res = it == g_scache.end() ? nullptr : it->second;
-        m = newOrCheckGSMat(nr, nc, nnz, realnnz, res);
+        m = newOrCheckGSMat(nr, nc, nnz, realnnz, res, like);
         if (m != res) g_scache[key] = m;
     }
     checkThread(m->myGPU, "newOrCheckGSMat3", m->GUID);
@@ -447,7 +497,7 @@ GSMatP GSMat::fromHost(int nr, int nc, int n, const float* data, const int* ir, 
     if (guid == 0) guid = Mat::newGUID();                  // bare arrays: never share a cached output
     GSMatP out = newOrCheckGSMat(nr, nc, n, n, b, guid, 0, 0, opHash("fromSMat"));
     out->nnz0 = n;
-    out->planHolder = std::make_shared<PlanHolder>();      // new pattern: any older plan is stale
+    out->ownPattern();                                     // new indices: nothing shared, any older plan is stale
     Staging st;
     st.upload(out->pjc, jc, sizeof(int) * ((size_t)nc + 1));
     st.upload(out->pir, ir, sizeof(int) * (size_t)n);
@@ -500,6 +550,12 @@ bidmat_plan* GSMat::plan(int k_hint) {
     return planHolder->plan;
 }
 
+bidmat_plan* GSMat::planIfDue(int k_hint) {
+    if (planHolder->plan) return planHolder->plan;
+    if (++planHolder->uses < 2) return nullptr;
+    return plan(k_hint);
+}
+
 GMatP GSMat::sum(int n, GMatP oldmat) {
     const int nn = n > 0 ? n : (nrows == 1 ? 2 : 1);
     GMatP out = GMat::newOrCheckGMat(nn == 1 ? 1 : nrows, nn == 1 ? ncols : 1, oldmat, GUID, n, opHash("sum"));
@@ -514,13 +570,12 @@ GMatP GSMat::sum(int n, GMatP oldmat) {
 }
 
 GSMatP GSMat::copy(GSMatP omat, long long key1, long long key2) {
-    GSMatP out = newOrCheckGSMat(nrows, ncols, nnz0, realnnz, omat, GUID, key1, key2, opHash("copy"));
+    GSMatP out = newOrCheckGSMat(nrows, ncols, nnz0, realnnz, omat, GUID, key1, key2, opHash("copy"), this);
     if (out.get() != this) {
-        hipcheck(bidmat_memcpy_d2d(out->pir, pir, (long long)sizeof(int) * nnz0), "GSMat.copy");
-        hipcheck(bidmat_memcpy_d2d(out->pic, pic, (long long)sizeof(int) * nnz0), "GSMat.copy");
-        hipcheck(bidmat_memcpy_d2d(out->pjc, pjc, (long long)sizeof(int) * ((long long)ncols + 1)), "GSMat.copy");
+        // the copy has values of its own and points at the same index arrays (and plan): the indices of
+        // a GSMat only ever change through calls that take private arrays first
+        if (out->pattern != pattern) out->sharePattern(*this);
         hipcheck(bidmat_memcpy_d2d(out->pdata, pdata, (long long)sizeof(float) * nnz0), "GSMat.copy");
-        out->planHolder = planHolder;
     }
     return out;
 }
@@ -550,7 +605,7 @@ GSMatP GSMat::nHot(const std::vector<int>& cats, int n, int ncols, int ncats0) {
 GSMatP GSMat::t(GSMatP omat) {
     GSMatP out = newOrCheckGSMat(ncols, nrows, nnz0, realnnz, omat, GUID, 0, 0, opHash("t"));
     out->nnz0 = nnz0;
-    out->planHolder = std::make_shared<PlanHolder>();
+    out->ownPattern();
     int err = bidmat_csc_transpose(nrows, ncols, nnz0, pdata, pir, pjc, out->pdata, out->pir, out->pjc);
     if (err == 0) err = bidmat_csc_expand_cols(out->ncols, nnz0, out->pjc, out->pic, nullptr);
     if (err == 0) err = bidmat_stream_synchronize(nullptr);
@@ -572,10 +627,10 @@ GSMatP GSMat::colslice(int col1, int col2, GSMatP omat) {
     hipcheck(bidmat_csc_colslice_range(ncols, col1, col2, pjc, &starti, &newnnz), "GSMAT.colslice");
     const int newncols = col2 - col1;
     GSMatP out = newOrCheckGSMat(nrows, newncols, newnnz, newnnz, omat, GUID, col1, col2, opHash("colslice"));
+    out->ownPattern();                                      // another pattern: any plan is rebuilt on demand
     int err = bidmat_csc_colslice(col1, col2, starti, newnnz, pjc, pir, pdata, out->pjc, out->pir, out->pic, out->pdata, nullptr);
     if (err == 0) err = bidmat_stream_synchronize(nullptr);
     if (err != 0) fail(std::string("HIP error in GSMAT.colslice ") + bidmat_error_string(err));
-    out->planHolder = std::make_shared<PlanHolder>();      // another pattern: any plan is rebuilt on demand
     return out;
 }
 
@@ -614,16 +669,17 @@ GMatP GSMat::SDTMult(const GMatP& a, GMatP omat) {
 GSMatP GSMat::DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat) {
     if (A->nrows != B->nrows || C->nrows != A->ncols || C->ncols != B->ncols)
         fail(fmt("dimensions mismatch %d,%d  %d,%d  %d,%d", A->nrows, A->ncols, B->nrows, B->ncols, C->nrows, C->ncols));
-    GSMatP out = newOrCheckGSMat(C->nrows, C->ncols, C->nnz(), C->realnnz, oldmat, A->GUID, B->GUID, C->GUID, opHash("DDS"));
-    if (out != C) {
-        // the result carries C's pattern: row indices, column indices AND the column pointer
-        // (the reference copies pir and pic only and leaves out.pjc stale, GSMat.scala:656-661)
-        hipcheck(bidmat_memcpy_d2d(out->pir, C->pir, (long long)sizeof(int) * C->nnz()), "DDS row copy error");
-        hipcheck(bidmat_memcpy_d2d(out->pic, C->pic, (long long)sizeof(int) * C->nnz()), "DDS column copy error");
-        hipcheck(bidmat_memcpy_d2d(out->pjc, C->pjc, (long long)sizeof(int) * ((long long)C->ncols + 1)), "DDS column pointer copy error");
-        out->planHolder = C->planHolder;       // same pattern, same plan
-    }
-    int err = bidmat_dds_csc(A->nrows, C->ncols, C->nnz(), A->pdata, B->pdata, C->pir, C->pjc, out->pdata, 0, nullptr);
+    GSMatP out = newOrCheckGSMat(C->nrows, C->ncols, C->nnz(), C->realnnz, oldmat, A->GUID, B->GUID, C->GUID, opHash("DDS"), C.get());
+    // The result carries C's pattern: row indices, column indices AND the column pointer (the reference
+    // copies pir and pic, 8 bytes per nonzero, and leaves out.pjc stale, GSMat.scala:656-661). Here the
+    // result points at C's index arrays; whoever rewrites the indices of either matrix later takes
+    // private arrays first (ownPattern).
+    if (out != C && out->pattern != C->pattern) out->sharePattern(*C);
+    int err;
+    if (bidmat_plan* p = C->planIfDue(A->nrows))
+        err = bidmat_dds_plan(p, A->nrows, A->pdata, B->pdata, C->pir, C->pjc, nullptr, 0, out->pdata, 0, nullptr);
+    else
+        err = bidmat_dds_csc(A->nrows, C->ncols, C->nnz(), A->pdata, B->pdata, C->pir, C->pjc, out->pdata, 0, nullptr);
     if (err == 0) err = bidmat_stream_synchronize(nullptr);
     if (err != 0) fail(fmt("GPU %d DDS kernel error %s", getGPU(), bidmat_error_string(err)));
     Mat::nflops += 2LL * C->nnz() * A->nrows;
@@ -632,12 +688,8 @@ GSMatP GSMat::DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat
 
 GSMatP GSMat::withValues(const GMatP& vals) const {
     if (vals->length() != nnz0) fail(fmt("withValues: %lld values for %d nonzeros", vals->length(), nnz0));
-    GSMatP out = make(nrows, ncols, nnz0, realnnz);
-    hipcheck(bidmat_memcpy_d2d(out->pir, pir, (long long)sizeof(int) * nnz0), "pattern copy error");
-    hipcheck(bidmat_memcpy_d2d(out->pic, pic, (long long)sizeof(int) * nnz0), "pattern copy error");
-    hipcheck(bidmat_memcpy_d2d(out->pjc, pjc, (long long)sizeof(int) * ((long long)ncols + 1)), "pattern copy error");
+    GSMatP out = std::make_shared<GSMat>(nrows, ncols, nnz0, realnnz, *this);      // same index arrays, same plan
     hipcheck(bidmat_memcpy_d2d(out->pdata, vals->pdata, (long long)sizeof(float) * nnz0), "value copy error");
-    out->planHolder = planHolder;
     return out;
 }
 

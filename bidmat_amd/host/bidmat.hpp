@@ -139,11 +139,29 @@ public:
     static GMatP newOrCheckGMat(int nr, int nc, GMatP outmat, long long g1, long long g2, long long opHash);
 };
 
-// shared by all GSMats that carry the same pattern buffers' content (a DDS result, V./R ...)
+// The plan of a pattern, shared by all GSMats that carry the same pattern (a DDS result, V./R ...).
+// A*^S and sparse row sums cannot run without a plan and build it at once; A*S and DDS run through it
+// when it exists and build it on their second call on the pattern (`uses` counts them), so a pattern
+// that is multiplied once never pays for a plan.
 struct PlanHolder {
     bidmat_plan* plan = nullptr;
     int k_hint = 0;
+    int uses = 0;
     ~PlanHolder();
+};
+
+// The index arrays of a device sparse matrix. Several GSMats may share one Pattern (the result of DDS
+// has the pattern of its third operand: the reference copies 8 bytes per nonzero for it,
+// GSMat.scala:656-661; here the result points at the same arrays). A GSMat that is about to have its
+// indices rewritten takes a private Pattern first (GSMat::ownPattern).
+struct Pattern {
+    int* pir = nullptr;
+    int* pic = nullptr;
+    int* pjc = nullptr;
+    Pattern(int ncols, int realnnz);       // allocates; throws on failure
+    ~Pattern();
+    Pattern(const Pattern&) = delete;
+    Pattern& operator=(const Pattern&) = delete;
 };
 
 // ---- device sparse (GSMat): pir/pic/pjc/pdata, all 0-based on the device
@@ -151,16 +169,19 @@ class GSMat : public std::enable_shared_from_this<GSMat> {
 public:
     int nrows, ncols;
     int nnz0;
-    int* pir;
+    int* pir;                  // = pattern->pir etc.: the names the reference uses
     int* pic;
     int* pjc;
     float* pdata;
     int realnnz;
     long long GUID;
     int myGPU;
+    std::shared_ptr<Pattern> pattern;
     std::shared_ptr<PlanHolder> planHolder;
 
     GSMat(int nr, int nc, int nnz, int realnnz);
+    // a matrix with its own values and the pattern (and plan) of `like`
+    GSMat(int nr, int nc, int nnz, int realnnz, const GSMat& like);
     ~GSMat();
     int nnz() const { return nnz0; }
     std::string mytype() const { return "GSMat"; }
@@ -189,11 +210,19 @@ public:
     static GSMatP DDS(const GMatP& A, const GMatP& B, const GSMatP& C, GSMatP oldmat);   // GSMat.scala:649-667
     // a sparse matrix with this pattern and other values (the V./R step keeps V's pattern)
     GSMatP withValues(const GMatP& vals) const;
+    // the plan of this pattern, built now if there is none
     bidmat_plan* plan(int k_hint);
+    // for A*S / DDS: the plan if there is one or if this is at least the second such call on the
+    // pattern (then it is built), otherwise nullptr (the caller runs without a plan)
+    bidmat_plan* planIfDue(int k_hint);
+    // private index arrays, about to be rewritten: nothing another matrix shares, no plan
+    void ownPattern();
+    // point at the pattern (and plan) of `like`
+    void sharePattern(const GSMat& like);
 
-    static GSMatP newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP oldmat);
+    static GSMatP newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP oldmat, const GSMat* like = nullptr);
     static GSMatP newOrCheckGSMat(int nr, int nc, int nnz, int realnnz, GSMatP outmat, long long g1,
-                                  long long g2, long long g3, long long opHash);
+                                  long long g2, long long g3, long long opHash, const GSMat* like = nullptr);
 };
 
 // ---- operators (GMat.scala:1684-1688, 1972-1976) and free functions

@@ -39,6 +39,11 @@ API int bmh_same_object(void* a, void* b) {
     return (H(a)->g && H(a)->g == H(b)->g) || (H(a)->s && H(a)->s == H(b)->s);
 }
 
+// 1 when two sparse matrices point at the same device index arrays
+API int bmh_same_pattern(void* a, void* b) { return S(a)->pir == S(b)->pir && S(a)->pjc == S(b)->pjc && S(a)->pic == S(b)->pic; }
+// 1 when the matrix's pattern has a plan by now
+API int bmh_has_plan(void* s) { return S(s)->planHolder && S(s)->planHolder->plan != nullptr; }
+
 API void* bmh_gmat_from_host(int nr, int nc, const float* data) {
     return guard_ptr([&] { return wrap(GMat::fromFMat(FMat(nr, nc, data))); });
 }

@@ -66,6 +66,8 @@ def _load():
         L.bmh_guid.restype = C.c_longlong
         L.bmh_guid.argtypes = [vp]
         L.bmh_same_object.argtypes = [vp, vp]
+        L.bmh_same_pattern.argtypes = [vp, vp]
+        L.bmh_has_plan.argtypes = [vp]
         L.bmh_gmat_dims.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.bmh_gmat_to_host.argtypes = [vp, vp]
         L.bmh_gsmat_dims.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]
@@ -239,6 +241,13 @@ class GSMat(_Handle):
         if _load().bmh_gsmat_to_host(self._h, data.ctypes.data, ir.ctypes.data, jc.ctypes.data) != 0:
             raise RuntimeError(_load().bmh_last_error().decode())
         return data, ir, jc
+
+    def same_pattern(self, other):
+        """True when both matrices point at the same device index arrays."""
+        return bool(_load().bmh_same_pattern(self._h, other._h))
+
+    def has_plan(self):
+        return bool(_load().bmh_has_plan(self._h))
 
     def device_jc(self):
         nr, nc, nnz = self.dims
