@@ -12,12 +12,13 @@ object of the DDS kernel (with a bound that cannot exceed 1: compulsory bytes at
 the same kernel's rate on an L2-resident operand, measured live), the CPU baseline and the check of
 every timed output against the CPU oracle ride along.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload headline|C1|C4|C5]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|headline|C1|C4|C5]
                   [--scale S] [--no-cpu] [--calibrate]
 
 The other workloads (C1: A*S k=32; C4: A*S k=1024 with Pareto columns; C5: the NMF update
-chain at k=128, ~400 M nonzeros) are the remaining BASELINE.json configurations; they are
-parity-test cases and are timed only on request. "next" times the callers either side of the
+chain at k=128, ~400 M nonzeros) are the remaining BASELINE.json configurations; the default run
+times each over a few steps, checks it against the oracle and reports it under `workloads`
+(`value` is always the headline's). "next" times the callers either side of the
 path on the headline pattern (tile products, S*A / S^T*A, sparse op edge vector, file load);
 "footprint" sweeps the gather kernels over the gathered footprint (where L1 / L2 / HBM serve).
 """
@@ -42,8 +43,8 @@ HBM_PEAK_GBS = 8000.0
 # was taken on; it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dds", 100003320): (25.45e9, "bidmat_amd/csrc/dds.hip", "f7e2c97e0cc1236f",
-                                     "profiles/headline_kernel_trace_and_hbm_counters.txt"),
+    ("headline", "dsmultT", 100003320): (31.6e9, "bidmat_amd/csrc/spmm.hip", "4df7d618119c5dec",
+                                         "profiles/headline_kernel_trace_and_hbm_counters.txt"),
     ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "4df7d618119c5dec",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
@@ -97,20 +98,55 @@ def flops(op, k, nnz, ncols):
     return float(k) * ncols
 
 
+def uncacheable_gather_bytes(ir, nrows, k, cache_bytes=32 << 20):
+    """Bytes of row gathers that even an ideal cache of `cache_bytes` (all eight 4 MiB L2s holding disjoint rows,
+    always the most frequent ones) would have to fetch from beyond L2: every gather of a row outside the
+    cache_bytes / 4k most frequent rows. A kernel that walks S column by column cannot order these
+    gathers away, so they bound its time at the rate of the memory side."""
+    cnt = np.bincount(ir, minlength=nrows)
+    keep = min(nrows, max(1, cache_bytes // (4 * k)))
+    if keep >= nrows:
+        return 0
+    top = np.partition(cnt, nrows - keep)[nrows - keep:].sum()
+    return int(cnt.sum() - top) * 4 * k
+
+
+def op_bounds(kind, k, nnz, nrows, ncols, l2_rate_GBps, uncacheable, heavy_nnz=None):
+    """Lower bounds on the time of one op in ms. compulsory: every array once at the HBM peak; l2_resident:
+    all gathered bytes at the rate the same kernel reaches when every gather hits L2; uncacheable: the gathers
+    an ideal 32 MiB L2 cannot hold, at the HBM peak. A*^S walks the plan's order, which an ideal-cache model of
+    S's rows does not describe: its third term is the bound of that schedule, heavy-row gathers (reused inside
+    a column panel) at the L2-resident rate plus light-row gathers (each dense column once per nonzero, no
+    reuse) at the HBM peak."""
+    terms = {"compulsory_ms": compulsory_bytes(kind, k, nnz, nrows, ncols) / (HBM_PEAK_GBS * 1e6)}
+    gathered = nnz * 4.0 * k
+    if l2_rate_GBps:
+        terms["l2_resident_ms"] = gathered / (l2_rate_GBps * 1e6)
+    if kind == "dsmultT":
+        if heavy_nnz is not None and l2_rate_GBps:
+            terms["plan_schedule_ms"] = heavy_nnz * 4.0 * k / (l2_rate_GBps * 1e6) + (nnz - heavy_nnz) * 4.0 * k / (HBM_PEAK_GBS * 1e6)
+    elif uncacheable is not None:
+        terms["uncacheable_ms"] = uncacheable / (HBM_PEAK_GBS * 1e6)
+    return terms
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="headline", choices=["headline", "C1", "C4", "C5", "next", "footprint"])
+    ap.add_argument("--workload", default="all", choices=["all", "headline", "C1", "C4", "C5", "next", "footprint"],
+                    help="all (default): the headline workload as the timed `value`, plus short runs of C1, C4 and C5 "
+                         "reported under `workloads`; any other name: that workload alone")
     ap.add_argument("--footprint-k", type=int, default=256, help="k of the footprint sweep")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows/columns of the pattern (testing)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs (baseline timing and verification)")
     ap.add_argument("--cpu-sample", type=float, default=1.0,
                     help="fraction of the columns timed on the CPU (1.0 = the whole workload)")
-    ap.add_argument("--sections", default="probe,shaped,graph,stored",
+    ap.add_argument("--sections", default="probe,shaped,operator,graph,stored",
                     help="side measurements around the timed steps, comma-separated: probe (L2-resident and streaming "
-                         "rates for the bounded roofline), shaped (reference-shaped entries), graph (HIP-graph replay), "
+                         "rates for the bounded roofline), shaped (reference-shaped entries, repeated and fresh patterns), "
+                         "operator (the GMat / GSMat operator layer), graph (HIP-graph replay), "
                          "stored (values stored in the plan); 'none' runs the timed steps only, which keeps a profiler's "
                          "per-kernel averages clean")
     ap.add_argument("--calibrate", action="store_true",
@@ -122,8 +158,7 @@ def main():
               "columns of S; a multi-GPU figure is not part of this build)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
-    from bidmat_amd import gen, hip_abi
-    from bidmat_amd.device import DeviceArray
+    from bidmat_amd import hip_abi
 
     lib = hip_abi.load()     # raises if the HIP library is not built: there is no fallback
     ndev = C.c_int(0)
@@ -131,10 +166,6 @@ def main():
     if ndev.value < 1:
         raise RuntimeError("no HIP device visible")
     hip_abi.check(lib.bidmat_set_device(0))
-    arch = C.create_string_buffer(64)
-    cus = C.c_int(0)
-    mem = C.c_longlong(0)
-    hip_abi.check(lib.bidmat_device_info(arch, 64, C.byref(cus), C.byref(mem)))
 
     sections = set() if args.sections == "none" else set(args.sections.split(","))
     if args.workload == "footprint":
@@ -142,8 +173,39 @@ def main():
     if args.workload == "next":
         return next_rows(lib, args)
 
+    main_name = "headline" if args.workload == "all" else args.workload
+    out = run_workload(lib, main_name, args.steps, args.warmup, args.scale, sections, not args.no_cpu, args.cpu_sample,
+                       args.calibrate)
+    if args.workload == "all":
+        # the other configurations of the path, each timed over a few steps and checked against the oracle;
+        # their CPU baselines run on labelled column samples so that the whole run stays within minutes
+        out["workloads"] = {}
+        for name, steps, sample in (("C1", 200, 1.0), ("C4", 10, 0.02), ("C5", 5, 0.005)):
+            w = run_workload(lib, name, steps, 2, args.scale, {"probe"} & sections, not args.no_cpu, sample, False)
+            out["workloads"][name] = {key: w[key] for key in ("metric", "value", "unit", "ms_per_step", "steps", "config", "ops", "roofline",
+                                                              "alg_frac_of_hbm_peak", "plan", "cpu_baseline", "verified", "rowsum")
+                                      if key in w}
+            hip_abi.check(lib.bidmat_release_caches())
+        out["verified"] = bool(out.get("verified")) and all(w.get("verified") for w in out["workloads"].values()) \
+            if not args.no_cpu else None
+    print(json.dumps(out))
+    if not args.no_cpu and not out["verified"]:
+        print("bench.py: the timed outputs differ from the CPU oracle beyond 1e-4", file=sys.stderr)
+        sys.exit(1)
+
+
+def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, calibrate):
+    """Times `steps` steps of one workload with inputs resident in HBM and returns its record."""
+    from bidmat_amd import gen, hip_abi
+    from bidmat_amd.device import DeviceArray
+
+    arch = C.create_string_buffer(64)
+    cus = C.c_int(0)
+    mem = C.c_longlong(0)
+    hip_abi.check(lib.bidmat_device_info(arch, 64, C.byref(cus), C.byref(mem)))
+
     t0 = time.time()
-    cfg = gen.config("HEAD" if args.workload == "headline" else args.workload, args.scale)
+    cfg = gen.config("HEAD" if name == "headline" else name, scale)
     k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
     ir, jc = cfg["ir"], cfg["jc"]
     nnz = int(ir.size)
@@ -178,34 +240,44 @@ def main():
             hip_abi.check(lib.bidmat_synchronize())
             t_plan[i] = time.time() - t
 
+    def ev():
+        e = C.c_void_p()
+        hip_abi.check(lib.bidmat_event_create(C.byref(e)))
+        return e
+
     # ---- the ops of one step: (name, kind, launcher). Every workload goes through a plan: the plan
     # holds what depends on the pattern alone, so no call builds or allocates anything.
     build_plan()
     outputs = {}
-    if args.workload == "headline":
+    stage_marks = None       # one event per step, recorded between the two stages of A*^S
+    if name == "headline":
         d_A, d_B, d_AT = (up(cfg[x]) for x in ("A", "B", "A_T"))
         d_P, d_C, d_G = DeviceArray(nnz, np.float32), DeviceArray(k * ncols, np.float32), DeviceArray(k * nrows, np.float32)
         keep += [d_A, d_B, d_AT, d_P, d_C, d_G]
         outputs = {"dds": d_P, "dsmult": d_C, "dsmultT": d_G}
+        stage_marks = [ev() for _ in range(steps)]
+        cur = {"step": 0}
         ops = [
             ("dds", "dds", lambda: lib.bidmat_dds_plan(plan, k, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, None, 0, d_P.ptr, 0, stream)),
             ("dsmult", "dsmult", lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream)),
-            ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_AT.ptr, d_v.ptr, d_G.ptr, 0, stream)),
+            ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan_staged(plan, k, d_AT.ptr, d_v.ptr, d_G.ptr, 0, stream,
+                                                                          stage_marks[cur["step"] % steps])),
         ]
         workload = "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), step = DDS, A*S, A*^S"
         metric = "algorithmic GB/s (gathered operand charged once per nonzero) and nnz/s for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
-        roof_op, roof_kernel = "dds", "k_dds_classed_nolds_k256 = the class-ordered DDS kernel at W=4,V=1,LPN=64 without LDS rows (one launch = DDS over the whole pattern)"
-    elif args.workload in ("C1", "C4"):
+        roof_op = "dsmultT"
+        roof_kernel = "k_gather_axpy<4,1,64,true> = stage 1 of A*^S, the time-dominant kernel of the step (one launch = the gathers of the whole pattern in plan order)"
+    elif name in ("C1", "C4"):
         d_A = up(cfg["A"])
         d_C = DeviceArray(k * ncols, np.float32)
         keep += [d_A, d_C]
         outputs = {"dsmult": d_C}
         ops = [("dsmult", "dsmult", lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, d_v.ptr, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream))]
-        workload = "configs[0]: A*S, k=32, 50 nnz per column" if args.workload == "C1" else \
+        workload = "configs[0]: A*S, k=32, 50 nnz per column" if name == "C1" else \
             "configs[3]: A*S, k=1024, Pareto(1.5) column lengths in [1,50000]"
-        metric = "algorithmic GB/s (gathered operand charged once per nonzero) for A*S (%s)" % args.workload
+        metric = "algorithmic GB/s (gathered operand charged once per nonzero) for A*S (%s)" % name
         roof_op = "dsmult"
-        roof_kernel = "k_gather_axpy<W=4,V=1,LPN=8>" if args.workload == "C1" else "k_gather_axpy<W=4,V=4,LPN=64>"
+        roof_kernel = "k_gather_axpy<W=4,V=1,LPN=8>" if name == "C1" else "k_gather_axpy<W=4,V=4,LPN=64>"
     else:  # C5: Q = V ./ DDS(W,H,V) in one launch; G = H *^ Q; rs = sum(H,2)
         d_W, d_H = up(cfg["W"]), up(cfg["H"])
         d_Q, d_G, d_rs = DeviceArray(nnz, np.float32), DeviceArray(k * nrows, np.float32), DeviceArray(k, np.float32)
@@ -220,22 +292,17 @@ def main():
         ]
         workload = "configs[4]: NMF update chain Q = V ./ DDS(W,H,V) (one fused launch), G = H *^ Q (dense row sums timed apart)"
         metric = "algorithmic GB/s (gathered operand charged once per nonzero) for the NMF update chain at k=128, ~400M nnz"
-        roof_op, roof_kernel = "dsmultT", "k_gather_axpy<W=4,V=1,LPN=32,plan> (stage 1 of A*^S)"
-
-    def ev():
-        e = C.c_void_p()
-        hip_abi.check(lib.bidmat_event_create(C.byref(e)))
-        return e
+        roof_op, roof_kernel = "dsmultT", "k_gather_axpy<W=4,V=1,LPN=32,plan> + k_reduce_segments (both stages of A*^S)"
 
     def step(marks=None):
-        for i, (name, _, fn) in enumerate(ops):
+        for i, (opname, _, fn) in enumerate(ops):
             if marks:
                 hip_abi.check(lib.bidmat_event_record(marks[i], stream))
-            hip_abi.check(fn(), name)
+            hip_abi.check(fn(), opname)
         if marks:
             hip_abi.check(lib.bidmat_event_record(marks[len(ops)], stream))
 
-    if args.calibrate:
+    if calibrate:
         ncal = 1 << 28                                   # 2^28 floats = 1 GiB per array
         cal = [DeviceArray(ncal, np.float32) for _ in range(3)]
         for c in cal:
@@ -246,19 +313,21 @@ def main():
         for c in cal:
             c.free()
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     hip_abi.check(lib.bidmat_stream_synchronize(stream))
 
-    marks = [[ev() for _ in range(len(ops) + 1)] for _ in range(args.steps)]
+    marks = [[ev() for _ in range(len(ops) + 1)] for _ in range(steps)]
     hip_abi.check(lib.bidmat_synchronize())
     t0 = time.perf_counter()
-    for s in range(args.steps):
+    for s in range(steps):
+        if stage_marks:
+            cur["step"] = s
         step(marks[s])
     hip_abi.check(lib.bidmat_stream_synchronize(stream))
     hip_abi.check(lib.bidmat_synchronize())
     wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
+    ms_per_step = wall * 1e3 / steps
 
     def elapsed(a, b):
         ms = C.c_float(0)
@@ -266,32 +335,53 @@ def main():
         return float(ms.value)
 
     per_op, total_bytes, total_flops = {}, 0, 0.0
-    for i, (name, kind, _) in enumerate(ops):
+    for i, (opname, kind, _) in enumerate(ops):
         t = [elapsed(m[i], m[i + 1]) for m in marks]
         b = alg_bytes(kind, k, nnz, nrows, ncols)
         total_bytes += b
         total_flops += flops(kind, k, nnz, ncols)
         avg = float(np.mean(t))
-        per_op[name] = {
+        per_op[opname] = {
             "ms_avg": round(avg, 4), "ms_median": round(float(np.median(t)), 4), "ms_min": round(float(np.min(t)), 4),
             "alg_GB": round(b / 1e9, 3), "compulsory_GB": round(compulsory_bytes(kind, k, nnz, nrows, ncols) / 1e9, 3),
             "alg_GBps": round(b / avg / 1e6, 1), "nnz_per_s": round(nnz / avg * 1e3, 1),
             "GFLOPs": round(flops(kind, k, nnz, ncols) / avg / 1e6, 1),
             "alg_frac_of_hbm_peak": round(b / avg / 1e6 / HBM_PEAK_GBS, 4),
         }
+    if stage_marks:
+        t1 = [elapsed(marks[s][2], stage_marks[s]) for s in range(steps)]
+        t2 = [elapsed(stage_marks[s], marks[s][3]) for s in range(steps)]
+        per_op["dsmultT"]["stage1_gather_ms_avg"] = round(float(np.mean(t1)), 4)
+        per_op["dsmultT"]["stage2_reduce_ms_avg"] = round(float(np.mean(t2)), 4)
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- what bounds the roofline kernel, measured on this device in this run: the rate of the
-    # same gather kernel when the gathered rows fit in L2 (the ceiling of a kernel whose every gather
-    # is served by L2), and the plain streaming rate of the device.
-    live = live_rates(lib, stream, k, "dds" if roof_op in ("dds", "dds_op") else "dsmult") if "probe" in sections else \
-        {"l2_resident_gather_GBps": None, "stream_GBps": None, "probe": None}
-    r_avg, r_bytes = per_op[roof_op]["ms_avg"], alg_bytes(roof_op, k, nnz, nrows, ncols)
-    r_comp = compulsory_bytes(roof_op, k, nnz, nrows, ncols)
-    gathered = nnz * 4 * k
-    bound_ms = max(r_comp / (HBM_PEAK_GBS * 1e9), gathered / (live["l2_resident_gather_GBps"] * 1e9)) * 1e3 \
-        if live["l2_resident_gather_GBps"] else None
-    traffic, traffic_src = measured_traffic(args.workload, roof_op, nnz)
+    # ---- what bounds every op, measured on this device in this run: the rate of the same gather kernels
+    # when the gathered rows fit in L2 (the ceiling of a kernel whose every gather is served by L2), the
+    # plain streaming rate of the device, and from the pattern itself the gathers no L2 could hold.
+    heavy_nnz = lib.bidmat_plan_heavy_nnz(plan) if "dsmultT" in per_op else None
+    uncache = uncacheable_gather_bytes(ir, nrows, k) if "probe" in sections else None
+    live = {}
+    if "probe" in sections:
+        for kind in sorted({("dds" if o[1] in ("dds", "dds_op") else "dsmult") for o in ops}):
+            live[kind] = live_rates(lib, stream, k, kind)
+    for opname, kind, _ in ops:
+        lr = live.get("dds" if kind in ("dds", "dds_op") else "dsmult")
+        terms = op_bounds(kind, k, nnz, nrows, ncols, lr["l2_resident_gather_GBps"] if lr else None, uncache, heavy_nnz)
+        bound = max(v for key, v in terms.items() if key != "plan_schedule_ms")
+        per_op[opname]["bound_terms_ms"] = {key: round(v, 4) for key, v in terms.items()}
+        per_op[opname]["bound_ms"] = round(bound, 4)
+        per_op[opname]["frac_of_bound"] = round(bound / per_op[opname]["ms_avg"], 4)
+        if "plan_schedule_ms" in terms:
+            per_op[opname]["frac_of_plan_schedule_bound"] = round(terms["plan_schedule_ms"] / per_op[opname]["ms_avg"], 4)
+    r = per_op[roof_op]
+    # the dominant kernel's own launch time where the step marks it (stage 1 of A*^S), else its op's time
+    r_avg = r.get("stage1_gather_ms_avg", r["ms_avg"])
+    r_bytes = alg_bytes(roof_op, k, nnz, nrows, ncols)
+    if "stage1_gather_ms_avg" in r:
+        # stage 1 alone: per nonzero one gathered column, its index and its value; per segment one partial sum written
+        r_bytes = nnz * (4 * k + 8) + lib.bidmat_plan_segments(plan) * (4 * k + 4) + 4
+    lr = live.get("dds" if roof_op in ("dds", "dds_op") else "dsmult")
+    traffic, traffic_src = measured_traffic(name, roof_op, nnz)
     roofline = {
         "kernel": roof_kernel, "bound": "hbm", "achieved": round(r_bytes / r_avg / 1e6, 1), "peak": HBM_PEAK_GBS,
         "unit": "GB/s", "frac": round(r_bytes / r_avg / 1e6 / HBM_PEAK_GBS, 4),
@@ -299,25 +389,33 @@ def main():
                       "most of them, so this can exceed 1; the bounded utilisation figure is frac_of_bound",
         "traffic": traffic, "traffic_source": traffic_src,
         "bytes_per_launch": r_bytes, "avg_launch_ms": round(r_avg, 4),
-        "compulsory_bytes": r_comp, "gathered_bytes": gathered,
-        "l2_resident_gather_GBps": live["l2_resident_gather_GBps"], "l2_resident_probe": live["probe"],
-        "stream_GBps": live["stream_GBps"],
-        "bound_ms": round(bound_ms, 4) if bound_ms else None, "frac_of_bound": round(bound_ms / r_avg, 4) if bound_ms else None,
-        "bound_basis": "max(compulsory bytes / 8 TB/s, gathered bytes / rate of the same kernel with an L2-resident operand)",
+        "compulsory_bytes": compulsory_bytes(roof_op, k, nnz, nrows, ncols), "gathered_bytes": nnz * 4 * k,
+        "uncacheable_gather_bytes": uncache if roof_op != "dsmultT" else None,
+        "heavy_row_nnz": heavy_nnz if roof_op == "dsmultT" else None,
+        "l2_resident_gather_GBps": lr["l2_resident_gather_GBps"] if lr else None, "l2_resident_probe": lr["probe"] if lr else None,
+        "stream_GBps": lr["stream_GBps"] if lr else None,
+        "bound_ms": r.get("bound_ms"), "frac_of_bound": round(r["bound_ms"] / r_avg, 4) if r.get("bound_ms") else None,
+        "frac_of_plan_schedule_bound": round(r["bound_terms_ms"]["plan_schedule_ms"] / r_avg, 4)
+        if r.get("bound_terms_ms", {}).get("plan_schedule_ms") else None,
+        "bound_basis": "max(compulsory bytes / 8 TB/s, gathered bytes / rate of the same kernel with an L2-resident operand, "
+                       "gathers that an ideal 32 MiB L2 cannot hold / 8 TB/s); plan_schedule: heavy-row gathers at the L2-resident "
+                       "rate + light-row gathers at 8 TB/s",
     }
     if traffic:
         # L2-miss (fabric-side) bytes over time: Infinity Cache and HBM together, not an HBM fraction
         roofline["l2_miss_GBps"] = round(traffic / r_avg / 1e6, 1)
 
     out = {
-        "metric": metric, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "metric": metric, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": workload, "k": k, "nrows": nrows, "ncols": ncols, "nnz": nnz, "scale": args.scale},
+        "config": {"workload": workload, "k": k, "nrows": nrows, "ncols": ncols, "nnz": nnz, "scale": scale},
         "nnz_per_s": round(len([o for o in ops if o[1] != "ewise"]) * nnz / (ms_per_step * 1e-3), 1),
         "GFLOPs": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),
         "alg_frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "ops": per_op, "roofline": roofline,
+        "api_form": "every op of the timed step goes through a plan handle (bidmat_*_plan); what callers without a handle get "
+                    "is under reference_shaped_ms_incl_clear and operator_api_ms",
         "device": {"arch": arch.value.decode(), "compute_units": cus.value, "mem_GiB": round(mem.value / 2**30, 1)},
         "gen_s": round(t_gen, 2),
         # informational: what one step would cost if every input crossed PCIe first (never `value`)
@@ -331,7 +429,7 @@ def main():
     if "dsmultT" in per_op:
         # what a caller with a fresh pattern on every call (a BIDMach minibatch) pays for A*^S
         per_op["dsmultT_incl_plan_ms"] = round(per_op["dsmultT"]["ms_avg"] + t_plan[1] * 1e3, 4)
-    if args.workload == "C5":      # the dense row sums of H, timed apart from the chain
+    if name == "C5":      # the dense row sums of H, timed apart from the chain
         e0, e1 = ev(), ev()
         hip_abi.check(lib.bidmat_reduce2op(k, ncols, d_H.ptr, d_rs.ptr, 0.0, 0))
         hip_abi.check(lib.bidmat_event_record(e0, None))
@@ -345,32 +443,15 @@ def main():
                          "frac_of_hbm_peak": round(b / t / 1e6 / HBM_PEAK_GBS, 4)}
 
     # the outputs of the timed steps, checked below
-    results = {name: d.numpy() for name, d in outputs.items()} if not args.no_cpu else {}
+    results = {opname: d.numpy() for opname, d in outputs.items()} if cpu else {}
 
-    if args.workload == "headline" and "shaped" in sections:
-        # What unchanged call sites get: the blocking entries with the reference's argument lists
-        # (per-nonzero column array, no column pointer, no plan handle), each preceded by the clear
-        # of its output that GSMult / GSMultT / DDS do; wall clock around clear + call.
-        d_ic = DeviceArray(nnz, np.int32)
-        hip_abi.check(lib.bidmat_csc_expand_cols(ncols, nnz, d_jc.ptr, d_ic.ptr, None))
-        hip_abi.check(lib.bidmat_synchronize())
-        keep.append(d_ic)
-        shaped = {}
-        for name, outbuf, call in (
-                ("dds", d_P, lambda: lib.bidmat_dds(k, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_ic.ptr, d_P.ptr)),
-                ("dsmult", d_C, lambda: lib.bidmat_dsmult(k, ncols, nnz, d_A.ptr, d_v.ptr, d_ir.ptr, d_ic.ptr, d_C.ptr)),
-                ("dsmultT", d_G, lambda: lib.bidmat_dsmultT(k, ncols, nnz, d_AT.ptr, d_v.ptr, d_ir.ptr, d_ic.ptr, d_G.ptr))):
-            ts = []
-            for r in range(4):
-                hip_abi.check(lib.bidmat_synchronize())
-                t0 = time.perf_counter()
-                hip_abi.check(lib.bidmat_memset(outbuf.ptr, 0, outbuf.nbytes))
-                hip_abi.check(call(), name)
-                ts.append((time.perf_counter() - t0) * 1e3)
-            shaped[name] = round(float(np.median(ts[1:])), 3)
-        out["reference_shaped_ms_incl_clear"] = shaped
+    if name == "headline" and "shaped" in sections:
+        out["reference_shaped_ms_incl_clear"] = shaped_entries(lib, k, nrows, ncols, nnz, d_ir, d_jc, d_v, d_A, d_B, d_AT,
+                                                               d_P, d_C, d_G)
+    if name == "headline" and "operator" in sections:
+        out["operator_api_ms"] = operator_layer(cfg)
 
-    if args.workload == "headline" and "stored" in sections:
+    if name == "headline" and "stored" in sections:
         # Callers whose values stay fixed over several calls (the data matrix of an LDA minibatch) can
         # store them in the plan, in plan order: A*^S, A*S and the sparse row sums then stream them.
         d_rs = DeviceArray(nrows, np.float32)
@@ -383,13 +464,15 @@ def main():
             sv["dsmult_ms"] = round(_timed(lib, lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, None, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream), stream, 5), 4)
         out["values_stored_in_plan"] = sv
 
-    if args.workload in ("C1", "headline") and "graph" in sections:
+    if name in ("C1", "headline") and "graph" in sections:
         # the same step recorded once into a HIP graph and replayed with one launch per step
+        if stage_marks:
+            ops[2] = ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_AT.ptr, d_v.ptr, d_G.ptr, 0, stream))
         gx = C.c_void_p()
         hip_abi.check(lib.bidmat_graph_begin_capture(stream))
         step()
         hip_abi.check(lib.bidmat_graph_end_capture(stream, C.byref(gx)))
-        reps = 200 if args.workload == "C1" else args.steps
+        reps = 200 if name == "C1" else steps
         for _ in range(3):
             hip_abi.check(lib.bidmat_graph_launch(gx, stream))
         e0, e1 = ev(), ev()
@@ -401,17 +484,98 @@ def main():
         out["graph_replay"] = {"ms_per_step": round(elapsed(e0, e1) / reps, 4), "steps": reps}
         hip_abi.check(lib.bidmat_graph_destroy(gx))
 
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_sample)
-        checks = verify_outputs(args.workload, cfg, results)
-        for name, c in checks.items():
-            per_op[name].update(c)
-        out["verified"] = bool(checks) and all(c["max_err_measure"] <= 1e-4 for c in checks.values())
+    # device memory back before the CPU legs (and the next workload)
+    hip_abi.check(lib.bidmat_synchronize())
+    hip_abi.check(lib.bidmat_plan_destroy(plan))
+    for d in keep:
+        d.free()
+    hip_abi.check(lib.bidmat_stream_destroy(stream))
 
-    print(json.dumps(out))
-    if not args.no_cpu and not out["verified"]:
-        print("bench.py: the timed outputs differ from the CPU oracle beyond 1e-4", file=sys.stderr)
-        sys.exit(1)
+    if cpu:
+        out["cpu_baseline"] = cpu_baseline(name, cfg, cpu_sample)
+        checks = verify_outputs(name, cfg, results)
+        for opname, c in checks.items():
+            per_op[opname].update(c)
+        out["verified"] = bool(checks) and all(c["max_err_measure"] <= 1e-4 for c in checks.values())
+    return out
+
+
+def shaped_entries(lib, k, nrows, ncols, nnz, d_ir, d_jc, d_v, d_A, d_B, d_AT, d_P, d_C, d_G):
+    """What unchanged call sites get: the blocking entries with the reference's argument lists (per-nonzero
+    column array, no column pointer, no plan handle), each preceded by the clear of its output that
+    GSMult / GSMultT / DDS do; wall clock around clear + call. `repeated`: the same device arrays call after
+    call (from the second call on the entries find the pattern's cached plan). `fresh`: a pattern the
+    library has not seen, in new device arrays, on every call (a new minibatch): DDS and A*S run the plain
+    kernels, A*^S builds its row plan inside the call."""
+    from bidmat_amd import hip_abi
+    from bidmat_amd.device import DeviceArray
+    d_ic = DeviceArray(nnz, np.int32)
+    hip_abi.check(lib.bidmat_csc_expand_cols(ncols, nnz, d_jc.ptr, d_ic.ptr, None))
+    hip_abi.check(lib.bidmat_synchronize())
+
+    def calls(ir_ptr, ic_ptr):
+        return (("dds", d_P, lambda: lib.bidmat_dds(k, nnz, d_A.ptr, d_B.ptr, ir_ptr, ic_ptr, d_P.ptr)),
+                ("dsmult", d_C, lambda: lib.bidmat_dsmult(k, ncols, nnz, d_A.ptr, d_v.ptr, ir_ptr, ic_ptr, d_C.ptr)),
+                ("dsmultT", d_G, lambda: lib.bidmat_dsmultT(k, ncols, nnz, d_AT.ptr, d_v.ptr, ir_ptr, ic_ptr, d_G.ptr)))
+
+    def timed(outbuf, call, what):
+        hip_abi.check(lib.bidmat_synchronize())
+        t0 = time.perf_counter()
+        hip_abi.check(lib.bidmat_memset(outbuf.ptr, 0, outbuf.nbytes))
+        hip_abi.check(call(), what)
+        return (time.perf_counter() - t0) * 1e3
+
+    hip_abi.check(lib.bidmat_release_caches())
+    repeated, first = {}, {}
+    for opname, outbuf, call in calls(d_ir.ptr, d_ic.ptr):
+        ts = [timed(outbuf, call, opname) for _ in range(7)]
+        first[opname] = [round(t, 3) for t in ts[:3]]      # 1st: plain kernel / plan build; 2nd: column side built
+        repeated[opname] = round(float(np.median(ts[3:])), 3)
+    fresh = {}
+    for opname in ("dds", "dsmult", "dsmultT"):
+        ts = []
+        for r in range(4):
+            # a copy of the pattern in device arrays of its own: new addresses, so nothing cached applies
+            f_ir, f_ic = DeviceArray(nnz, np.int32), DeviceArray(nnz, np.int32)
+            hip_abi.check(lib.bidmat_memcpy_d2d(f_ir.ptr, d_ir.ptr, 4 * nnz))
+            hip_abi.check(lib.bidmat_memcpy_d2d(f_ic.ptr, d_ic.ptr, 4 * nnz))
+            _, outbuf, call = [c for c in calls(f_ir.ptr, f_ic.ptr) if c[0] == opname][0]
+            ts.append(timed(outbuf, call, opname))
+            f_ir.free(); f_ic.free()
+        fresh[opname] = round(float(np.median(ts[1:])), 3)
+    hip_abi.check(lib.bidmat_release_caches())
+    d_ic.free()
+    return {"repeated_pattern": repeated, "fresh_pattern": fresh, "first_three_calls": first}
+
+
+def operator_layer(cfg):
+    """The same three products through the GMat / GSMat operator layer (libbidmathost, the stand-in for the
+    Scala classes): wall clock around each blocking operator call with the output matrix reused, median of
+    five calls after the two that build the pattern's plan."""
+    from bidmat_amd import mats
+    k, nrows, ncols = cfg["k"], cfg["nrows"], cfg["ncols"]
+    mats.Mat.set("ioneBased", 0)
+    try:
+        S = mats.GSMat.from_csc(nrows, ncols, cfg["vals"], cfg["ir"], cfg["jc"])
+        gA = mats.GMat.from_numpy(cfg["A"].reshape(nrows, k).T)
+        gB = mats.GMat.from_numpy(cfg["B"].reshape(ncols, k).T)
+        gAT = mats.GMat.from_numpy(cfg["A_T"].reshape(ncols, k).T)
+        res = {}
+        for opname, first, again in (
+                ("DDS", lambda: mats.DDS(gA, gB, S), lambda o: mats.DDS(gA, gB, S, o)),
+                ("GSMult (A*S)", lambda: gA.GSMult(S), lambda o: gA.GSMult(S, o)),
+                ("GSMultT (A*^S)", lambda: gAT.GSMultT(S), lambda o: gAT.GSMultT(S, o))):
+            o = first()
+            ts = []
+            for _ in range(7):
+                t0 = time.perf_counter()
+                again(o)
+                ts.append((time.perf_counter() - t0) * 1e3)
+            res[opname] = round(float(np.median(ts[2:])), 3)
+            del o
+        return res
+    finally:
+        mats.Mat.set("ioneBased", 1)
 
 
 def live_rates(lib, stream, k, op):

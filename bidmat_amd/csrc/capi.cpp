@@ -89,22 +89,24 @@ enum Need { NEED_ROWS, NEED_COLS };
 // built when that side is due; *out stays empty when A*S / DDS should run without a plan. *jc_out
 // (nullable) receives the pattern's column pointer, built in the same pass over ic into the default
 // stream's scratch: valid until the caller's next scratch request for WS_JC.
+// zcheck != nullptr: *all_zero tells whether the nz floats there are all +0.0f (checked in the same pass).
 hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_hint, Need need, PlanRef* out,
-                       int** jc_out = nullptr) {
+                       int** jc_out = nullptr, const float* zcheck = nullptr, long long nz = 0, bool* all_zero = nullptr) {
     out->reset();
     hipError_t err;
     int dev = 0;
     if ((err = hipGetDevice(&dev)) != hipSuccess) return err;
     hipStream_t s = nullptr;
-    unsigned long long* d_misc = (unsigned long long*)bm::ws_get(bm::WS_MISC, 64, &err);
+    unsigned long long* d_misc = (unsigned long long*)bm::ws_get(bm::WS_MISC, sizeof(unsigned long long) * bm::pattern_digest_words(), &err);
     if (!d_misc) return err;
     int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
     if (!jc) return err;
     if (jc_out) *jc_out = jc;
-    // misc layout: [0..1] digests of ir and ic, [2] (as int) max row
-    if ((err = bm::pattern_digest(ir, ic, nnz, d_misc, s, ncols, jc)) != hipSuccess) return err;
-    unsigned long long h[3];
+    // misc layout: [0..1] two digests of the (ic, ir) pair sequence, [2] (as int) max row
+    if ((err = bm::pattern_digest(ir, ic, nnz, d_misc, s, ncols, jc, zcheck, nz)) != hipSuccess) return err;
+    unsigned long long h[4];
     if ((err = hipMemcpy(h, d_misc, sizeof(h), hipMemcpyDeviceToHost)) != hipSuccess) return err;
+    if (all_zero) *all_zero = zcheck != nullptr && h[3] == 0;
     int maxrow;
     memcpy(&maxrow, &h[2], sizeof(int));
     const int nrows = maxrow + 1;
@@ -157,14 +159,16 @@ float* row_partial(const bidmat_plan* plan, int k, hipStream_t s, hipError_t* er
 }
 
 // vals == nullptr: the values stored in the plan by bidmat_plan_set_values (already in plan order)
+// between != nullptr: an event recorded after stage 1 (the gathers), before stage 2 (the row reduction)
 hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* vals, float* C, int beta,
-                       hipStream_t s) {
+                       hipStream_t s, hipEvent_t between = nullptr) {
     hipError_t err;
     if (!vals && !plan->pvals && plan->nnz > 0) return hipErrorInvalidValue;
     float* partial = row_partial(plan, k, s, &err);
     if (!partial) return err;
     if ((err = bm::gather_segments(k, plan->nseg, plan->xcd_start, A, vals ? vals : plan->pvals, plan->pc,
                                    vals ? plan->perm : nullptr, plan->segstart, partial, s)) != hipSuccess) return err;
+    if (between && (err = hipEventRecord(between, s)) != hipSuccess) return err;
     return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, partial, C, beta, s);
 }
 
@@ -275,12 +279,15 @@ API int bidmat_dsmult(int nrows, int ncols, int nnz, const float* A, const float
     hipError_t err;
     if (bm::g_cache_cols_after.load() > 0) {
         // a pattern met before runs through the column side of its cached plan
+        // (callers clear C before they call, GMat.scala:1047: a C found all zero is overwritten, not read)
         PlanRef plan;
         int* jc = nullptr;
-        err = cached_plan(ncols, nnz, Bir, Bic, nrows, NEED_COLS, &plan, &jc);
+        bool zero = false;
+        err = cached_plan(ncols, nnz, Bir, Bic, nrows, NEED_COLS, &plan, &jc, C, (long long)nrows * ncols, &zero);
         if (err != hipSuccess) return finish_blocking(err);
-        if (plan) return finish_blocking((hipError_t)dsmult_through_plan(plan.get(), nrows, A, Bdata, Bir, jc, C, 1, nullptr));
-        return finish_blocking(bm::dsmult_csc(nrows, ncols, nnz, A, Bdata, Bir, jc, C, 1, nullptr));
+        const int beta = zero ? 0 : 1;
+        if (plan) return finish_blocking((hipError_t)dsmult_through_plan(plan.get(), nrows, A, Bdata, Bir, jc, C, beta, nullptr));
+        return finish_blocking(bm::dsmult_csc(nrows, ncols, nnz, A, Bdata, Bir, jc, C, beta, nullptr));
     }
     int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
     if (!jc) return (int)err;
@@ -378,12 +385,15 @@ API int bidmat_dds(int nrows, int nnz, const float* A, const float* B, const int
     const int ncols = last + 1;
     if (bm::g_cache_cols_after.load() > 0 && nrows > 0) {
         // a pattern met before runs through the column side of its cached plan
+        // (callers clear P before they call, GSMat.scala:662: a P found all zero is overwritten, not read)
         PlanRef plan;
         int* jc = nullptr;
-        err = cached_plan(ncols, nnz, Cir, Cic, nrows, NEED_COLS, &plan, &jc);
+        bool zero = false;
+        err = cached_plan(ncols, nnz, Cir, Cic, nrows, NEED_COLS, &plan, &jc, P, nnz, &zero);
         if (err != hipSuccess) return finish_blocking(err);
-        if (plan) return finish_blocking((hipError_t)dds_through_plan(plan.get(), nrows, A, B, Cir, jc, nullptr, false, 0, P, 1, nullptr));
-        return finish_blocking(bm::dds_csc(nrows, ncols, nnz, A, B, Cir, jc, P, 1, nullptr));
+        const int beta = zero ? 0 : 1;
+        if (plan) return finish_blocking((hipError_t)dds_through_plan(plan.get(), nrows, A, B, Cir, jc, nullptr, false, 0, P, beta, nullptr));
+        return finish_blocking(bm::dds_csc(nrows, ncols, nnz, A, B, Cir, jc, P, beta, nullptr));
     }
     int* jc = (int*)bm::ws_get(bm::WS_JC, sizeof(int) * ((size_t)ncols + 1), &err);
     if (!jc) return (int)err;
@@ -531,6 +541,26 @@ API int bidmat_dsmultT_plan(bidmat_plan* plan, int k, const float* A, const floa
     if (k == 0 || plan->nrows == 0) return 0;
     if (!C || (plan->nnz > 0 && (!A || (!Sdata && !plan->pvals)))) return kInvalid;
     return (int)run_dsmultT(plan, k, A, Sdata, C, beta, as_stream(stream));
+}
+
+API int bidmat_dsmultT_plan_staged(bidmat_plan* plan, int k, const float* A, const float* Sdata, float* C,
+                                   int beta, void* stream, void* event_between) {
+    auto lock = bm::device_lock();
+    if (!plan || k < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (!(plan->sides & bm::PLAN_ROWS)) return kInvalid;
+    if (k == 0 || plan->nrows == 0) return 0;
+    if (!C || (plan->nnz > 0 && (!A || (!Sdata && !plan->pvals)))) return kInvalid;
+    return (int)run_dsmultT(plan, k, A, Sdata, C, beta, as_stream(stream), (hipEvent_t)event_between);
+}
+
+API long long bidmat_plan_heavy_nnz(const bidmat_plan* plan) {
+    if (!plan || !(plan->sides & bm::PLAN_ROWS) || plan->nseg == 0 || !plan_on_current_device(plan)) return 0;
+    // heavy segments come first in plan order: the light ones start at segment xcd_start[8]
+    if (plan->xcd_start[8] >= plan->nseg) return plan->nnz;
+    int first_light = 0;
+    if (hipMemcpy(&first_light, plan->segstart + plan->xcd_start[8], sizeof(int), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+    return first_light;
 }
 
 API int bidmat_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float* Sdata, const int* Sir,

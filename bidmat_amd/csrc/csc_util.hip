@@ -66,65 +66,97 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fill(T* __restrict__ out, long lon
     for (; i < n; i += stride) out[i] = v;
 }
 
-// 64-bit finaliser (splitmix64): every input bit reaches every output bit.
-__device__ __forceinline__ unsigned long long mix64(unsigned long long x) {
-    x ^= x >> 30; x *= 0xBF58476D1CE4E5B9ULL;
-    x ^= x >> 27; x *= 0x94D049BB133111EBULL;
-    x ^= x >> 31;
-    return x;
-}
-// Contribution of (position i, value v) to a digest: a non-linear 64-bit hash of the pair, so that
-// neither moving a value to another position nor trading amounts between two positions cancels out.
-__device__ __forceinline__ unsigned long long digest_term(unsigned long long i, unsigned v, unsigned long long salt) {
-    return mix64(((i + 1ULL) << 32 | (unsigned long long)v) ^ salt);
-}
+constexpr int DIGEST_MAX_BLOCKS = 4096;
 
-// One pass over both index arrays of a pattern: digests sum_i hash64(i, value_i) of ir and of ic
-// (64-bit integer sums: position-sensitive, independent of the order in which threads contribute)
-// and the largest row index. A workgroup walks tiles of 4 x 256 positions with four
-// loads per array in flight per thread. out: [0] digest of ir, [1] digest of ic, [2] (int) max.
+// One pass over both index arrays of a pattern. With p_j = (j+1) * 0x9E3779B9 (32 bits), position j adds
+//   out[0] += fold32((ir[j] ^ p_j) * 0x85EBCA6B) << 32 | fold32(((ir[j] + 0x27D4EB2F * ic[j]) ^ ~p_j) * 0xC2B2AE35)
+//             with fold32(h) = h ^ (h >> 15): two different non-linear 32-bit hashes of (position, row, column)
+//             side by side (xor before the multiplication, fold after it), so that neither moving an entry to
+//             another position nor trading amounts between positions cancels out;
+//   out[1] += ic[j] << 32 | ir[j]       the plain sum of the pairs.
+// Both are 64-bit integer sums, independent of the order in which threads add.
+// out[2] (as int) = the largest entry of ir. Every thread takes four consecutive positions at a time
+// (one 128-bit load per array when both are 16-byte aligned; the position word advances by addition).
 // jc != nullptr: the column pointer of the pattern is written in the same pass (what k_compress_cols
 // does): position j closes the columns ic[j-1]+1 .. ic[j], the last position also those behind ic[n-1].
+// z != nullptr: the fourth word counts the workgroups that met a word of z[0..nz) other than +0.0f (callers
+// that accumulate into an output they have just cleared can then overwrite it instead of reading it).
+// Workgroup b leaves its four words at out[4*(b+1) ..]; k_digest_final combines them into out[0..3].
+template <bool VEC>
 __global__ __launch_bounds__(BM_BLOCK) void k_pattern_digest(const int* __restrict__ ir, const int* __restrict__ ic,
                                                              long long n, unsigned long long* out, int ncols,
-                                                             int* __restrict__ jc) {
-    constexpr int UN = 4;
-    long long i = (long long)blockIdx.x * (UN * BM_BLOCK) + threadIdx.x;
-    const long long stride = (long long)gridDim.x * (UN * BM_BLOCK);
+                                                             int* __restrict__ jc, const unsigned* __restrict__ z,
+                                                             long long nz) {
+    constexpr unsigned G = 0x9E3779B9u;
+    constexpr int T = 2;                                  // tiles of four positions per thread and trip: 4 T loads in flight
+    const long long first = 4 * ((long long)blockIdx.x * BM_BLOCK + threadIdx.x);
+    const long long tile = 4LL * gridDim.x * BM_BLOCK;    // positions one sweep of the grid covers
     unsigned long long ha = 0, hb = 0;
     int m = -1;
-    for (; i < n; i += stride) {
-        int r[UN], c[UN], cp[UN];
+    unsigned any = 0;
+    for (long long i0 = first; i0 < n; i0 += T * tile) {
+        int r[T][4], c[T][4], before[T];
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const long long j = i + u * BM_BLOCK;
-            r[u] = j < n ? ir[j] : -1;
-            c[u] = j < n ? ic[j] : -1;
-            cp[u] = (jc != nullptr && j > 0 && j < n) ? ic[j - 1] : -1;      // the neighbour's line: a cache hit
-        }
-        if (jc != nullptr) {
+        for (int t = 0; t < T; ++t) {
+            const long long i = i0 + t * tile;
+            if (VEC && i + 4 <= n) {
+                const int4 rv = *reinterpret_cast<const int4*>(ir + i);
+                const int4 cv = *reinterpret_cast<const int4*>(ic + i);
+                r[t][0] = rv.x; r[t][1] = rv.y; r[t][2] = rv.z; r[t][3] = rv.w;
+                c[t][0] = cv.x; c[t][1] = cv.y; c[t][2] = cv.z; c[t][3] = cv.w;
+            } else {
 #pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                const long long j = i + u * BM_BLOCK;
-                if (j < n) {
-                    // malformed input: stay inside jc
-                    int prev = cp[u] < -1 ? -1 : (cp[u] >= ncols ? ncols - 1 : cp[u]);
-                    int cur = c[u] > ncols ? ncols : c[u];
-                    for (int q = prev + 1; q <= cur; ++q) jc[q] = (int)j;
-                    if (j == n - 1) {
-                        prev = cur < -1 ? -1 : (cur >= ncols ? ncols - 1 : cur);
-                        for (int q = prev + 1; q <= ncols; ++q) jc[q] = (int)n;
-                    }
+                for (int u = 0; u < 4; ++u) {
+                    r[t][u] = i + u < n ? ir[i + u] : -1;
+                    c[t][u] = i + u < n ? ic[i + u] : -1;
                 }
             }
+            before[t] = (jc != nullptr && i > 0 && i < n) ? ic[i - 1] : -1;      // the neighbour's line: a cache hit
         }
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const long long j = i + u * BM_BLOCK;
-            if (j < n) {
-                ha += digest_term((unsigned long long)j, (unsigned)r[u], 0x7F4A7C159E3779B9ULL);
-                hb += digest_term((unsigned long long)j, (unsigned)c[u], 0x2545F4914F6CDD1DULL);
-                m = max(m, r[u]);
+        for (int t = 0; t < T; ++t) {
+            const long long i = i0 + t * tile;
+            unsigned pos = (unsigned)(i + 1) * G;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const long long j = i + u;
+                if (j < n) {
+                    unsigned h1 = ((unsigned)r[t][u] ^ pos) * 0x85EBCA6Bu;
+                    unsigned h2 = (((unsigned)r[t][u] + 0x27D4EB2Fu * (unsigned)c[t][u]) ^ ~pos) * 0xC2B2AE35u;
+                    h1 ^= h1 >> 15;
+                    h2 ^= h2 >> 15;
+                    ha += ((unsigned long long)h1 << 32) | h2;
+                    hb += ((unsigned long long)(unsigned)c[t][u] << 32) | (unsigned)r[t][u];
+                    m = max(m, r[t][u]);
+                    if (jc != nullptr && c[t][u] != before[t]) {
+                        // malformed input: stay inside jc
+                        const int prev = before[t] < -1 ? -1 : (before[t] >= ncols ? ncols - 1 : before[t]);
+                        const int cur = c[t][u] > ncols ? ncols : c[t][u];
+                        for (int q = prev + 1; q <= cur; ++q) jc[q] = (int)j;
+                        before[t] = c[t][u];
+                    }
+                    if (jc != nullptr && j == n - 1) {
+                        const int last = c[t][u] < -1 ? -1 : (c[t][u] >= ncols ? ncols - 1 : c[t][u]);
+                        for (int q = last + 1; q <= ncols; ++q) jc[q] = (int)n;
+                    }
+                }
+                pos += G;
+            }
+        }
+    }
+    if (z != nullptr) {
+        const bool zvec = (reinterpret_cast<uintptr_t>(z) & 15) == 0;
+        constexpr int TZ = 4;
+        for (long long t0 = first; t0 < nz; t0 += TZ * tile) {
+#pragma unroll
+            for (int t = 0; t < TZ; ++t) {
+                const long long p = t0 + t * tile;
+                if (zvec && p + 4 <= nz) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(z + p);
+                    any |= v.x | v.y | v.z | v.w;
+                } else {
+                    for (int u = 0; u < 4 && p + u < nz; ++u) any |= z[p + u];
+                }
             }
         }
     }
@@ -134,24 +166,56 @@ __global__ __launch_bounds__(BM_BLOCK) void k_pattern_digest(const int* __restri
         hb += __shfl_xor(hb, d, 64);
         m = max(m, __shfl_xor(m, d, 64));
     }
-    // one set of atomics per workgroup: thousands of them on three addresses would serialise
+    const bool wave_any = __ballot(any != 0) != 0ULL;
+    // one line of four words per workgroup, summed up by k_digest_final (thousands of atomics on
+    // three addresses would serialise and cost more than the pass itself)
     __shared__ unsigned long long sa[BM_WAVES_PER_BLOCK], sb[BM_WAVES_PER_BLOCK];
-    __shared__ int sm[BM_WAVES_PER_BLOCK];
-    if ((threadIdx.x & 63) == 0) { sa[threadIdx.x >> 6] = ha; sb[threadIdx.x >> 6] = hb; sm[threadIdx.x >> 6] = m; }
+    __shared__ int sm[BM_WAVES_PER_BLOCK], sz[BM_WAVES_PER_BLOCK];
+    if ((threadIdx.x & 63) == 0) {
+        sa[threadIdx.x >> 6] = ha; sb[threadIdx.x >> 6] = hb; sm[threadIdx.x >> 6] = m; sz[threadIdx.x >> 6] = wave_any ? 1 : 0;
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
+        int zany = sz[0];
 #pragma unroll
-        for (int w = 1; w < BM_WAVES_PER_BLOCK; ++w) { ha += sa[w]; hb += sb[w]; m = max(m, sm[w]); }
-        atomicAdd(out, ha);
-        atomicAdd(out + 1, hb);
-        if (m >= 0) atomicMax(reinterpret_cast<int*>(out + 2), m);
+        for (int w = 1; w < BM_WAVES_PER_BLOCK; ++w) { ha += sa[w]; hb += sb[w]; m = max(m, sm[w]); zany |= sz[w]; }
+        unsigned long long* mine = out + 4 * (size_t)(blockIdx.x + 1);
+        mine[0] = ha;
+        mine[1] = hb;
+        mine[2] = (unsigned long long)(long long)m;
+        mine[3] = (unsigned long long)zany;
     }
 }
 
-// out[0..1] = 0, (int)out[2] = -1
-__global__ void k_digest_init(unsigned long long* out) {
-    if (threadIdx.x < 2) out[threadIdx.x] = 0;
-    if (threadIdx.x == 2) { out[2] = 0; *reinterpret_cast<int*>(out + 2) = -1; }
+// out[0..3] = the workgroups' lines out[4*(b+1) ..] combined: two sums, the maximum (as int in out[2]),
+// the count of workgroups that met a nonzero word. One workgroup.
+__global__ __launch_bounds__(BM_BLOCK) void k_digest_final(int nblocks, unsigned long long* out) {
+    unsigned long long ha = 0, hb = 0, nz = 0;
+    int m = -1;
+    for (int b = threadIdx.x; b < nblocks; b += BM_BLOCK) {
+        const unsigned long long* p = out + 4 * (size_t)(b + 1);
+        ha += p[0]; hb += p[1]; m = max(m, (int)(long long)p[2]); nz += p[3];
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        ha += __shfl_xor(ha, d, 64);
+        hb += __shfl_xor(hb, d, 64);
+        nz += __shfl_xor(nz, d, 64);
+        m = max(m, __shfl_xor(m, d, 64));
+    }
+    __shared__ unsigned long long sa[BM_WAVES_PER_BLOCK], sb[BM_WAVES_PER_BLOCK], sn[BM_WAVES_PER_BLOCK];
+    __shared__ int sm[BM_WAVES_PER_BLOCK];
+    if ((threadIdx.x & 63) == 0) { sa[threadIdx.x >> 6] = ha; sb[threadIdx.x >> 6] = hb; sn[threadIdx.x >> 6] = nz; sm[threadIdx.x >> 6] = m; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < BM_WAVES_PER_BLOCK; ++w) { ha += sa[w]; hb += sb[w]; nz += sn[w]; m = max(m, sm[w]); }
+        out[0] = ha;
+        out[1] = hb;
+        out[2] = 0;
+        *reinterpret_cast<int*>(out + 2) = m;
+        out[3] = nz;
+    }
 }
 
 // Columns [col1, col1+nc) of a CSC matrix as a matrix of its own: nonzero range copied, column
@@ -303,14 +367,23 @@ hipError_t index_shift(int* p, long long n, int delta, hipStream_t s) {
     return hipGetLastError();
 }
 
+size_t pattern_digest_words() { return 4 * (size_t)(DIGEST_MAX_BLOCKS + 1); }
+
 hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s,
-                          int ncols, int* jc) {
-    hipLaunchKernelGGL(k_digest_init, dim3(1), dim3(64), 0, s, d_out);
-    if (nnz > 0)
-        hipLaunchKernelGGL(k_pattern_digest, dim3(grid_for((nnz + 3) / 4, 2048)), dim3(BM_BLOCK), 0, s, ir, ic, nnz, d_out,
-                           ncols, jc);
-    else if (jc != nullptr)
-        return fill_i32(jc, (long long)ncols + 1, 0, s);
+                          int ncols, int* jc, const float* z, long long nz) {
+    int nblocks = 0;
+    if (nnz > 0) {
+        const bool vec = ((reinterpret_cast<uintptr_t>(ir) | reinterpret_cast<uintptr_t>(ic)) & 15) == 0;
+        nblocks = (int)grid_for((nnz + 3) / 4, DIGEST_MAX_BLOCKS);
+        const dim3 grid((unsigned)nblocks), block(BM_BLOCK);
+        const unsigned* zw = reinterpret_cast<const unsigned*>(z);
+        if (vec) hipLaunchKernelGGL(k_pattern_digest<true>, grid, block, 0, s, ir, ic, nnz, d_out, ncols, jc, zw, nz);
+        else hipLaunchKernelGGL(k_pattern_digest<false>, grid, block, 0, s, ir, ic, nnz, d_out, ncols, jc, zw, nz);
+    } else if (jc != nullptr) {
+        hipError_t e = fill_i32(jc, (long long)ncols + 1, 0, s);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(k_digest_final, dim3(1), dim3(BM_BLOCK), 0, s, nblocks, d_out);
     return hipGetLastError();
 }
 

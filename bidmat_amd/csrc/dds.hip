@@ -99,7 +99,7 @@ __device__ __forceinline__ float dds_round(const float* __restrict__ A, int k, i
 template <int W, int V, int LPN, bool EXACT, bool FULL, bool LDSROWS = false>
 __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, int myrow, float* o, int rem, int g,
                                           int l, const int (&eld)[V], const bool (&ev)[V],
-                                          const Vec<W> (&b)[V], bool accumulate, bool apply, float vval, int opn) {
+                                          const Vec<W> (&b)[V], float oldp, bool apply, float vval, int opn) {
     constexpr int NG = 64 / LPN;
     constexpr int U = Unroll<V, LPN>::U;
     const int q = l * NG + g;            // the nonzero of this chunk whose result this lane keeps
@@ -121,7 +121,7 @@ __device__ __forceinline__ void dds_chunk(const float* __restrict__ A, int k, in
             res = dds_round<W, V, LPN, EXACT, true, LDSROWS>(A, k, myrow, it0, rem, g, l, label, eld, ev, b, res);
     }
     if (FULL || q < rem) {                                        // o: where this lane's nonzero goes
-        if (accumulate) res += *o;
+        res += oldp;                                              // the addend (0 when the output is overwritten)
         if (apply) res = binop_rt(opn, vval, res);               // only on the last pass over k
         *o = res;
     }
@@ -181,8 +181,10 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dds(DdsArgs a) {
             // the epilogue's operand is requested before the gathers, so that it is there when they are done
             const bool apply = a.V != nullptr && k0 + KT >= a.k;
             const float vval = (apply && q < rem) ? a.V[j0 + q] : 0.f;
-            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
-            else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
+            // so is the addend of an accumulating call (and the running sum of an earlier pass over k)
+            const float oldp = (accumulate && q < rem) ? *o : 0.f;
+            if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, oldp, apply, vval, a.opn);
+            else dds_chunk<W, V, LPN, EXACT, false>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, oldp, apply, vval, a.opn);
             crow = nrow;
             j0 += 64;
             rem -= 64;
@@ -231,8 +233,9 @@ __device__ __forceinline__ void dds_classed_run(const DdsClassedArgs& a, int jst
         float* o = a.P + cpos;
         const bool apply = a.V != nullptr && last;
         const float vval = (apply && q < rem) ? (a.v_classed ? a.V[j0 + q] : a.V[cpos]) : 0.f;     // requested before the gathers
-        if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true, LDSROWS>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
-        else dds_chunk<W, V, LPN, EXACT, false, LDSROWS>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, accumulate, apply, vval, a.opn);
+        const float oldp = (accumulate && q < rem) ? *o : 0.f;                                     // likewise
+        if (rem >= 64) dds_chunk<W, V, LPN, EXACT, true, LDSROWS>(a.A, a.k, crow, o, 64, g, l, eld, ev, b, oldp, apply, vval, a.opn);
+        else dds_chunk<W, V, LPN, EXACT, false, LDSROWS>(a.A, a.k, crow, o, rem, g, l, eld, ev, b, oldp, apply, vval, a.opn);
         crow = nrow; cpos = npos;
         j0 += 64;
         rem -= 64;

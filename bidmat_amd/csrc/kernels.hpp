@@ -44,11 +44,14 @@ hipError_t index_shift(int* p, long long n, int delta, hipStream_t s);
 // out[i] = v for i < n (a kernel, so that callers may record it into a HIP graph)
 hipError_t fill_f32(float* out, long long n, float v, hipStream_t s);
 hipError_t fill_i32(int* out, long long n, int v, hipStream_t s);
-// One pass over the two index arrays of a pattern (device result, 3 x uint64): [0], [1] order- and
-// position-sensitive 64-bit digests of ir and ic, [2] (as int) the largest entry of ir (-1: empty).
+// One pass over the two index arrays of a pattern (device result, 4 x uint64): [0], [1] two 64-bit digests
+// of the sequence of (ic, ir) pairs, [2] (as int) the largest entry of ir (-1: empty). d_out must hold
+// pattern_digest_words() words (the rest is scratch of the pass).
+size_t pattern_digest_words();
 // jc != nullptr: also writes the column pointer jc[ncols+1] that ic implies (ic non-decreasing), in the same pass.
+// z != nullptr (and nnz > 0): d_out[3] = 0 exactly when every word of z[0..nz) is +0.0f.
 hipError_t pattern_digest(const int* ir, const int* ic, long long nnz, unsigned long long* d_out, hipStream_t s,
-                          int ncols = 0, int* jc = nullptr);
+                          int ncols = 0, int* jc = nullptr, const float* z = nullptr, long long nz = 0);
 
 // ---- overflow-segment table shared by dsmult and dds (spmm.hip)
 // Returns in *d_ovf a device table int[ncols+1] (exclusive scan of the number of extra

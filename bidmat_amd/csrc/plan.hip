@@ -760,15 +760,13 @@ std::mutex g_build_mu;
 hipError_t plan_digest(int nnz, int ncols, const int* ir, const int* jc, unsigned long long d[2]) {
     d[0] = d[1] = 0;
     hipError_t e;
-    unsigned long long* dm = (unsigned long long*)ws_get(WS_MISC, 64, &e);
+    const size_t words = pattern_digest_words();
+    unsigned long long* dm = (unsigned long long*)ws_get(WS_MISC, 2 * sizeof(unsigned long long) * words, &e);
     if (!dm) return e;
     if ((e = pattern_digest(ir, ir, nnz, dm, nullptr)) != hipSuccess) return e;
-    if ((e = pattern_digest(jc, jc, (long long)ncols + 1, dm + 4, nullptr)) != hipSuccess) return e;
-    unsigned long long h[5];
-    if ((e = hipMemcpy(h, dm, sizeof(h), hipMemcpyDeviceToHost)) != hipSuccess) return e;
-    d[0] = h[0];
-    d[1] = h[4];
-    return hipSuccess;
+    if ((e = pattern_digest(jc, jc, (long long)ncols + 1, dm + words, nullptr)) != hipSuccess) return e;
+    if ((e = hipMemcpy(&d[0], dm, sizeof(unsigned long long), hipMemcpyDeviceToHost)) != hipSuccess) return e;
+    return hipMemcpy(&d[1], dm + words, sizeof(unsigned long long), hipMemcpyDeviceToHost);
 }
 
 hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* jc, int k_hint,

@@ -206,6 +206,15 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
             eld[i] = ev[i] ? est[i] : 0;     // lanes past k re-read element 0; never stored
             acc[i] = Vec<W>::zero();
         }
+        // An accumulating call's addend is requested now, so that it is there when the column's gathers are
+        // done (with V > 2 the sixteen registers it would hold cost more occupancy than the wait at the end).
+        constexpr bool EARLY_ADDEND = !PLAN && V <= 2;
+        Vec<W> addend[V];
+        if constexpr (EARLY_ADDEND) {
+#pragma unroll
+            for (int i = 0; i < V; ++i)
+                addend[i] = (accumulate && g == 0 && ev[i]) ? Vec<W>::load(outp + est[i]) : Vec<W>::zero();
+        }
         // The next chunk's indices and values are requested before the current chunk's gathers,
         // so their latency overlaps the gathers instead of preceding them.
         const int q = l * (64 / LPN) + g;
@@ -241,7 +250,8 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
                 if (ev[i]) {
                     float* o = outp + est[i];
                     Vec<W> r = acc[i];
-                    if (accumulate) r.add(Vec<W>::load(o));
+                    if constexpr (EARLY_ADDEND) r.add(addend[i]);
+                    else if (accumulate) r.add(Vec<W>::load(o));
                     r.store(o);
                 }
             }

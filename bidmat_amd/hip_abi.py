@@ -44,6 +44,8 @@ SIGNATURES = {
     "bidmat_plan_bytes": (C.c_longlong, [vp]),
     "bidmat_plan_segments": (C.c_int, [vp]),
     "bidmat_dsmultT_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, C.c_int, vp]),
+    "bidmat_dsmultT_plan_staged": (C.c_int, [vp, C.c_int, vp, vp, vp, C.c_int, vp, vp]),
+    "bidmat_plan_heavy_nnz": (C.c_longlong, [vp]),
     "bidmat_spsum_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, C.c_int, vp]),
     "bidmat_spsum_rows_plan": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "bidmat_csc_expand_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),

@@ -84,7 +84,10 @@ int bidmat_sdoprow(int nrows, int ncols, int nnz, float *A, const int *Aic, cons
 int bidmat_sdopcol(int nrows, int ncols, int nnz, float *A, const int *Air, const float *B, int len, int opn);
 
 /* P[j] += dot(A[:,Cir[j]], B[:,Cic[j]]).  Replaces `int dds(int nrows,int nnz,float*A,float*B,
- * int*Cir,int*Cic,float*P)` (Arith.cu:381-389; CUMAT.java:211; caller GSMat.scala:663). */
+ * int*Cir,int*Cic,float*P)` (Arith.cu:381-389; CUMAT.java:211; caller GSMat.scala:663).
+ * bidmat_dds and bidmat_dsmult recognise a pattern they have met before (same device arrays, same
+ * contents: one pass over Cir / Cic per call checks it) and run it through a cached plan from the second
+ * call on; see "cache_cols_after".  DDS results are the same bits either way. */
 int bidmat_dds(int nrows, int nnz, const float *A, const float *B, const int *Cir,
                const int *Cic, float *P);
 
@@ -151,7 +154,9 @@ int bidmat_dds_static_max_cols(void);
  * P[j] = op(V[j], dot_j) with a BinOp code opn (3 = V ./ DDS).  One launch instead of
  * GSMat.DDS + GMat.gOp on the value arrays (GSMat.scala:649-667, GMat.scala:1119-1128,
  * Operators.cu:455-461); bit-identical to bidmat_dds_csc followed by bidmat_applyop_flat.
- * V and P must not overlap (wide k is walked in several passes that keep their running sums in P). */
+ * P == V (the update in place) is allowed while one pass covers k (k <= 1024 with 16-byte aligned A, B and
+ * k % 4 == 0, otherwise k <= 256); beyond that, and for any other overlap of V and P, the call returns
+ * hipErrorInvalidValue (wide k is walked in several passes that keep their running sums in P). */
 int bidmat_dds_csc_op(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir,
                       const int *Sjc, const float *V, int opn, float *P, void *stream);
 
@@ -176,6 +181,15 @@ int bidmat_plan_segments(const bidmat_plan *plan);
  * rows of S). */
 int bidmat_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *Sdata, float *C,
                         int beta, void *stream);
+
+/* bidmat_dsmultT_plan for harnesses that time its two stages apart: event_between (a hipEvent_t passed as
+ * void*, nullable) is recorded on the stream after stage 1 (the gathers into per-segment partial sums) and
+ * before stage 2 (the addition of every row's partial sums).  No counterpart in the reference. */
+int bidmat_dsmultT_plan_staged(bidmat_plan *plan, int k, const float *A, const float *Sdata, float *C,
+                               int beta, void *stream, void *event_between);
+/* Nonzeros that belong to rows cut by column panels ("heavy" rows, whose gathers reuse a panel of A that
+ * stays in L2); the remaining nnz - heavy nonzeros are gathered once each with no reuse.  Blocking. */
+long long bidmat_plan_heavy_nnz(const bidmat_plan *plan);
 
 /* The values of the pattern in plan order, stored in the plan (nnz floats): afterwards
  * bidmat_dsmultT_plan, bidmat_sdmult_plan and bidmat_spsum_rows_plan accept Sdata == NULL and stream
@@ -354,6 +368,14 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *              disjoint share of the row classes so that the L2s hold more of the rows that matter
  *              (1, 2, 4 or 8; default 2; 0 = always the plain one-pass kernel)
  *   "class_strip" columns per wavefront in the class-ordered DDS kernel (default 16, 1..64)
+ *   "cache_cols_after" the reference-shaped bidmat_dsmult / bidmat_dds (which receive no plan handle) find
+ *              their pattern in a fingerprint cache; from this many calls on a pattern they build the column
+ *              side of a plan for it and run through it (default 2; 0 = never look, always the plain kernels)
+ *   "cache_plans" patterns the fingerprint cache keeps, least recently used dropped first (default 4; a
+ *              cached plan of a 100 M-nonzero pattern holds 0.8 GB per side)
+ *   "check_plan" 1 = plans made from now on keep a digest of their pattern and bidmat_dsmult_plan /
+ *              bidmat_dds_plan[_stored] return hipErrorInvalidValue for any other Sir / Sjc (one extra pass
+ *              over the index arrays per call; default 0: passing the plan's own pattern is the caller's duty)
  *   "plan_keep_mb" temporaries of a plan build up to this many MiB stay allocated on the device for the
  *              next build (default 4096: a 100 M-nonzero pattern needs 3.7 GB; 0 = always give them
  *              back); bidmat_release_caches frees them
