@@ -133,6 +133,22 @@ def test_config4_wide_k_power_law_columns(hip):
     sv, sir, sjc, _ = sub_csc(ir, jc, vals, cols)
     ref64, sa = oracle.fsmult_f64(A, k, sv, sir, sjc, nthreads=8)
     close(got, ref64, sa, "C4 sampled + longest columns")
+    # the form bench.py times: through a plan (the plan holds the table of the 3 391 extra segments of the long
+    # columns; uniform rows get no class ordering), the whole 4.1 GB output bit for bit
+    plan = make_plan(hip, nrows, ncols, nnz, dir_, djc, k)
+    assert hip.bidmat_plan_overflow_segments(plan) > 1000
+    dCp = DeviceArray(k * ncols, np.float32)
+    hip_abi.check(hip.bidmat_dsmult_plan(plan, k, dA.ptr, dv.ptr, dir_.ptr, djc.ptr, dCp.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    step = 1 << 28
+    for off in range(0, k * ncols, step):                 # 1 GiB at a time
+        n = min(step, k * ncols - off)
+        a, b = np.empty(n, np.float32), np.empty(n, np.float32)
+        hip_abi.check(hip.bidmat_memcpy_d2h(a.ctypes.data, dC.ptr + 4 * off, 4 * n))
+        hip_abi.check(hip.bidmat_memcpy_d2h(b.ctypes.data, dCp.ptr + 4 * off, 4 * n))
+        assert np.array_equal(a, b), "bidmat_dsmult_plan differs from bidmat_dsmult_csc in floats %d.." % off
+    dCp.free()
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
     # linearity in the values: A*(2S) == 2*(A*S) exactly (scaling by 2 is exact in fp32)
     dv2 = DeviceArray.from_numpy(vals * np.float32(2))
     dC2 = DeviceArray(k * 4096, np.float32)
@@ -182,6 +198,20 @@ def test_config5_nmf_step(hip):
     # dense row sums of H
     ref = H.reshape(ncols, k).astype(np.float64).sum(axis=0)
     np.testing.assert_allclose(drs.numpy(), ref, rtol=1e-5)
+    # the forms bench.py times: V stored in the plan once, Q = V ./ DDS in ONE launch of the class-ordered kernel
+    # (hot rows of every class in LDS, persistent workgroups), G = H *^ Q fed by it: the same bits as the chain above
+    hip_abi.check(hip.bidmat_plan_set_values(plan, dv.ptr, None))
+    dQ2, dG2 = DeviceArray(nnz, np.float32), DeviceArray(k * nrows, np.float32)
+    hip_abi.check(hip.bidmat_dds_plan_stored(plan, k, dW.ptr, dH.ptr, dir_.ptr, djc.ptr, 3, dQ2.ptr, None))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, dH.ptr, dQ2.ptr, dG2.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert np.array_equal(dQ2.numpy(), Q), "bidmat_dds_plan_stored(op_div) differs from DDS + V./R"
+    assert np.array_equal(dG2.numpy(), G)
+    # ... and with the caller's V instead of the stored copy (the fused step reads V through the class order)
+    hip_abi.check(hip.bidmat_dds_plan(plan, k, dW.ptr, dH.ptr, dir_.ptr, djc.ptr, dv.ptr, 3, dQ2.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert np.array_equal(dQ2.numpy(), Q)
+    dQ2.free(), dG2.free()
     hip_abi.check(hip.bidmat_plan_destroy(plan))
 
 
@@ -257,3 +287,48 @@ def test_very_long_columns_keep_their_accuracy_through_the_plan(hip):
     nz = ref64 > 0
     assert float(np.max(np.abs(G.numpy()[nz] - ref64[nz]) / ref64[nz])) <= 5e-6
     hip_abi.check(hip.bidmat_plan_destroy(plan))
+
+
+@pytest.mark.timeout(900)
+def test_three_fresh_100M_patterns_through_the_reference_shaped_dsmultT(hip):
+    """What BIDMach does with every minibatch: a pattern the library has not seen, handed to the reference-shaped
+    A*^S (no plan handle, per-nonzero column array). Three different ~100 M-nonzero patterns one after the other
+    through a fingerprint cache of two entries (so the third evicts the first, 0.8 GB of plan each), then the first
+    again (rebuilt): sampled rows of every result against the oracle, the repeat bit-equal to the first run; the
+    reference-shaped row sums and DDS on the way."""
+    k, nrows, ncols = 256, 100000, 500000
+    rng = np.random.default_rng(6)
+    AT = gen.normal(k * ncols, 31)
+    dAT = DeviceArray.from_numpy(AT)
+    old = hip.bidmat_get_option(b"cache_plans")
+    hip_abi.check(hip.bidmat_release_caches())
+    hip_abi.check(hip.bidmat_set_option(b"cache_plans", 2))
+    try:
+        first = None
+        for seed in (2, 202, 302, 2):
+            ir, jc = gen.pattern(nrows, ncols, ("poisson", 200), ("zipf", 1.1), seed)
+            nnz = int(ir.size)
+            assert 0.9e8 < nnz < 1.1e8
+            vals = gen.uniform_open0(nnz, seed + 30)
+            dir_, djc, dv = DeviceArray.from_numpy(ir), DeviceArray.from_numpy(jc), DeviceArray.from_numpy(vals)
+            dic = DeviceArray(nnz, np.int32)
+            hip_abi.check(hip.bidmat_csc_expand_cols(ncols, nnz, djc.ptr, dic.ptr, None))
+            dG, drs = DeviceArray.zeros(k * nrows), DeviceArray.zeros(nrows)
+            hip_abi.check(hip.bidmat_dsmultT(k, ncols, nnz, dAT.ptr, dv.ptr, dir_.ptr, dic.ptr, dG.ptr), "dsmultT seed %d" % seed)
+            hip_abi.check(hip.bidmat_spsum(nrows, ncols, nnz, dir_.ptr, dic.ptr, dv.ptr, drs.ptr, 2), "spsum seed %d" % seed)
+            G = dG.numpy()
+            rows = np.unique(np.concatenate([rng.integers(0, nrows, 200), [0, 1, 2, int(ir.max())]]))
+            rv, rir, rjc = rows_sub_csc(ir, jc, vals, rows)
+            ref64, sa = oracle.fsmultT_f64(AT, k, rows.size, rv, rir, rjc, nthreads=oracle.max_threads())
+            close(G.reshape(nrows, k)[rows].ravel(), ref64, sa, "bidmat_dsmultT on a fresh pattern (seed %d), sampled rows" % seed)
+            ref = np.bincount(ir, weights=vals.astype(np.float64), minlength=nrows)
+            assert np.allclose(drs.numpy(), ref, rtol=RTOL, atol=0)
+            if seed == 2 and first is None:
+                first = G
+            elif seed == 2:
+                assert np.array_equal(first, G)          # the evicted plan, rebuilt: a function of the pattern only
+            for d in (dir_, djc, dv, dic, dG, drs):
+                d.free()
+    finally:
+        hip_abi.check(hip.bidmat_set_option(b"cache_plans", old))
+        hip_abi.check(hip.bidmat_release_caches())
