@@ -31,7 +31,9 @@ std::atomic<int> g_plan_keep_mb{4096};
 std::atomic<int> g_cache_cols_after{2};
 std::atomic<int> g_cache_plans{4};
 std::atomic<int> g_check_plan{0};
+std::atomic<int> g_plan_builder{0};
 }  // namespace
+int opt_plan_builder() { return g_plan_builder.load(std::memory_order_relaxed); }
 int opt_check_plan() { return g_check_plan.load(std::memory_order_relaxed); }
 int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
 int opt_plan_keep_mb() { return g_plan_keep_mb.load(std::memory_order_relaxed); }
@@ -532,6 +534,44 @@ API long long bidmat_plan_bytes(const bidmat_plan* plan) {
 
 API int bidmat_plan_segments(const bidmat_plan* plan) { return plan ? plan->nseg : 0; }
 
+API long long bidmat_plan_info(const bidmat_plan* plan, const char* name) {
+    if (!plan || !name) return -1;
+    if (!strcmp(name, "nrows")) return plan->nrows;
+    if (!strcmp(name, "ncols")) return plan->ncols;
+    if (!strcmp(name, "nnz")) return plan->nnz;
+    if (!strcmp(name, "sides")) return plan->sides;
+    if (!strcmp(name, "nseg")) return plan->nseg;
+    if (!strcmp(name, "nheavy")) return plan->nheavy;
+    if (!strcmp(name, "npanels")) return plan->npanels;
+    if (!strcmp(name, "panel_cols")) return plan->panel_cols;
+    if (!strcmp(name, "seglen")) return plan->seglen;
+    if (!strcmp(name, "col_classes")) return plan->ncls;
+    if (!strcmp(name, "class_hot")) return plan->hcap;
+    if (!strcmp(name, "longest_column")) return plan->maxlen;
+    if (!strncmp(name, "xcd_start", 9) && name[9] >= '0' && name[9] <= '8' && !name[10]) return plan->xcd_start[name[9] - '0'];
+    return -1;
+}
+
+API int bidmat_plan_array(const bidmat_plan* plan, const char* name, const void** dptr, long long* count) {
+    if (!plan || !name || !dptr || !count) return kInvalid;
+    *dptr = nullptr;
+    *count = 0;
+    const bool rows = (plan->sides & bm::PLAN_ROWS) != 0;
+    const bool cls = (plan->sides & bm::PLAN_COLS) != 0 && plan->ncls == 8;
+    struct { const char* n; const void* p; long long c; } tab[] = {
+        {"pc", plan->pc, rows ? plan->nnz : 0}, {"perm", plan->perm, rows ? plan->nnz : 0},
+        {"segstart", plan->segstart, rows && plan->segstart ? (long long)plan->nseg + 1 : 0},
+        {"segrow", plan->segrow, rows ? plan->nseg : 0}, {"rowseg", plan->rowseg, rows ? plan->nseg : 0},
+        {"rowptr", plan->rowptr, rows ? (long long)plan->nrows + 1 : 0},
+        {"cir", plan->cir, cls ? plan->nnz : 0}, {"cperm", plan->cperm, cls ? plan->nnz : 0},
+        {"cptr", plan->cptr, cls ? 16LL * plan->ncols + 1 : 0},
+        {"ovf", plan->ovf, plan->ovf ? (long long)plan->ncols + 1 : 0},
+    };
+    for (auto& t : tab)
+        if (!strcmp(name, t.n)) { *dptr = t.c > 0 ? t.p : nullptr; *count = t.p ? t.c : 0; return 0; }
+    return kInvalid;
+}
+
 API int bidmat_dsmultT_plan(bidmat_plan* plan, int k, const float* A, const float* Sdata, float* C,
                             int beta, void* stream) {
     auto lock = bm::device_lock();
@@ -952,6 +992,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_check_plan.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "plan_builder")) {
+        if (value != 0 && value != 1) return kInvalid;
+        bm::g_plan_builder.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "class_threads")) {
         if (value != 256 && value != 512 && value != 1024) return kInvalid;
         bm::g_class_threads.store((int)value);
@@ -989,6 +1034,7 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "cache_cols_after")) return bm::g_cache_cols_after.load();
     if (!strcmp(name, "cache_plans")) return bm::g_cache_plans.load();
     if (!strcmp(name, "check_plan")) return bm::opt_check_plan();
+    if (!strcmp(name, "plan_builder")) return bm::opt_plan_builder();
     return -2;
 }
 

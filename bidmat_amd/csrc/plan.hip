@@ -6,6 +6,9 @@
 #include "kernels.hpp"
 #include "scan.hpp"
 #include "workspace.hpp"
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
@@ -421,11 +424,9 @@ hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, c
 
 // Temporaries of one build, carved out of the library's workspace.
 struct BuildTmp {
-    int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *crank = nullptr, *scantmp = nullptr,
-        *class_count = nullptr, *segidx = nullptr, *bad = nullptr;
+    int *cnt = nullptr, *hflag = nullptr, *hrank = nullptr, *hrow = nullptr, *crank = nullptr, *scantmp = nullptr, *bad = nullptr;
     unsigned *keys_in = nullptr, *keys_out = nullptr;
     unsigned long long *colpos_in = nullptr, *colpos_out = nullptr;
-    unsigned char* segclass = nullptr;
     char* sorttmp = nullptr;
     size_t sort_bytes = 0, arena_bytes = 0;
     int sample = 1;
@@ -526,11 +527,10 @@ hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const Bui
     return hipGetLastError();
 }
 
-// Row side through one stable radix sort (rocPRIM) of (panel,row) keys.
-hipError_t build_rows_sorted(bidmat_plan* plan, const int* ir, const int* jc, const BuildTmp& t, int p8, hipStream_t s) {
-    const int nrows = plan->nrows, ncols = plan->ncols, nnz = plan->nnz;
-    const int rbits = bits_for((unsigned long long)nrows);
-    // heavy rows and their ranks
+// Ranks the heavy rows (those the row side cuts by column panels): t.hflag becomes every row's code (heavy
+// rank, or -1), t.hrow the row of every rank. Returns their number in *nheavy_out.
+hipError_t detect_heavy(bidmat_plan* plan, const BuildTmp& t, int p8, int* nheavy_out, hipStream_t s) {
+    const int nrows = plan->nrows;
     int nheavy = 0;
     int h2[2] = {0, 0};                                  // {number of heavy rows, bad-index flag}
     if (plan->npanels >= 2) {
@@ -553,34 +553,79 @@ hipError_t build_rows_sorted(bidmat_plan* plan, const int* ir, const int* jc, co
     } else {
         hipLaunchKernelGGL(k_heavy_rows, dim3(grid_for(nrows, 1 << 30)), dim3(BM_BLOCK), 0, s, nrows, t.hflag, t.hrank, t.hrow);
     }
-    plan->nheavy = nheavy;
+    *nheavy_out = nheavy;
+    return hipGetLastError();
+}
+
+// Row side through one stable radix sort (rocPRIM) of (panel,row) keys: the reference the binned builder
+// (plan_rows.hip) is tested against, and the way out when there are more heavy rows than its LDS bins hold.
+hipError_t build_rows_sorted(bidmat_plan* plan, const int* ir, const int* jc, const BuildTmp& t, int nheavy, int p8, hipStream_t s) {
+    const int nrows = plan->nrows, ncols = plan->ncols, nnz = plan->nnz;
+    const int rbits = bits_for((unsigned long long)nrows);
+    // temporaries sized by the nonzeros
+    unsigned *keys_in = nullptr, *keys_out = nullptr;
+    unsigned long long *colpos_in = nullptr, *colpos_out = nullptr;
+    int *segidx = nullptr, *class_count = nullptr;
+    unsigned char* segclass = nullptr;
+    char* sorttmp = nullptr;
+    size_t sort_bytes = 0;
+    {
+        const unsigned long long maxkey_bound = 8ULL * (unsigned long long)p8 * (unsigned long long)nrows + (unsigned long long)nrows;
+        size_t b1 = 0, b2 = 0, b3 = 0;
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b1, (unsigned*)nullptr, (unsigned*)nullptr, (unsigned long long*)nullptr,
+                                           (unsigned long long*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, b2, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
+                                           (int*)nullptr, (size_t)nnz, 0, rbits, s));
+        auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u),
+                                                   SegmentStart{nullptr, (unsigned)nnz, 1u});
+        PB_CHECK(rocprim::exclusive_scan(nullptr, b3, in, (int*)nullptr, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        sort_bytes = b1 > b2 ? b1 : b2;
+        if (b3 > sort_bytes) sort_bytes = b3;
+    }
+    Arena tmp;
+    for (int pass = 0; pass < 2; ++pass) {
+        tmp.used = 0;
+        class_count = tmp.take<int>(9);
+        keys_in = tmp.take<unsigned>((size_t)nnz);               // later: ids of the segments
+        keys_out = tmp.take<unsigned>((size_t)nnz);
+        colpos_in = tmp.take<unsigned long long>((size_t)nnz);   // later: segment rows in sorted order
+        colpos_out = tmp.take<unsigned long long>((size_t)nnz);
+        segidx = tmp.take<int>((size_t)nnz + 1);
+        segclass = tmp.take<unsigned char>((size_t)nnz);
+        sorttmp = tmp.take<char>(sort_bytes);
+        if (pass == 0) {
+            hipError_t werr;
+            tmp.base = static_cast<char*>(ws_get(WS_PLAN_ROWS_A, tmp.used, &werr, s));
+            if (!tmp.base) return werr;
+        }
+    }
 
     // keys + stable radix sort
     {
         long long nblk = ((long long)ncols * 16 + BM_BLOCK - 1) / BM_BLOCK;
         hipLaunchKernelGGL(k_make_keys, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nrows, jc, ir,
-                           t.hflag, nheavy, plan->npanels, plan->panel_cols, p8, t.keys_in, t.colpos_in, t.bad);
+                           t.hflag, nheavy, plan->npanels, plan->panel_cols, p8, keys_in, colpos_in, t.bad);
     }
     const unsigned long long maxkey = 8ULL * (unsigned long long)p8 * nheavy + (unsigned long long)nrows;
     const int end_bit = bits_for(maxkey);
     {
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, t.keys_in, t.keys_out, t.colpos_in, t.colpos_out, (size_t)nnz, 0, end_bit, s));
-        if (tmp_bytes > t.sort_bytes) return hipErrorOutOfMemory;
-        PB_CHECK(rocprim::radix_sort_pairs(t.sorttmp, tmp_bytes, t.keys_in, t.keys_out, t.colpos_in, t.colpos_out, (size_t)nnz, 0, end_bit, s));
+        PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in, keys_out, colpos_in, colpos_out, (size_t)nnz, 0, end_bit, s));
+        if (tmp_bytes > sort_bytes) return hipErrorOutOfMemory;
+        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, keys_in, keys_out, colpos_in, colpos_out, (size_t)nnz, 0, end_bit, s));
     }
 
     // segment boundaries
-    const SegmentStart starts{t.keys_out, (unsigned)nnz, (unsigned)plan->seglen};
+    const SegmentStart starts{keys_out, (unsigned)nnz, (unsigned)plan->seglen};
     {
         auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u), starts);
         size_t tmp_bytes = 0;
-        PB_CHECK(rocprim::exclusive_scan(nullptr, tmp_bytes, in, t.segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
-        if (tmp_bytes > t.sort_bytes) return hipErrorOutOfMemory;
-        PB_CHECK(rocprim::exclusive_scan(t.sorttmp, tmp_bytes, in, t.segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        PB_CHECK(rocprim::exclusive_scan(nullptr, tmp_bytes, in, segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
+        if (tmp_bytes > sort_bytes) return hipErrorOutOfMemory;
+        PB_CHECK(rocprim::exclusive_scan(sorttmp, tmp_bytes, in, segidx, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
     }
     int nseg = 0;
-    PB_CHECK(hipMemcpy(&nseg, t.segidx + nnz, sizeof(int), hipMemcpyDeviceToHost));
+    PB_CHECK(hipMemcpy(&nseg, segidx + nnz, sizeof(int), hipMemcpyDeviceToHost));
     {
         int badv = 0;                                    // k_make_keys has seen every row index by now
         PB_CHECK(hipMemcpy(&badv, t.bad, sizeof(int), hipMemcpyDeviceToHost));
@@ -604,32 +649,53 @@ hipError_t build_rows_sorted(bidmat_plan* plan, const int* ir, const int* jc, co
         }
     }
     // the sort's inputs are dead by now: their space holds the segment ids and the sorted rows
-    int* const segid = reinterpret_cast<int*>(t.keys_in);
-    unsigned* const segrow_sorted = reinterpret_cast<unsigned*>(t.colpos_in);
+    int* const segid = reinterpret_cast<int*>(keys_in);
+    unsigned* const segrow_sorted = reinterpret_cast<unsigned*>(colpos_in);
     unsigned* const segrow_u = reinterpret_cast<unsigned*>(plan->segrow);
-    PB_CHECK(fill_i32(t.class_count, 9, nseg, s));
-    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, t.keys_out, t.colpos_out,
-                       starts, t.segidx, t.hrow, nheavy > 0 ? nheavy : 1,
-                       nheavy > 0 ? p8 : 0, plan->pc, plan->perm, plan->segstart, segrow_u, segid, t.segclass);
+    PB_CHECK(fill_i32(class_count, 9, nseg, s));
+    hipLaunchKernelGGL(k_emit, dim3(grid_for(nnz)), dim3(BM_BLOCK), 0, s, nnz, keys_out, colpos_out,
+                       starts, segidx, t.hrow, nheavy > 0 ? nheavy : 1,
+                       nheavy > 0 ? p8 : 0, plan->pc, plan->perm, plan->segstart, segrow_u, segid, segclass);
     PB_CHECK(fill_i32(plan->segstart + nseg, 1, nnz, s));
-    hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg, t.segclass, t.class_count);
-    PB_CHECK(hipMemcpy(plan->xcd_start, t.class_count, sizeof(int) * 9, hipMemcpyDeviceToHost));
+    hipLaunchKernelGGL(k_class_bounds, dim3(grid_for(nseg, 1 << 30)), dim3(BM_BLOCK), 0, s, nseg, segclass, class_count);
+    PB_CHECK(hipMemcpy(plan->xcd_start, class_count, sizeof(int) * 9, hipMemcpyDeviceToHost));
 
     // a row's segments, in ascending segment order (stable sort by row)
     {
         size_t tmp_bytes = 0;
         PB_CHECK(rocprim::radix_sort_pairs(nullptr, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
-        if (tmp_bytes > t.sort_bytes) return hipErrorOutOfMemory;
-        PB_CHECK(rocprim::radix_sort_pairs(t.sorttmp, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
+        if (tmp_bytes > sort_bytes) return hipErrorOutOfMemory;
+        PB_CHECK(rocprim::radix_sort_pairs(sorttmp, tmp_bytes, segrow_u, segrow_sorted, segid, plan->rowseg, (size_t)nseg, 0, rbits, s));
         PB_CHECK(coo_compress_cols(nrows, nseg, reinterpret_cast<const int*>(segrow_sorted), plan->rowptr, s));
         PB_CHECK(hipStreamSynchronize(s));
     }
+    if (tmp.used > ((size_t)opt_plan_keep_mb() << 20)) PB_CHECK(ws_drop(WS_PLAN_ROWS_A, s));
     return hipGetLastError();
 }
+
+// BIDMAT_PLAN_TIMING=1 in the environment: every stage of a build is followed by a device synchronisation and
+// its wall-clock time printed (a build then takes longer than without).
+struct StageClock {
+    bool on;
+    std::chrono::steady_clock::time_point t0;
+    StageClock() : on(false) {
+        const char* e = getenv("BIDMAT_PLAN_TIMING");
+        on = e && e[0] == '1';
+        t0 = std::chrono::steady_clock::now();
+    }
+    void mark(const char* what) {
+        if (!on) return;
+        (void)hipDeviceSynchronize();
+        const auto t1 = std::chrono::steady_clock::now();
+        fprintf(stderr, "[bidmathip] plan build: %-28s %8.3f ms\n", what, std::chrono::duration<double, std::milli>(t1 - t0).count());
+        t0 = t1;
+    }
+};
 
 // Builds the halves named in `sides` into `plan` (whose sizes and k_hint are set). On failure the
 // caller drops what was begun.
 hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int sides) {
+    StageClock clock;
     const bool rows = (sides & PLAN_ROWS) != 0, cols = (sides & PLAN_COLS) != 0;
     const int nrows = plan->nrows, ncols = plan->ncols, nnz = plan->nnz;
     const int k_hint = plan->k_hint;
@@ -670,6 +736,7 @@ hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int side
             }
         }
     }
+    clock.mark("row-side arrays allocated");
     if (nnz == 0 || nrows == 0 || ncols == 0) {
         if (rows) {
             PB_CHECK(fill_i32(plan->rowptr, (long long)nrows + 1, 0, s));
@@ -679,32 +746,12 @@ hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int side
         return hipSuccess;
     }
 
-    // temporaries: one arena out of the library's workspace. The row side sorts all nonzeros; the
-    // column side alone only ranks the rows.
-    const size_t nitem = rows ? (size_t)nnz : (size_t)(nrows > (1 << 14) ? nrows : (1 << 14));
-    const size_t scan_n = (size_t)(rows && nnz > nrows ? nnz : nrows);
-    const unsigned long long maxkey_bound = 8ULL * (unsigned long long)p8 * (unsigned long long)nrows + (unsigned long long)nrows;
-    const int rbits = bits_for((unsigned long long)nrows);
+    // temporaries sized by the rows: one arena out of the library's workspace (the row-side builders take
+    // what they need per nonzero from slots of their own)
+    const size_t nitem = (size_t)(nrows > (1 << 14) ? nrows : (1 << 14));
     BuildTmp t;
-    {
-        // all sorts and scans share one scratch area, sized for the largest request
-        size_t b1 = 0, b2 = 0, b3 = 0, b4 = 0;
-        if (rows) {
-            PB_CHECK(rocprim::radix_sort_pairs(nullptr, b1, (unsigned*)nullptr, (unsigned*)nullptr, (unsigned long long*)nullptr,
-                                               (unsigned long long*)nullptr, (size_t)nnz, 0, bits_for(maxkey_bound > 0xffffffffULL ? 0xffffffffULL : maxkey_bound), s));
-            PB_CHECK(rocprim::radix_sort_pairs(nullptr, b2, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr,
-                                               (int*)nullptr, (size_t)nnz, 0, rbits, s));
-            auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<unsigned>(0u),
-                                                       SegmentStart{nullptr, (unsigned)nnz, 1u});
-            PB_CHECK(rocprim::exclusive_scan(nullptr, b3, in, (int*)nullptr, 0, (size_t)nnz + 1, rocprim::plus<int>(), s));
-        } else {
-            PB_CHECK(rocprim::radix_sort_pairs_desc(nullptr, b4, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr, (int*)nullptr,
-                                                    (size_t)nrows, 0, 32, s));
-        }
-        t.sort_bytes = b1 > b2 ? b1 : b2;
-        if (b3 > t.sort_bytes) t.sort_bytes = b3;
-        if (b4 > t.sort_bytes) t.sort_bytes = b4;
-    }
+    PB_CHECK(rocprim::radix_sort_pairs_desc(nullptr, t.sort_bytes, (unsigned*)nullptr, (unsigned*)nullptr, (int*)nullptr, (int*)nullptr,
+                                            (size_t)nrows, 0, 32, s));
     Arena tmp;
     for (int pass = 0; pass < 2; ++pass) {
         tmp.used = 0;
@@ -713,14 +760,11 @@ hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int side
         t.hrank = tmp.take<int>((size_t)nrows + 2);        // [nrows] = number of heavy rows, [nrows+1] = bad-index flag
         t.hrow = tmp.take<int>((size_t)nrows);
         t.crank = tmp.take<int>((size_t)nrows);            // rank of a row among its class's hot rows, or -1
-        t.scantmp = tmp.take<int>(scan_tmp_ints((long long)scan_n));
-        t.class_count = tmp.take<int>(9);
-        t.keys_in = tmp.take<unsigned>(nitem);             // later: ids of the segments
+        t.scantmp = tmp.take<int>(scan_tmp_ints((long long)nrows));
+        t.keys_in = tmp.take<unsigned>(nitem);             // the ranking of the rows by count (column side)
         t.keys_out = tmp.take<unsigned>(nitem);
-        t.colpos_in = tmp.take<unsigned long long>(nitem); // later: segment rows in sorted order
+        t.colpos_in = tmp.take<unsigned long long>(nitem);
         t.colpos_out = tmp.take<unsigned long long>(nitem);
-        t.segidx = tmp.take<int>(rows ? (size_t)nnz + 1 : 1);
-        t.segclass = tmp.take<unsigned char>(rows ? (size_t)nnz : 1);
         t.sorttmp = tmp.take<char>(t.sort_bytes);
         if (pass == 0) {
             hipError_t werr;
@@ -737,16 +781,27 @@ hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int side
     // few, long-lived workgroups: every one flushes its LDS histogram once at the end
     t.sample = (long long)nnz >= HIST_SAMPLE_FROM ? HIST_SAMPLE : 1;     // cnt[r] ~ (nonzeros of row r) / sample
     hipLaunchKernelGGL(k_row_hist, dim3(grid_for(nnz, 1024)), dim3(BM_BLOCK), 0, s, nnz, nrows, t.sample, ir, t.cnt, t.bad);
+    clock.mark("workspace + row histogram");
 
     if (cols) {
         PB_CHECK(build_cols(plan, ir, jc, t, s));
+        clock.mark("column side");
         if (!rows) {
             int badv = 0;                                // set by the histogram (as far as it looked) or the class ordering
             PB_CHECK(hipMemcpy(&badv, t.bad, sizeof(int), hipMemcpyDeviceToHost));
             if (badv) return hipErrorInvalidValue;
         }
     }
-    if (rows) PB_CHECK(build_rows_sorted(plan, ir, jc, t, p8, s));
+    if (rows) {
+        int nheavy = 0;
+        PB_CHECK(detect_heavy(plan, t, p8, &nheavy, s));
+        plan->nheavy = nheavy;
+        clock.mark("heavy rows ranked");
+        int unfit = 1;
+        if (opt_plan_builder() == 0) PB_CHECK(build_rows_binned(plan, ir, jc, t.hflag, t.hrow, nheavy, p8, t.bad, &unfit, s));
+        if (unfit) PB_CHECK(build_rows_sorted(plan, ir, jc, t, nheavy, p8, s));
+        clock.mark(unfit ? "row side (library sort)" : "row side (counting sorts)");
+    }
     PB_CHECK(hipGetLastError());
     if (t.arena_bytes > ((size_t)opt_plan_keep_mb() << 20)) PB_CHECK(ws_drop(WS_PLAN));
     return hipSuccess;

@@ -80,6 +80,13 @@ hipError_t plan_build(int nrows, int ncols, int nnz, const int* ir, const int* j
 // made from. On failure the plan keeps the halves it had.
 hipError_t plan_extend(bidmat_plan* p, const int* ir, const int* jc, int sides);
 hipError_t plan_free(bidmat_plan* p);
+// Row side by per-panel counting sorts (plan_rows.hip): fills pc, perm, rowptr (allocated by the caller) and
+// allocates and fills the segment tables. hcode[r]: heavy rank of row r or -1; hrow: row of every rank.
+// At most rows_binned_max_heavy() heavy rows.
+int rows_binned_max_heavy();
+// *unfit = 1 (with hipSuccess, nothing allocated in the plan) when the pattern does not fit this builder.
+hipError_t build_rows_binned(bidmat_plan* plan, const int* ir, const int* jc, const int* hcode, const int* hrow,
+                             int nheavy, int p8, int* bad, int* unfit, hipStream_t s);
 // d[0], d[1] = digests of ir[nnz] and jc[ncols+1] (blocking; default stream)
 hipError_t plan_digest(int nnz, int ncols, const int* ir, const int* jc, unsigned long long d[2]);
 // pvals[p] = data[perm[p]] (allocates pvals on first use).

@@ -18,7 +18,9 @@ enum WsSlot {
     WS_REDUCE,        // float[...]    partials of the dense reductions
     WS_TRANS_IN,      // float[...]    transposed dense operand of S*A / S^T*A
     WS_TRANS_OUT,     // float[...]    transposed result of S*A / S^T*A
-    WS_PLAN,          // bytes         temporaries of a plan build (dropped again when large)
+    WS_PLAN,          // bytes         temporaries of a plan build sized by the rows
+    WS_PLAN_ROWS_A,   // bytes         temporaries of the row side of a plan build (dropped again when large)
+    WS_PLAN_ROWS_B,   // bytes         likewise, the part sized by the nonzeros of light rows
     WS_TRANSPOSE,     // bytes         sort buffers of the sparse transpose
     WS_NSLOTS
 };

@@ -43,6 +43,8 @@ SIGNATURES = {
     "bidmat_plan_destroy": (C.c_int, [vp]),
     "bidmat_plan_bytes": (C.c_longlong, [vp]),
     "bidmat_plan_segments": (C.c_int, [vp]),
+    "bidmat_plan_info": (C.c_longlong, [vp, C.c_char_p]),
+    "bidmat_plan_array": (C.c_int, [vp, C.c_char_p, C.POINTER(vp), C.POINTER(C.c_longlong)]),
     "bidmat_dsmultT_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, C.c_int, vp]),
     "bidmat_dsmultT_plan_staged": (C.c_int, [vp, C.c_int, vp, vp, vp, C.c_int, vp, vp]),
     "bidmat_plan_heavy_nnz": (C.c_longlong, [vp]),

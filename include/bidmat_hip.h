@@ -175,6 +175,14 @@ int bidmat_plan_destroy(bidmat_plan *plan);
 long long bidmat_plan_bytes(const bidmat_plan *plan);
 /* Number of row segments of the plan (each yields one k-vector partial sum). */
 int bidmat_plan_segments(const bidmat_plan *plan);
+/* Inspection (tests, tools; no counterpart in the reference).  bidmat_plan_info: a scalar of the plan by name
+ * ("nrows", "ncols", "nnz", "sides" (1 row side | 2 column side), "nseg", "nheavy", "npanels", "panel_cols",
+ * "seglen", "col_classes", "class_hot", "longest_column", "xcd_start0" .. "xcd_start8"); -1 for an unknown name.
+ * bidmat_plan_array: device address and element count (int32 each) of one of the plan's index arrays
+ * ("pc", "perm", "segstart", "segrow", "rowseg", "rowptr", "cir", "cperm", "cptr", "ovf"; count 0 when the
+ * plan does not hold it).  The arrays stay the plan's. */
+long long bidmat_plan_info(const bidmat_plan *plan, const char *name);
+int bidmat_plan_array(const bidmat_plan *plan, const char *name, const void **dptr, long long *count);
 
 /* C = beta*C + A*S^T through a plan.  A k x ncols, C k x nrows(S).  Sdata: the nnz values
  * in the original CSC order.  With beta == 0 every column of C is written (zeros for empty
@@ -376,6 +384,9 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "check_plan" 1 = plans made from now on keep a digest of their pattern and bidmat_dsmult_plan /
  *              bidmat_dds_plan[_stored] return hipErrorInvalidValue for any other Sir / Sjc (one extra pass
  *              over the index arrays per call; default 0: passing the plan's own pattern is the caller's duty)
+ *   "plan_builder" how the row side of a plan is put in order: 0 = stable counting sorts per column panel and by
+ *              row, written for this layout (default), 1 = one library radix sort of (key, position) pairs (also
+ *              taken by itself when more than 24 575 rows are cut by panels); both give the same plan, bit for bit
  *   "plan_keep_mb" temporaries of a plan build up to this many MiB stay allocated on the device for the
  *              next build (default 4096: a 100 M-nonzero pattern needs 3.7 GB; 0 = always give them
  *              back); bidmat_release_caches frees them
