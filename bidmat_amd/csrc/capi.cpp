@@ -32,7 +32,9 @@ std::atomic<int> g_cache_cols_after{2};
 std::atomic<int> g_cache_plans{4};
 std::atomic<int> g_check_plan{0};
 std::atomic<int> g_plan_builder{0};
+std::atomic<int> g_plan_pool_mb{4096};
 }  // namespace
+int opt_plan_pool_mb() { return g_plan_pool_mb.load(std::memory_order_relaxed); }
 int opt_plan_builder() { return g_plan_builder.load(std::memory_order_relaxed); }
 int opt_check_plan() { return g_check_plan.load(std::memory_order_relaxed); }
 int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
@@ -997,6 +999,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_plan_builder.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "plan_pool_mb")) {
+        if (value < 0 || value > (1 << 20)) return kInvalid;
+        bm::g_plan_pool_mb.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "class_threads")) {
         if (value != 256 && value != 512 && value != 1024) return kInvalid;
         bm::g_class_threads.store((int)value);
@@ -1035,6 +1042,7 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "cache_plans")) return bm::g_cache_plans.load();
     if (!strcmp(name, "check_plan")) return bm::opt_check_plan();
     if (!strcmp(name, "plan_builder")) return bm::opt_plan_builder();
+    if (!strcmp(name, "plan_pool_mb")) return bm::opt_plan_pool_mb();
     return -2;
 }
 
@@ -1051,5 +1059,7 @@ API int bidmat_release_caches(void) {
             else ++it;
         }
     }
-    return (int)bm::ws_release();
+    hipError_t p = bm::pool_release();
+    hipError_t w = bm::ws_release();
+    return (int)(p != hipSuccess ? p : w);
 }

@@ -14,6 +14,7 @@ int opt_class_phases(); // passes of A*S over a class-ordered pattern (1, 2, 4, 
 int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..64)
 int opt_plan_keep_mb(); // plan-build temporaries up to this many MiB stay allocated for the next build
 int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: -1 = by k_hint (default), 0 = none
+int opt_plan_pool_mb(); // MiB of freed plan blocks kept per device for the next plans
 int opt_plan_builder(); // row side of a plan: 0 = per-panel counting sorts (default), 1 = one library radix sort
 int opt_check_plan();  // 1: plans keep a digest of their pattern and the plan-taking calls compare it
 int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always

@@ -285,6 +285,62 @@ __global__ __launch_bounds__(BM_BLOCK) void k_top_coverage(int nrows, const int*
     if (threadIdx.x == 0) { out[0] = s1[0]; out[1] = s8[0]; }
 }
 
+// Nonzeros in the N most frequent rows without sorting the counts: rows are binned by count (exactly below
+// 2048, above that by the exponent and six more bits: under 2 % wide), per bin the rows and the sum of their
+// counts. k_top_from_bins then walks the bins from the top until N rows are in. The result steers a yes/no
+// choice that changes no product, so the small error of the wide bins is of no account.
+constexpr int TOPBINS = 2048 + 21 * 64;
+__device__ __forceinline__ int count_bin(unsigned c) {
+    if (c < 2048u) return (int)c;
+    const int e = 31 - __clz((int)c);                       // >= 11
+    return 2048 + (e - 11) * 64 + (int)((c >> (e - 6)) & 63u);
+}
+__global__ __launch_bounds__(BM_BLOCK) void k_count_bins(int nrows, const int* __restrict__ cnt, int* __restrict__ brows,
+                                                         unsigned long long* __restrict__ bsum) {
+    __shared__ int lr[TOPBINS];
+    __shared__ unsigned long long ls[TOPBINS];
+    for (int i = threadIdx.x; i < TOPBINS; i += BM_BLOCK) { lr[i] = 0; ls[i] = 0; }
+    __syncthreads();
+    for (long long r = (long long)blockIdx.x * BM_BLOCK + threadIdx.x; r < nrows; r += (long long)gridDim.x * BM_BLOCK) {
+        const unsigned c = (unsigned)cnt[r];
+        if (c == 0) continue;
+        const int b = count_bin(c);
+        atomicAdd(&lr[b], 1);
+        atomicAdd(&ls[b], (unsigned long long)c);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < TOPBINS; i += BM_BLOCK) {
+        if (lr[i]) { atomicAdd(&brows[i], lr[i]); atomicAdd(&bsum[i], ls[i]); }
+    }
+}
+// out[0], out[1] = nonzeros in the n1 / n8 most frequent rows (one wave; the bins are few)
+__global__ void k_top_from_bins(const int* __restrict__ brows, const unsigned long long* __restrict__ bsum, int n1, int n8,
+                                unsigned long long* __restrict__ out) {
+    if (threadIdx.x != 0) return;
+    long long rows = 0;
+    unsigned long long sum = 0;
+    bool done1 = false;
+    out[0] = out[1] = 0;
+    for (int b = TOPBINS - 1; b >= 0; --b) {
+        const long long nr = brows[b];
+        if (nr == 0) continue;
+        const unsigned long long sb = bsum[b];
+        for (int which = done1 ? 1 : 0; which < 2; ++which) {
+            const long long want = which == 0 ? n1 : n8;
+            if (rows + nr >= want) {
+                out[which] = sum + (unsigned long long)((double)sb * (double)(want - rows) / (double)nr);
+                if (which == 0) done1 = true; else return;
+            } else {
+                break;
+            }
+        }
+        rows += nr;
+        sum += sb;
+    }
+    if (!done1) out[0] = sum;
+    out[1] = sum;
+}
+
 inline unsigned grid_for(long long n, int maxblocks = 16384) {
     long long b = (n + BM_BLOCK - 1) / BM_BLOCK;
     if (b < 1) b = 1;
@@ -301,14 +357,22 @@ inline int bits_for(unsigned long long maxval) {
 }  // namespace
 
 namespace {
+// The plan's memory goes back to the pool of plan blocks (idle by then: plan_free and the failure paths of
+// a build synchronise first).
 void free_all(std::initializer_list<void**> bufs, hipError_t* e) {
     for (void** b : bufs) {
         if (*b) {
-            hipError_t f = hipFree(*b);
+            hipError_t f = pool_free(*b);
             if (f != hipSuccess) *e = f;
             *b = nullptr;
         }
     }
+}
+template <typename T>
+hipError_t plan_alloc(T** p, size_t bytes) {
+    hipError_t e;
+    *p = static_cast<T*>(pool_alloc(bytes, &e));
+    return e;
 }
 // Frees one half of a plan and marks it absent.
 hipError_t drop_rows(bidmat_plan* p) {
@@ -334,6 +398,7 @@ hipError_t drop_cols(bidmat_plan* p) {
 
 hipError_t plan_free(bidmat_plan* p) {
     if (!p) return hipSuccess;
+    (void)hipDeviceSynchronize();            // kernels that still read the plan finish before its blocks can be reused
     hipError_t e = drop_rows(p), f = drop_cols(p);
     delete p;
     return e != hipSuccess ? e : f;
@@ -360,7 +425,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_permute_values(long long n, const 
 
 hipError_t value_buffer(float** buf, int nnz) {
     if (*buf) return hipSuccess;
-    hipError_t e = hipMalloc((void**)buf, sizeof(float) * (size_t)nnz);
+    hipError_t e = plan_alloc(buf, sizeof(float) * (size_t)nnz);
     if (e != hipSuccess) { (void)hipGetLastError(); *buf = nullptr; }
     return e;
 }
@@ -397,9 +462,9 @@ hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, c
     if (ncols <= 0 || nnz <= 0 || (long long)ncols * 16 + 1 > 0x7fffffffLL) return hipSuccess;
     hipError_t e;
     const size_t nsub = (size_t)ncols * 16 + 1;
-    if ((e = hipMalloc((void**)&plan->cptr, sizeof(int) * (nsub + 1))) != hipSuccess) { (void)hipGetLastError(); return e; }
-    if ((e = hipMalloc((void**)&plan->cir, sizeof(int) * (size_t)nnz)) != hipSuccess) { (void)hipGetLastError(); return e; }
-    if ((e = hipMalloc((void**)&plan->cperm, sizeof(int) * (size_t)nnz)) != hipSuccess) { (void)hipGetLastError(); return e; }
+    if ((e = plan_alloc(&plan->cptr, sizeof(int) * (nsub + 1))) != hipSuccess) return e;
+    if ((e = plan_alloc(&plan->cir, sizeof(int) * (size_t)nnz)) != hipSuccess) return e;
+    if ((e = plan_alloc(&plan->cperm, sizeof(int) * (size_t)nnz)) != hipSuccess) return e;
     int* d_maxlen = plan->cptr + nsub;                   // one spare int behind the table
     if ((e = fill_i32(d_maxlen, 1, 0, s)) != hipSuccess) return e;
     const long long nblk = ((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
@@ -445,7 +510,7 @@ hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const Bui
             int n = 0;
             PB_CHECK(hipMemcpy(&n, tbl + ncols, sizeof(int), hipMemcpyDeviceToHost));
             if (n > 0) {
-                PB_CHECK(hipMalloc((void**)&plan->ovf, sizeof(int) * ((size_t)ncols + 1)));
+                PB_CHECK(plan_alloc(&plan->ovf, sizeof(int) * ((size_t)ncols + 1)));
                 PB_CHECK(hipMemcpy(plan->ovf, tbl, sizeof(int) * ((size_t)ncols + 1), hipMemcpyDeviceToDevice));
                 plan->novf = n;
                 plan->col_bytes += sizeof(int) * ((size_t)ncols + 1);
@@ -465,9 +530,30 @@ hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const Bui
     const bool candidate = mode == 1 || (mode < 0 && ncols > 0 && nnz / ncols >= 64 &&
                                          (long long)nrows * 4 * k_hint > (8LL << 20));
     int* hotrank = nullptr;
-    if (candidate && (size_t)nrows <= (size_t)nnz) {
-        const long long n1 = (4LL << 20) / (4LL * k_hint);
-        int* iota = reinterpret_cast<int*>(t.keys_in);             // all free until the key sort
+    // hot rows per class kept in LDS. -1 (default): what the LDS budget holds when k_hint < 256, none
+    // from k = 256 on, where they were measured to change nothing (4.78 ms without, 4.85 ms with
+    // 128 rows per class: the 1024-thread persistent workgroups that share the LDS rows cost
+    // what the rows save).
+    long long hcap = opt_class_hot();
+    if (hcap < 0) hcap = k_hint < 256 ? (long long)(dds_classed_lds_budget() / (4 * (size_t)k_hint)) : 0;
+    if (hcap > 1024) hcap = 1024;
+    const long long n1 = (4LL << 20) / (4LL * k_hint);
+    if (candidate && (size_t)nrows <= (size_t)nnz && hcap == 0) {
+        // no list of hot rows to make: the coverage of the top rows comes from a histogram of the counts
+        int* brows = reinterpret_cast<int*>(t.colpos_in);
+        unsigned long long* bsum = t.colpos_out + 8;
+        unsigned long long* cov = t.colpos_out;
+        PB_CHECK(fill_i32(brows, TOPBINS, 0, s));
+        PB_CHECK(fill_i32(reinterpret_cast<int*>(bsum), 2 * TOPBINS, 0, s));
+        hipLaunchKernelGGL(k_count_bins, dim3(grid_for(nrows, 256)), dim3(BM_BLOCK), 0, s, nrows, t.cnt, brows, bsum);
+        hipLaunchKernelGGL(k_top_from_bins, dim3(1), dim3(64), 0, s, brows, bsum, (int)(n1 < nrows ? n1 : nrows),
+                           (int)(8 * n1 < nrows ? 8 * n1 : nrows), cov);
+        unsigned long long h[2] = {0, 0};
+        PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
+        // at least a tenth of all gathers must move from "misses L2" to "hits L2"
+        if (mode < 0) want = (double)(h[1] - h[0]) * t.sample >= 0.10 * (double)nnz;
+    } else if (candidate && (size_t)nrows <= (size_t)nnz) {
+        int* iota = reinterpret_cast<int*>(t.keys_in);
         unsigned* cnt_sorted = t.keys_out;
         int* rows_sorted = reinterpret_cast<int*>(t.colpos_in);
         unsigned long long* cov = reinterpret_cast<unsigned long long*>(t.colpos_out);
@@ -484,14 +570,7 @@ hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const Bui
             PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));
             // at least a tenth of all gathers must move from "misses L2" to "hits L2"
             if (mode < 0) want = (double)(h[1] - h[0]) * t.sample >= 0.10 * (double)nnz;
-            // hot rows per class kept in LDS. -1 (default): what 128 KiB hold when k_hint < 256, none
-            // from k = 256 on, where they were measured to change nothing (4.78 ms without, 4.85 ms with
-            // 128 rows per class: the 1024-thread persistent workgroups that share the LDS rows cost
-            // what the rows save).
-            long long hcap = opt_class_hot();
-            if (hcap < 0) hcap = k_hint < 256 ? (long long)(dds_classed_lds_budget() / (4 * (size_t)k_hint)) : 0;
-            if (hcap > 1024) hcap = 1024;
-            if (want && hcap > 0) {
+            if (want) {
                 const int ntop = (int)(8 * hcap < nrows ? 8 * hcap : nrows);
                 std::vector<int> top((size_t)ntop), cnts((size_t)ntop);
                 PB_CHECK(hipMemcpy(top.data(), rows_sorted, sizeof(int) * (size_t)ntop, hipMemcpyDeviceToHost));
@@ -506,7 +585,7 @@ hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const Bui
                     ranks.push_back(filled[x]++);
                 }
                 if (!rows.empty()) {
-                    PB_CHECK(hipMalloc((void**)&plan->hotrows, sizeof(int) * hotrows.size()));
+                    PB_CHECK(plan_alloc(&plan->hotrows, sizeof(int) * hotrows.size()));
                     PB_CHECK(hipMemcpy(plan->hotrows, hotrows.data(), sizeof(int) * hotrows.size(), hipMemcpyHostToDevice));
                     plan->hcap = (int)hcap;
                     plan->col_bytes += sizeof(int) * hotrows.size();
@@ -642,7 +721,7 @@ hipError_t build_rows_sorted(bidmat_plan* plan, const int* ir, const int* jc, co
             plan->segrow = own.take<int>((size_t)nseg);
             plan->rowseg = own.take<int>((size_t)nseg);
             if (pass == 0) {
-                PB_CHECK(hipMalloc(&plan->block_seg, own.used));
+                PB_CHECK(plan_alloc(&plan->block_seg, own.used));
                 own.base = static_cast<char*>(plan->block_seg);
                 plan->row_bytes += own.used;
             }
@@ -730,7 +809,7 @@ hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int side
             plan->perm = own.take<int>((size_t)nnz);
             plan->pc = own.take<int>((size_t)nnz);
             if (pass == 0) {
-                PB_CHECK(hipMalloc(&plan->block_nnz, own.used));
+                PB_CHECK(plan_alloc(&plan->block_nnz, own.used));
                 own.base = static_cast<char*>(plan->block_nnz);
                 plan->row_bytes += own.used;
             }

@@ -773,7 +773,9 @@ hipError_t build_rows_binned(bidmat_plan* plan, const int* ir, const int* jc, co
             plan->segrow = own.take<int>((size_t)nseg);
             plan->rowseg = own.take<int>((size_t)nseg);
             if (pass == 0) {
-                RB_CHECK(hipMalloc(&plan->block_seg, own.used));
+                hipError_t perr;
+                plan->block_seg = pool_alloc(own.used, &perr);
+                RB_CHECK(perr);
                 own.base = static_cast<char*>(plan->block_seg);
                 plan->row_bytes += own.used;
             }

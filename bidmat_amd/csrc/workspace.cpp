@@ -5,8 +5,11 @@
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 
 namespace bm {
+
+int opt_plan_pool_mb();
 
 namespace {
 struct Slot { void* ptr = nullptr; size_t bytes = 0; };
@@ -105,6 +108,93 @@ hipError_t ws_release() {
             ++it;
         }
     }
+    return e;
+}
+
+// ---- pool of plan blocks
+namespace {
+struct PoolBlock { void* p; size_t bytes; };
+struct Pool {
+    std::vector<PoolBlock> kept;                 // idle blocks
+    std::map<void*, size_t> live;                // blocks handed out
+    size_t kept_bytes = 0;
+};
+std::map<int, Pool> g_pools;
+std::mutex g_pool_mu;
+}  // namespace
+
+void* pool_alloc(size_t bytes, hipError_t* err) {
+    int dev = 0;
+    *err = hipGetDevice(&dev);
+    if (*err != hipSuccess) return nullptr;
+    if (bytes == 0) bytes = 256;
+    std::lock_guard<std::mutex> lock(g_pool_mu);
+    Pool& pool = g_pools[dev];
+    // best fit among the kept blocks that do not waste more than a quarter
+    int best = -1;
+    for (int i = 0; i < (int)pool.kept.size(); ++i) {
+        const size_t b = pool.kept[i].bytes;
+        if (b >= bytes && b <= bytes + bytes / 4 + (1u << 20) && (best < 0 || b < pool.kept[best].bytes)) best = i;
+    }
+    if (best >= 0) {
+        PoolBlock blk = pool.kept[best];
+        pool.kept.erase(pool.kept.begin() + best);
+        pool.kept_bytes -= blk.bytes;
+        pool.live[blk.p] = blk.bytes;
+        return blk.p;
+    }
+    void* p = nullptr;
+    *err = hipMalloc(&p, bytes);
+    if (*err != hipSuccess) {
+        // out of memory with idle blocks in the pool: give them back to the device and try once more
+        (void)hipGetLastError();
+        for (PoolBlock& b : pool.kept) (void)hipFree(b.p);
+        pool.kept.clear();
+        pool.kept_bytes = 0;
+        *err = hipMalloc(&p, bytes);
+        if (*err != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    }
+    pool.live[p] = bytes;
+    return p;
+}
+
+hipError_t pool_free(void* p) {
+    if (!p) return hipSuccess;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(g_pool_mu);
+    Pool& pool = g_pools[dev];
+    auto it = pool.live.find(p);
+    if (it == pool.live.end()) return hipFree(p);          // not from this device's pool
+    const size_t bytes = it->second;
+    pool.live.erase(it);
+    const size_t limit = (size_t)opt_plan_pool_mb() << 20;
+    if (bytes > limit) return hipFree(p);
+    // make room: the oldest kept blocks go first
+    while (!pool.kept.empty() && pool.kept_bytes + bytes > limit) {
+        e = hipFree(pool.kept.front().p);
+        pool.kept_bytes -= pool.kept.front().bytes;
+        pool.kept.erase(pool.kept.begin());
+        if (e != hipSuccess) return e;
+    }
+    pool.kept.push_back(PoolBlock{p, bytes});
+    pool.kept_bytes += bytes;
+    return hipSuccess;
+}
+
+hipError_t pool_release() {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(g_pool_mu);
+    Pool& pool = g_pools[dev];
+    for (PoolBlock& b : pool.kept) {
+        hipError_t f = hipFree(b.p);
+        if (f != hipSuccess) e = f;
+    }
+    pool.kept.clear();
+    pool.kept_bytes = 0;
     return e;
 }
 

@@ -38,6 +38,15 @@ hipError_t ws_release();
 // Total bytes currently held on the current device.
 size_t ws_bytes();
 
+// Device memory of plans comes from a small pool per device: a block given back is kept (up to
+// opt_plan_pool_mb() MiB in all) and handed out again to a request it fits without wasting more than a
+// quarter, so that callers who build a plan per minibatch do not pay hipMalloc + hipFree (each a device-wide
+// synchronisation) for the same sizes over and over. Blocks must be idle when they are given back.
+void* pool_alloc(size_t bytes, hipError_t* err);
+hipError_t pool_free(void* p);
+// Frees every kept block of the current device.
+hipError_t pool_release();
+
 // Host threads that share a device also share its scratch buffers and cached plans. Every entry
 // point that takes scratch or a cached plan holds this lock of the current device from its first
 // ws_get to its last launch (the blocking entries: until their synchronisation), so that another

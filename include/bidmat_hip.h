@@ -387,6 +387,9 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "plan_builder" how the row side of a plan is put in order: 0 = stable counting sorts per column panel and by
  *              row, written for this layout (default), 1 = one library radix sort of (key, position) pairs (also
  *              taken by itself when more than 24 575 rows are cut by panels); both give the same plan, bit for bit
+ *   "plan_pool_mb" device memory of destroyed (or evicted) plans kept for the next plans, MiB per device (default
+ *              4096; 0 = give every block back at once): a caller that meets a new pattern with every minibatch
+ *              would otherwise pay hipMalloc + hipFree for the same sizes on every call; bidmat_release_caches frees it
  *   "plan_keep_mb" temporaries of a plan build up to this many MiB stay allocated on the device for the
  *              next build (default 4096: a 100 M-nonzero pattern needs 3.7 GB; 0 = always give them
  *              back); bidmat_release_caches frees them
