@@ -2,6 +2,7 @@
 // bandwidth-bound kernels; every sum has a fixed order (two-stage, no atomics).
 #include "common.hpp"
 #include "kernels.hpp"
+#include "ops.hpp"
 #include "workspace.hpp"
 #include <math.h>
 
@@ -261,6 +262,43 @@ hipError_t reduce2_impl(int nrows, int ncols, const float* A, float* B, hipStrea
     return hipGetLastError();
 }
 
+// Reduction with ANY of the 15 binary ops (most are neither associative nor commutative, so the order IS the
+// result): the order of the reference's kernels (Operators.cu:650-671, 828-851). 32 lanes per output; lane t
+// folds elements t, t+32, ... from the left, then for i = 1, 2, 4, ... the lanes t with t + i < L = min(n, 32)
+// take op(own, lane t+i's value of the step before). DIM == 1: one output per column (elements are
+// contiguous), DIM == 2: one per row (elements nrows apart).
+template <int DIM>
+__global__ __launch_bounds__(BM_BLOCK) void k_reduce_tree(int nrows, int ncols, const float* __restrict__ A,
+                                                          float* __restrict__ out, int opn) {
+    const long long o = ((long long)blockIdx.x * BM_BLOCK + threadIdx.x) >> 5;
+    const int t = threadIdx.x & 31;
+    const int nout = DIM == 1 ? ncols : nrows;
+    const int n = DIM == 1 ? nrows : ncols;
+    const bool live = o < nout;
+    const int L = n < 32 ? n : 32;
+    float v = 0.f;
+    if (live && t < L) {
+        const float* base = DIM == 1 ? A + (size_t)o * nrows : A + o;
+        const size_t step = DIM == 1 ? 1 : (size_t)nrows;
+        v = base[(size_t)t * step];
+        for (long long e = t + 32; e < n; e += 32) v = binop_rt(opn, v, base[(size_t)e * step]);
+    }
+    for (int i = 1; i < L; i <<= 1) {
+        const float other = __shfl_down(v, i, 32);
+        if (t + i < L) v = binop_rt(opn, v, other);
+    }
+    if (live && t == 0) out[o] = v;
+}
+
+template <int DIM>
+hipError_t reduce_tree(int nrows, int ncols, const float* A, float* B, int opn, hipStream_t s) {
+    const long long nout = DIM == 1 ? ncols : nrows;
+    const long long nblk = (nout * 32 + BM_BLOCK - 1) / BM_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_reduce_tree<DIM>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, nrows, ncols, A, B, opn);
+    return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, float* out, int beta, hipStream_t s) {
@@ -295,7 +333,7 @@ hipError_t reduce1op(int nrows, int ncols, const float* A, float* B, float initv
     case 2: return reduce1_impl<2>(nrows, ncols, A, B, s);
     case 10: return reduce1_impl<10>(nrows, ncols, A, B, s);
     case 11: return reduce1_impl<11>(nrows, ncols, A, B, s);
-    default: return hipErrorInvalidValue;
+    default: return (opn > 0 && opn <= 14) ? reduce_tree<1>(nrows, ncols, A, B, opn, s) : hipErrorInvalidValue;
     }
 }
 
@@ -307,7 +345,7 @@ hipError_t reduce2op(int nrows, int ncols, const float* A, float* B, float initv
     case 2: return reduce2_impl<2>(nrows, ncols, A, B, s);
     case 10: return reduce2_impl<10>(nrows, ncols, A, B, s);
     case 11: return reduce2_impl<11>(nrows, ncols, A, B, s);
-    default: return hipErrorInvalidValue;
+    default: return (opn > 0 && opn <= 14) ? reduce_tree<2>(nrows, ncols, A, B, opn, s) : hipErrorInvalidValue;
     }
 }
 

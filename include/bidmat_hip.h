@@ -107,13 +107,19 @@ int bidmat_spsum(int nrows, int ncols, int nnz, const int *Air, const int *Aic, 
 
 /* Dense column reduce B[c] = op_r A[r,c] (B has ncols entries).  Replaces
  * `int reduce1op(int nrows,int ncols,float*A,float*B,float initv,int opn)`
- * (Operators.cu:735-748; CUMAT.java:111; caller GMat.scala:1186).  Supported opn:
- * ADD, MUL, MAX, MIN (the ones BIDMat's sum/prod/maxi/mini issue, GFunctions.scala:225-228);
- * any other code returns hipErrorInvalidValue. */
+ * (Operators.cu:735-748; CUMAT.java:111; caller GMat.scala:1186).  All 15 op codes.  ADD, MUL, MAX, MIN
+ * (the ones BIDMat's sum/prod/maxi/mini issue, GFunctions.scala:225-228) run bandwidth-bound kernels whose
+ * order of operations is fixed but not the reference's (they agree with it to rounding).  For every other
+ * code the order IS the result (a - b, a / b, a > b ... are not associative), so those follow the reference's
+ * kernel step by step (Operators.cu:650-671): 32 lanes per column, lane t folds rows t, t+32, ... from the
+ * left, then lanes combine pairwise at distances 1, 2, 4, ...; also for one-column inputs, where the
+ * reference's launcher (thrust, Operators.cu:718-731) handles only ADD / MAX / MIN and leaves B untouched
+ * for the rest.  nrows == 0 fills B with initv. */
 int bidmat_reduce1op(int nrows, int ncols, const float *A, float *B, float initv, int opn);
 
 /* Dense row reduce B[r] = op_c A[r,c] (B has nrows entries).  Replaces `int reduce2op(...)`
- * (Operators.cu:853-866; CUMAT.java:119; caller GMat.scala:1193). Same op set. */
+ * (Operators.cu:853-866; CUMAT.java:119; caller GMat.scala:1193).  Same op set and the same rules, along the
+ * row (Operators.cu:828-851). */
 int bidmat_reduce2op(int nrows, int ncols, const float *A, float *B, float initv, int opn);
 
 /* Elementwise C = op(A, B) with BIDMat's broadcasting (equal shapes, row/column vector on

@@ -49,6 +49,8 @@ def lib():
         L.oracle_dsum_f64.argtypes = [i, i, vp, i, vp]
         L.oracle_applyop.argtypes = [vp, vp, vp, C.c_longlong, i]
         L.oracle_applyop.restype = i
+        L.oracle_reduce_tree.argtypes = [i, i, vp, vp, C.c_float, i, i]
+        L.oracle_reduce_tree.restype = i
         L.oracle_check.argtypes = [i, i, i, vp, vp, i, vp]
         L.oracle_check.restype = i
         L.oracle_compress_inds.argtypes = [vp, i, vp, i, i]
@@ -209,6 +211,16 @@ def applyop(A, B, opn):
     out = np.empty_like(A)
     if lib().oracle_applyop(A.ctypes.data, B.ctypes.data, out.ctypes.data, A.size, opn) != 0:
         raise RuntimeError("unknown op %d" % opn)
+    return out
+
+
+def reduce_tree(A, nrows, ncols, opn, dim, initv=0.0):
+    """reduce1op (dim 1: per column) / reduce2op (dim 2: per row) with any of the 15 ops, in the order of the
+    reference's device kernels. A: column-major nrows x ncols."""
+    A = _f32(A)
+    out = np.empty(ncols if dim == 1 else nrows, dtype=np.float32)
+    if lib().oracle_reduce_tree(nrows, ncols, A.ctypes.data, out.ctypes.data, initv, opn, dim) != 0:
+        raise RuntimeError("unknown op %d or dim %d" % (opn, dim))
     return out
 
 

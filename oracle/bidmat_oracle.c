@@ -27,6 +27,8 @@
  *   oracle_check                      hand-built valid/invalid patterns (every branch)
  *   oracle_compress/uncompress_inds   np.searchsorted / np.repeat
  *   oracle_applyop                    numpy elementwise results
+ *   oracle_reduce_tree                a literal lane-by-lane simulation in Python, numpy for the associative ops,
+ *                                     closed forms for sub / div (signs follow the parity of the lane's bit count)
  * No function of this file is left "parity unpinned".
  */
 #include <stddef.h>
@@ -431,6 +433,47 @@ EXPORT int oracle_applyop(const float *A, const float *B, float *C, long long n,
         default: c = (a > 0) ? b : 0.0f; break;
         }
         C[i] = c;
+    }
+    return 0;
+}
+
+static float oracle_binop(int opn, float a, float b)
+{
+    float c;
+    oracle_applyop(&a, &b, &c, 1, opn);
+    return c;
+}
+
+/* Dense reduction with any of the 15 binary ops, in the order of the reference's device kernels
+ * (there is no CPU counterpart for ops other than sum: DenseMat.ggReduceOpv is only called with
+ * add / max / min).  __reduce1op (Operators.cu:650-671): for a column of n = nrows elements, lane t of
+ * L = min(n, 32) lanes folds x[t], x[t+32], x[t+64], ... from the left, v = op(v, next); then for
+ * i = 1, 2, 4, ... < L every lane t with t + i < L takes v[t] = op(v[t], v[t+i]) (all lanes read the
+ * values of the step before); lane 0 holds the result.  __reduce2op (Operators.cu:828-851) does the
+ * same along a row with L = min(ncols, 32) lanes striding over the columns.  dim == 1: one result per
+ * column (reduce1op), dim == 2: one per row (reduce2op).  n == 0 gives initv.  Returns -1 on an unknown op. */
+EXPORT int oracle_reduce_tree(int nrows, int ncols, const float *A, float *out, float initv, int opn, int dim)
+{
+    int nout = dim == 1 ? ncols : nrows;
+    int n = dim == 1 ? nrows : ncols;
+    int o, t, i;
+    if (opn < 0 || opn > 14 || (dim != 1 && dim != 2)) return -1;
+    for (o = 0; o < nout; o++) {
+        float v[32], w[32];
+        int L = n < 32 ? n : 32;
+        if (n == 0) { out[o] = initv; continue; }
+        for (t = 0; t < L; t++) {
+            int e;
+            for (e = t; e < n; e += 32) {
+                float x = dim == 1 ? A[(size_t)o * nrows + e] : A[(size_t)e * nrows + o];
+                v[t] = e == t ? x : oracle_binop(opn, v[t], x);
+            }
+        }
+        for (i = 1; i < L; i *= 2) {
+            for (t = 0; t < L; t++) w[t] = (t + i < L) ? oracle_binop(opn, v[t], v[t + i]) : v[t];
+            memcpy(v, w, sizeof(float) * (size_t)L);
+        }
+        out[o] = v[0];
     }
     return 0;
 }

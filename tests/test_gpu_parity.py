@@ -392,10 +392,39 @@ def test_dense_reduce(hip, shape, opn, initv):
     d.free()
 
 
-def test_dense_reduce_rejects_unsupported_op(hip):
+def test_dense_reduce_rejects_unknown_op(hip):
     d = Dev(A=np.ones(6, dtype=np.float32))
     d.zeros("c", 3)
-    assert hip.bidmat_reduce1op(2, 3, d.A.ptr, d.c.ptr, 0.0, 1) == 1     # op_sub is not a reduction
+    assert hip.bidmat_reduce1op(2, 3, d.A.ptr, d.c.ptr, 0.0, 15) == 1
+    assert hip.bidmat_reduce2op(2, 3, d.A.ptr, d.c.ptr, 0.0, -1) == 1
+    d.free()
+
+
+@pytest.mark.parametrize("shape", [(10, 20), (1, 50), (50, 1), (33, 7), (7, 33), (100, 65), (64, 1000), (2000, 3), (5, 4097)])
+@pytest.mark.parametrize("opn", [1, 3, 4, 5, 6, 7, 8, 9, 12, 13, 14])
+def test_dense_reduce_with_every_other_op_follows_the_reference_tree(hip, shape, opn):
+    """The ops that BIDMat's own reductions never issue (sub, div, the comparisons, atan2, pow, ifpos) are not
+    associative: the result is defined by the order of the reference's kernels (Operators.cu:650-671,828-851),
+    which the oracle restates. Bit for bit, except atan2 / pow (device and host libm differ in the last bit)."""
+    nrows, ncols = shape
+    rng = np.random.default_rng(70 + 31 * nrows + ncols + opn)
+    if opn in (3, 13):
+        A = (0.5 + rng.random(nrows * ncols)).astype(np.float32)           # near 1: quotients / powers stay finite
+    elif opn in (4, 5, 6, 7, 8, 9):
+        A = rng.integers(0, 3, size=nrows * ncols).astype(np.float32)       # ties happen
+    else:
+        A = rng.standard_normal(nrows * ncols).astype(np.float32)
+    d = Dev(A=A)
+    d.zeros("c", ncols), d.zeros("r", nrows)
+    hip_abi.check(hip.bidmat_reduce1op(nrows, ncols, d.A.ptr, d.c.ptr, 0.0, opn))
+    hip_abi.check(hip.bidmat_reduce2op(nrows, ncols, d.A.ptr, d.r.ptr, 0.0, opn))
+    want_c, want_r = oracle.reduce_tree(A, nrows, ncols, opn, 1), oracle.reduce_tree(A, nrows, ncols, opn, 2)
+    if opn in (12, 13):
+        np.testing.assert_allclose(d.c.numpy(), want_c, rtol=2e-5, atol=1e-6)
+        np.testing.assert_allclose(d.r.numpy(), want_r, rtol=2e-5, atol=1e-6)
+    else:
+        assert np.array_equal(d.c.numpy(), want_c, equal_nan=True), "reduce1op op %d" % opn
+        assert np.array_equal(d.r.numpy(), want_r, equal_nan=True), "reduce2op op %d" % opn
     d.free()
 
 

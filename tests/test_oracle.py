@@ -260,6 +260,60 @@ def test_applyop_matches_numpy():
         oracle.applyop(a, b, 15)
 
 
+def _lanes_reduce(x, op):
+    """The reference's reduce kernels, lane by lane (Operators.cu:650-671): lane t of L = min(n, 32) folds
+    x[t], x[t+32], ... from the left; then for i = 1, 2, 4, ... every lane t with t + i < L takes
+    op(own, value of lane t+i before the step)."""
+    n = len(x)
+    L = min(n, 32)
+    v = []
+    for t in range(L):
+        acc = x[t]
+        for e in range(t + 32, n, 32):
+            acc = op(acc, x[e])
+        v.append(acc)
+    i = 1
+    while i < L:
+        v = [op(v[t], v[t + i]) if t + i < L else v[t] for t in range(L)]
+        i *= 2
+    return v[0]
+
+
+def test_reduce_tree_against_a_lane_by_lane_simulation_and_closed_forms():
+    """oracle.reduce_tree (every op, both directions) against a literal simulation of the reference's lanes; for the
+    associative ops against numpy; for sub against its closed form: lane t's partial is x[t] - x[t+32] - ..., and
+    the tree gives lane t the sign (-1)^popcount(t) (checked in exact integer arithmetic)."""
+    rng = np.random.default_rng(91)
+    f32 = np.float32
+    ops = {0: lambda a, b: f32(a + b), 1: lambda a, b: f32(a - b), 2: lambda a, b: f32(a * b), 3: lambda a, b: f32(a / b),
+           4: lambda a, b: f32(a > b), 5: lambda a, b: f32(a < b), 6: lambda a, b: f32(a == b), 7: lambda a, b: f32(a >= b),
+           8: lambda a, b: f32(a <= b), 9: lambda a, b: f32(a != b), 10: lambda a, b: max(a, b), 11: lambda a, b: min(a, b),
+           14: lambda a, b: b if a > 0 else f32(0)}
+    for nrows, ncols in ((1, 1), (3, 5), (31, 4), (32, 3), (33, 3), (70, 2), (5, 100), (2, 64), (129, 1)):
+        A = rng.integers(-4, 5, size=nrows * ncols).astype(np.float32)
+        A[A == 0] = 1                                     # no division by zero
+        M = A.reshape(ncols, nrows).T                     # M[r, c]
+        for opn, op in ops.items():
+            got1, got2 = oracle.reduce_tree(A, nrows, ncols, opn, 1), oracle.reduce_tree(A, nrows, ncols, opn, 2)
+            want1 = np.array([_lanes_reduce(list(M[:, c]), op) for c in range(ncols)], dtype=np.float32)
+            want2 = np.array([_lanes_reduce(list(M[r, :]), op) for r in range(nrows)], dtype=np.float32)
+            assert np.array_equal(got1, want1), (nrows, ncols, opn)
+            assert np.array_equal(got2, want2), (nrows, ncols, opn)
+        # small integers: sums, maxima and minima are exact whatever the order
+        assert np.array_equal(oracle.reduce_tree(A, nrows, ncols, 0, 1), M.sum(axis=0))
+        assert np.array_equal(oracle.reduce_tree(A, nrows, ncols, 10, 2), M.max(axis=1))
+        assert np.array_equal(oracle.reduce_tree(A, nrows, ncols, 11, 1), M.min(axis=0))
+        # sub, closed form
+        L = min(nrows, 32)
+        part = np.array([[M[t, c] - M[t + 32::32, c].sum() for t in range(L)] for c in range(ncols)])
+        sign = np.array([(-1) ** bin(t).count("1") for t in range(L)])
+        assert np.array_equal(oracle.reduce_tree(A, nrows, ncols, 1, 1), (part * sign).sum(axis=1).astype(np.float32))
+    # n == 0: the initial value
+    assert np.array_equal(oracle.reduce_tree(np.zeros(0, np.float32), 0, 3, 1, 1, initv=7.0), np.full(3, 7.0, np.float32))
+    with pytest.raises(RuntimeError):
+        oracle.reduce_tree(np.ones(4, np.float32), 2, 2, 15, 1)
+
+
 def test_tolerance_rule():
     ref = np.array([1.0, 0.0, 1e-9])
     sa = np.array([1.0, 10.0, 10.0])
