@@ -459,7 +459,8 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
         sv = {"set_values_ms": round(_timed(lib, lambda: lib.bidmat_plan_set_values(plan, d_v.ptr, stream), stream, 5), 4),
               "dsmultT_ms": round(_timed(lib, lambda: lib.bidmat_dsmultT_plan(plan, k, d_AT.ptr, None, d_G.ptr, 0, stream), stream, 5), 4),
               "spsum_rows_ms": round(_timed(lib, lambda: lib.bidmat_spsum_rows_plan(plan, None, d_rs.ptr, 0, stream), stream, 5), 4),
-              "spsum_rows_fresh_values_ms": round(_timed(lib, lambda: lib.bidmat_spsum_rows_plan(plan, d_v.ptr, d_rs.ptr, 0, stream), stream, 5), 4)}
+              "spsum_rows_fresh_values_ms": round(_timed(lib, lambda: lib.bidmat_spsum_rows_csc(nrows, nnz, d_ir.ptr, d_v.ptr, d_rs.ptr, 0, stream), stream, 5), 4),
+              "spsum_rows_fresh_values_through_plan_ms": round(_timed(lib, lambda: lib.bidmat_spsum_rows_plan(plan, d_v.ptr, d_rs.ptr, 0, stream), stream, 5), 4)}
         if lib.bidmat_dsmult_plan(plan, k, d_A.ptr, None, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream) == 0:
             sv["dsmult_ms"] = round(_timed(lib, lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, None, d_ir.ptr, d_jc.ptr, d_C.ptr, 0, stream), stream, 5), 4)
         out["values_stored_in_plan"] = sv

@@ -32,10 +32,12 @@ std::atomic<int> g_cache_cols_after{2};
 std::atomic<int> g_cache_plans{4};
 std::atomic<int> g_check_plan{0};
 std::atomic<int> g_plan_builder{0};
+std::atomic<int> g_rowsum_form{0};
 std::atomic<int> g_plan_pool_mb{4096};
 }  // namespace
 int opt_plan_pool_mb() { return g_plan_pool_mb.load(std::memory_order_relaxed); }
 int opt_plan_builder() { return g_plan_builder.load(std::memory_order_relaxed); }
+int opt_rowsum_form() { return g_rowsum_form.load(std::memory_order_relaxed); }
 int opt_check_plan() { return g_check_plan.load(std::memory_order_relaxed); }
 int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
 int opt_plan_keep_mb() { return g_plan_keep_mb.load(std::memory_order_relaxed); }
@@ -419,10 +421,9 @@ API int bidmat_spsum(int nrows, int ncols, int nnz, const int* Air, const int* A
         err = bm::coo_compress_cols(ncols, nnz, Aic, jc, nullptr);
         if (err == hipSuccess) err = bm::spsum_cols(ncols, nnz, P, jc, B, 1, nullptr);
     } else {
-        PlanRef plan;
-        err = cached_plan(ncols, nnz, Air, Aic, 0, NEED_ROWS, &plan);
-        if (err == hipSuccess && plan->nrows > nrows) err = hipErrorInvalidValue;   // row index outside B
-        if (err == hipSuccess) err = run_spsum_rows(plan.get(), P, B, 1, nullptr);
+        int bad = 0;
+        err = bm::spsum_rows_exact(nrows, nnz, Air, P, B, 1, &bad, nullptr);
+        if (err == hipSuccess && bad) err = hipErrorInvalidValue;                   // row index outside B
     }
     return finish_blocking(err);
 }
@@ -661,6 +662,15 @@ API int bidmat_spsum_rows_plan(bidmat_plan* plan, const float* Sdata, float* out
     if (plan->nrows == 0) return 0;
     if (!out || (plan->nnz > 0 && !Sdata && !plan->pvals)) return kInvalid;
     return (int)run_spsum_rows(plan, Sdata, out, beta, as_stream(stream));
+}
+
+API int bidmat_spsum_rows_csc(int nrows, int nnz, const int* Sir, const float* Sdata, float* out, int beta,
+                              void* stream) {
+    auto lock = bm::device_lock();
+    if (nrows < 0 || nnz < 0 || (beta != 0 && beta != 1)) return kInvalid;
+    if (nrows == 0) return 0;
+    if (!out || (nnz > 0 && (!Sir || !Sdata))) return kInvalid;
+    return (int)bm::spsum_rows_exact(nrows, nnz, Sir, Sdata, out, beta, nullptr, as_stream(stream));
 }
 
 API int bidmat_transpose(int nrows, int ncols, const float* in, int ldi, float* out, int ldo, void* stream) {
@@ -999,6 +1009,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_plan_builder.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "rowsum_form")) {
+        if (value != 0 && value != 2) return kInvalid;
+        bm::g_rowsum_form.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "plan_pool_mb")) {
         if (value < 0 || value > (1 << 20)) return kInvalid;
         bm::g_plan_pool_mb.store((int)value);
@@ -1042,6 +1057,7 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "cache_plans")) return bm::g_cache_plans.load();
     if (!strcmp(name, "check_plan")) return bm::opt_check_plan();
     if (!strcmp(name, "plan_builder")) return bm::opt_plan_builder();
+    if (!strcmp(name, "rowsum_form")) return bm::opt_rowsum_form();
     if (!strcmp(name, "plan_pool_mb")) return bm::opt_plan_pool_mb();
     return -2;
 }

@@ -15,6 +15,7 @@ int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..6
 int opt_plan_keep_mb(); // plan-build temporaries up to this many MiB stay allocated for the next build
 int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: -1 = by k_hint (default), 0 = none
 int opt_plan_pool_mb(); // MiB of freed plan blocks kept per device for the next plans
+int opt_rowsum_form();  // bidmat_spsum_rows_csc: 0 = by the row count (default), 2 = always the hashed tables with global accumulators
 int opt_plan_builder(); // row side of a plan: 0 = per-panel counting sorts (default), 1 = one library radix sort
 int opt_check_plan();  // 1: plans keep a digest of their pattern and the plan-taking calls compare it
 int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always
@@ -126,6 +127,12 @@ hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, floa
                       hipStream_t s);
 hipError_t spsum_segments(int nseg, const int* xcd_start, const float* vals, const int* perm, const int* segstart,
                           float* partial, hipStream_t s);
+// out[r] (+)= sum of vals[j] over ir[j] == r, from the unordered (row, value) list itself: exact
+// 64-bit integer accumulation after one common scaling, so the result does not depend on the order
+// in which nonzeros arrive. If a row index lies outside [0, nrows) nothing is written; `bad_rows`
+// (optional) makes the call wait for the stream and reports that.
+hipError_t spsum_rows_exact(int nrows, long long nnz, const int* ir, const float* vals, float* out, int beta,
+                            int* bad_rows, hipStream_t s);
 hipError_t reduce1op(int nrows, int ncols, const float* A, float* B, float initv, int opn,
                      hipStream_t s);
 hipError_t reduce2op(int nrows, int ncols, const float* A, float* B, float initv, int opn,

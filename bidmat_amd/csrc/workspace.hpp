@@ -22,6 +22,8 @@ enum WsSlot {
     WS_PLAN_ROWS_A,   // bytes         temporaries of the row side of a plan build (dropped again when large)
     WS_PLAN_ROWS_B,   // bytes         likewise, the part sized by the nonzeros of light rows
     WS_TRANSPOSE,     // bytes         sort buffers of the sparse transpose
+    WS_ROWSUM,        // bytes         exact row sums: block maxima, 64-bit accumulators, flags
+    WS_ROWSUM_TABLES, // u64[...]      exact row sums: the accumulator tables of the workgroups
     WS_NSLOTS
 };
 

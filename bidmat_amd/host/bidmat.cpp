@@ -562,7 +562,7 @@ GMatP GSMat::sum(int n, GMatP oldmat) {
     Mat::nflops += nnz0;
     int err;
     if (nn == 1) err = bidmat_spsum_cols(ncols, nnz0, pdata, pjc, out->pdata, 0, nullptr);
-    else if (nn == 2) err = bidmat_spsum_rows_plan(plan(0), pdata, out->pdata, 0, nullptr);
+    else if (nn == 2) err = bidmat_spsum_rows_csc(nrows, nnz0, pir, pdata, out->pdata, 0, nullptr);
     else fail("index must 1 or 2");
     if (err == 0) err = bidmat_stream_synchronize(nullptr);
     if (err != 0) fail(std::string("HIP error in GSMat.sum ") + bidmat_error_string(err));

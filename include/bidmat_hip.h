@@ -235,12 +235,22 @@ int bidmat_dds_plan_stored(bidmat_plan *plan, int k, const float *A, const float
 /* Number of extra wave segments of the plan's long columns (0: every column fits one segment). */
 int bidmat_plan_overflow_segments(const bidmat_plan *plan);
 
-/* Sparse sums with jc / a plan: out = beta*out + sums.  Column sums need only jc;
- * row sums need a plan. */
+/* Sparse sums: out = beta*out + sums.  Column sums need only jc.  Row sums come in two forms:
+ * through a plan (the values stored in the plan, Sdata == NULL, are summed in the plan's row order
+ * at streaming speed; values passed in are gathered through the plan's permutation), or, for
+ * values that were just produced, straight from the row indices (bidmat_spsum_rows_csc: one
+ * pass over Sir and Sdata in any order, no plan, no jc).  The reference adds with float atomics in
+ * arrival order (Arith.cu:250-264), so its row sums vary from run to run; bidmat_spsum_rows_csc
+ * rounds every value once to a common step of 2^-(61 - bits of nnz) of the largest magnitude's
+ * binade and adds 64-bit integers: the same bits whatever the order, and closer to the exact sum
+ * than a float running sum.  Rows with NaN, or infinities of both signs, give NaN.  A row index
+ * outside [0, nrows) leaves `out` untouched (bidmat_spsum reports it as hipErrorInvalidValue). */
 int bidmat_spsum_cols(int ncols, int nnz, const float *Sdata, const int *Sjc, float *out,
                       int beta, void *stream);
 int bidmat_spsum_rows_plan(bidmat_plan *plan, const float *Sdata, float *out, int beta,
                            void *stream);
+int bidmat_spsum_rows_csc(int nrows, int nnz, const int *Sir, const float *Sdata, float *out,
+                          int beta, void *stream);
 
 /* jc[ncols+1] -> ic[nnz] (per-nonzero column index).  Replaces cusparseXcsr2coo at
  * GSMat.scala:639.  Enqueues on stream. */
@@ -393,6 +403,9 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "plan_builder" how the row side of a plan is put in order: 0 = stable counting sorts per column panel and by
  *              row, written for this layout (default), 1 = one library radix sort of (key, position) pairs (also
  *              taken by itself when more than 24 575 rows are cut by panels); both give the same plan, bit for bit
+ *   "rowsum_form" which kernel bidmat_spsum_rows_csc / bidmat_spsum(n = 2) take: 0 = by the number of rows (up to
+ *              262 144 rows: every workgroup owns a range of rows with all accumulators in LDS; more: hashed
+ *              tables in LDS in front of accumulators in global memory), 2 = always the latter; the same bits
  *   "plan_pool_mb" device memory of destroyed (or evicted) plans kept for the next plans, MiB per device (default
  *              4096; 0 = give every block back at once): a caller that meets a new pattern with every minibatch
  *              would otherwise pay hipMalloc + hipFree for the same sizes on every call; bidmat_release_caches frees it
