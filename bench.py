@@ -70,6 +70,8 @@ def alg_bytes(op, k, nnz, nrows, ncols):
         return nnz * (4 * k + 8) + ncols * (4 * k + 4) + 4 + (4 * nnz if op == "dds_op" else 0)
     if op == "dsmultT":
         return nnz * (4 * k + 8) + nrows * (4 * k + 4) + 4
+    if op == "fused":              # the chain as the reference runs it: DDS with the elementwise op, then A*^S
+        return alg_bytes("dds_op", k, nnz, nrows, ncols) + alg_bytes("dsmultT", k, nnz, nrows, ncols)
     if op == "ewise":              # elementwise on the nonzero values: two reads, one write
         return 12 * nnz
     if op == "rowsum":             # dense row sums of a k x ncols matrix
@@ -85,6 +87,8 @@ def compulsory_bytes(op, k, nnz, nrows, ncols):
         return 4 * k * (nrows + ncols) + 8 * nnz + 4 * (ncols + 1)
     if op == "dsmultT":            # A, values, column of each nonzero, row pointer, C
         return 4 * k * (nrows + ncols) + 8 * nnz + 4 * (nrows + 1)
+    if op == "fused":              # both dense operands, values, column of each nonzero, row pointer, G
+        return 4 * k * (2 * nrows + ncols) + 8 * nnz + 4 * (nrows + 1)
     return alg_bytes(op, k, nnz, nrows, ncols)
 
 
@@ -93,6 +97,8 @@ def flops(op, k, nnz, ncols):
     elementwise op and the reduction)."""
     if op in ("dds", "dsmult", "dsmultT", "dds_op"):
         return 2.0 * k * nnz + (nnz if op == "dds_op" else 0)
+    if op == "fused":
+        return 4.0 * k * nnz + nnz
     if op == "ewise":
         return float(nnz)
     return float(k) * ncols
@@ -122,7 +128,7 @@ def op_bounds(kind, k, nnz, nrows, ncols, l2_rate_GBps, uncacheable, heavy_nnz=N
     gathered = nnz * 4.0 * k
     if l2_rate_GBps:
         terms["l2_resident_ms"] = gathered / (l2_rate_GBps * 1e6)
-    if kind == "dsmultT":
+    if kind in ("dsmultT", "fused"):
         if heavy_nnz is not None and l2_rate_GBps:
             terms["plan_schedule_ms"] = heavy_nnz * 4.0 * k / (l2_rate_GBps * 1e6) + (nnz - heavy_nnz) * 4.0 * k / (HBM_PEAK_GBS * 1e6)
     elif uncacheable is not None:
@@ -149,6 +155,8 @@ def main():
                          "operator (the GMat / GSMat operator layer), graph (HIP-graph replay), "
                          "stored (values stored in the plan); 'none' runs the timed steps only, which keeps a profiler's "
                          "per-kernel averages clean")
+    ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE",
+                    help="library option set before anything runs (bidmat_set_option), repeatable")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain streaming kernel of known size (C = A + B on 3 x 1 GiB) "
                          "before the steps: the scale for rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
@@ -166,6 +174,9 @@ def main():
     if ndev.value < 1:
         raise RuntimeError("no HIP device visible")
     hip_abi.check(lib.bidmat_set_device(0))
+    for item in args.set:
+        oname, _, oval = item.partition("=")
+        hip_abi.check(lib.bidmat_set_option(oname.encode(), int(oval)), "set_option " + item)
 
     sections = set() if args.sections == "none" else set(args.sections.split(","))
     if args.workload == "footprint":
@@ -183,7 +194,7 @@ def main():
         for name, steps, sample in (("C1", 200, 1.0), ("C4", 10, 0.02), ("C5", 5, 0.005)):
             w = run_workload(lib, name, steps, 2, args.scale, {"probe"} & sections, not args.no_cpu, sample, False)
             out["workloads"][name] = {key: w[key] for key in ("metric", "value", "unit", "ms_per_step", "steps", "config", "ops", "roofline",
-                                                              "alg_frac_of_hbm_peak", "plan", "cpu_baseline", "verified", "rowsum")
+                                                              "alg_frac_of_hbm_peak", "plan", "cpu_baseline", "verified", "rowsum", "chain_forms")
                                       if key in w}
             hip_abi.check(lib.bidmat_release_caches())
         out["verified"] = bool(out.get("verified")) and all(w.get("verified") for w in out["workloads"].values()) \
@@ -281,18 +292,24 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
     else:  # C5: Q = V ./ DDS(W,H,V) in one launch; G = H *^ Q; rs = sum(H,2)
         d_W, d_H = up(cfg["W"]), up(cfg["H"])
         d_Q, d_G, d_rs = DeviceArray(nnz, np.float32), DeviceArray(k * nrows, np.float32), DeviceArray(k, np.float32)
-        keep += [d_W, d_H, d_Q, d_G, d_rs]
+        d_rs2 = DeviceArray(k * nrows, np.float32)
+        keep += [d_W, d_H, d_Q, d_G, d_rs, d_rs2]
         outputs = {"dds_op": d_Q, "dsmultT": d_G}
         # V, the data matrix, is the same in every iteration of the update: its values are stored in the
         # plan once (like the plan itself, outside the step) and the fused DDS streams them from there
         hip_abi.check(lib.bidmat_plan_set_values(plan, d_v.ptr, stream))
-        ops = [
-            ("dds_op", "dds_op", lambda: lib.bidmat_dds_plan_stored(plan, k, d_W.ptr, d_H.ptr, d_ir.ptr, d_jc.ptr, 3, d_Q.ptr, stream)),
-            ("dsmultT", "dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_H.ptr, d_Q.ptr, d_G.ptr, 0, stream)),
+        # One walk over the plan's rows does the whole chain: every nonzero's column of H is gathered once and serves
+        # the dot product and the accumulation; Q stays in registers (the two calls it replaces, and the variant that
+        # also writes Q, are timed beside it under `chain_forms`).
+        two_calls = [
+            ("dds_op", lambda: lib.bidmat_dds_plan_stored(plan, k, d_W.ptr, d_H.ptr, d_ir.ptr, d_jc.ptr, 3, d_Q.ptr, stream)),
+            ("dsmultT", lambda: lib.bidmat_dsmultT_plan(plan, k, d_H.ptr, d_Q.ptr, d_G.ptr, 0, stream)),
         ]
-        workload = "configs[4]: NMF update chain Q = V ./ DDS(W,H,V) (one fused launch), G = H *^ Q (dense row sums timed apart)"
-        metric = "algorithmic GB/s (gathered operand charged once per nonzero) for the NMF update chain at k=128, ~400M nnz"
-        roof_op, roof_kernel = "dsmultT", "k_gather_axpy<W=4,V=1,LPN=32,plan> + k_reduce_segments (both stages of A*^S)"
+        ops = [("dds_dsmultT", "fused",
+                lambda: lib.bidmat_dds_dsmultT_plan(plan, k, d_W.ptr, d_H.ptr, None, 3, None, d_G.ptr, 0, stream))]
+        workload = "configs[4]: NMF update chain Q = V ./ DDS(W,H,V), G = H *^ Q in one launch over the plan's rows (dense row sums timed apart)"
+        metric = "algorithmic GB/s (the chain's two gathers per nonzero charged as the reference runs them) for the NMF update chain at k=128, ~400M nnz"
+        roof_op, roof_kernel = "dds_dsmultT", "k_fused_rows<W=4,V=1,LPN=32> + k_reduce_segments"
 
     def step(marks=None):
         for i, (opname, _, fn) in enumerate(ops):
@@ -358,7 +375,7 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
     # ---- what bounds every op, measured on this device in this run: the rate of the same gather kernels
     # when the gathered rows fit in L2 (the ceiling of a kernel whose every gather is served by L2), the
     # plain streaming rate of the device, and from the pattern itself the gathers no L2 could hold.
-    heavy_nnz = lib.bidmat_plan_heavy_nnz(plan) if "dsmultT" in per_op else None
+    heavy_nnz = lib.bidmat_plan_heavy_nnz(plan) if any(o[1] in ("dsmultT", "fused") for o in ops) else None
     uncache = uncacheable_gather_bytes(ir, nrows, k) if "probe" in sections else None
     live = {}
     if "probe" in sections:
@@ -376,7 +393,8 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
     r = per_op[roof_op]
     # the dominant kernel's own launch time where the step marks it (stage 1 of A*^S), else its op's time
     r_avg = r.get("stage1_gather_ms_avg", r["ms_avg"])
-    r_bytes = alg_bytes(roof_op, k, nnz, nrows, ncols)
+    roof_kind = [o[1] for o in ops if o[0] == roof_op][0]
+    r_bytes = alg_bytes(roof_kind, k, nnz, nrows, ncols)
     if "stage1_gather_ms_avg" in r:
         # stage 1 alone: per nonzero one gathered column, its index and its value; per segment one partial sum written
         r_bytes = nnz * (4 * k + 8) + lib.bidmat_plan_segments(plan) * (4 * k + 4) + 4
@@ -389,9 +407,9 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
                       "most of them, so this can exceed 1; the bounded utilisation figure is frac_of_bound",
         "traffic": traffic, "traffic_source": traffic_src,
         "bytes_per_launch": r_bytes, "avg_launch_ms": round(r_avg, 4),
-        "compulsory_bytes": compulsory_bytes(roof_op, k, nnz, nrows, ncols), "gathered_bytes": nnz * 4 * k,
-        "uncacheable_gather_bytes": uncache if roof_op != "dsmultT" else None,
-        "heavy_row_nnz": heavy_nnz if roof_op == "dsmultT" else None,
+        "compulsory_bytes": compulsory_bytes(roof_kind, k, nnz, nrows, ncols), "gathered_bytes": nnz * 4 * k,
+        "uncacheable_gather_bytes": uncache if roof_op not in ("dsmultT", "dds_dsmultT") else None,
+        "heavy_row_nnz": heavy_nnz if roof_op in ("dsmultT", "dds_dsmultT") else None,
         "l2_resident_gather_GBps": lr["l2_resident_gather_GBps"] if lr else None, "l2_resident_probe": lr["probe"] if lr else None,
         "stream_GBps": lr["stream_GBps"] if lr else None,
         "bound_ms": r.get("bound_ms"), "frac_of_bound": round(r["bound_ms"] / r_avg, 4) if r.get("bound_ms") else None,
@@ -429,6 +447,23 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
     if "dsmultT" in per_op:
         # what a caller with a fresh pattern on every call (a BIDMach minibatch) pays for A*^S
         per_op["dsmultT_incl_plan_ms"] = round(per_op["dsmultT"]["ms_avg"] + t_plan[1] * 1e3, 4)
+    if name == "C5":
+        # the chain's other forms: the two calls the fused launch replaces, and the fused launch that also writes Q
+        forms = {n + "_ms": round(_timed(lib, f, stream, 3, warm=1), 4) for n, f in two_calls}
+        forms["two_calls_ms"] = round(forms["dds_op_ms"] + forms["dsmultT_ms"], 4)
+        g_two = d_G.numpy()
+        q_two = d_Q.numpy()
+        fq = lambda: lib.bidmat_dds_dsmultT_plan(plan, k, d_W.ptr, d_H.ptr, None, 3, d_Q.ptr, d_G.ptr, 0, stream)
+        hip_abi.check(lib.bidmat_memset(d_Q.ptr, 0, d_Q.nbytes))
+        forms["one_launch_also_writing_Q_ms"] = round(_timed(lib, fq, stream, 3, warm=1), 4)
+        forms["one_launch_same_bits_as_two_calls"] = bool(np.array_equal(g_two.view(np.uint32), d_G.numpy().view(np.uint32)) and
+                                                          np.array_equal(q_two.view(np.uint32), d_Q.numpy().view(np.uint32)))
+        del g_two, q_two
+        # the gathers alone, for scale: A*^S with the plan's stored values (V, not Q: a timing, not a result of the chain)
+        forms["dsmultT_alone_values_in_plan_order_ms"] = round(_timed(
+            lib, lambda: lib.bidmat_dsmultT_plan(plan, k, d_H.ptr, None, d_rs2.ptr, 0, stream), stream, 3, warm=1), 4)
+        out["chain_forms"] = forms
+        per_op["dds_dsmultT_incl_plan_ms"] = round(per_op["dds_dsmultT"]["ms_avg"] + t_plan[1] * 1e3, 4)
     if name == "C5":      # the dense row sums of H, timed apart from the chain
         e0, e1 = ev(), ev()
         hip_abi.check(lib.bidmat_reduce2op(k, ncols, d_H.ptr, d_rs.ptr, 0.0, 0))
@@ -496,7 +531,10 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
         out["cpu_baseline"] = cpu_baseline(name, cfg, cpu_sample)
         checks = verify_outputs(name, cfg, results)
         for opname, c in checks.items():
-            per_op[opname].update(c)
+            if opname in per_op:
+                per_op[opname].update(c)
+            else:                       # an output of a fused launch: filed under the launch
+                per_op[ops[0][0]]["check_" + opname] = c
         out["verified"] = bool(checks) and all(c["max_err_measure"] <= 1e-4 for c in checks.values())
     return out
 

@@ -33,10 +33,12 @@ std::atomic<int> g_cache_plans{4};
 std::atomic<int> g_check_plan{0};
 std::atomic<int> g_plan_builder{0};
 std::atomic<int> g_rowsum_form{0};
+std::atomic<int> g_class_shift{-1};
 std::atomic<int> g_plan_pool_mb{4096};
 }  // namespace
 int opt_plan_pool_mb() { return g_plan_pool_mb.load(std::memory_order_relaxed); }
 int opt_plan_builder() { return g_plan_builder.load(std::memory_order_relaxed); }
+int opt_class_shift() { return g_class_shift.load(std::memory_order_relaxed); }
 int opt_rowsum_form() { return g_rowsum_form.load(std::memory_order_relaxed); }
 int opt_check_plan() { return g_check_plan.load(std::memory_order_relaxed); }
 int opt_class_threads() { return g_class_threads.load(std::memory_order_relaxed); }
@@ -635,6 +637,24 @@ API int bidmat_dds_plan_stored(bidmat_plan* plan, int k, const float* A, const f
     return dds_plan_entry(plan, k, A, B, Sir, Sjc, nullptr, true, opn, P, 0, stream);
 }
 
+API int bidmat_dds_dsmultT_plan(bidmat_plan* plan, int k, const float* A, const float* B, const float* V, int opn,
+                                float* Q, float* G, int beta, void* stream) {
+    auto lock = bm::device_lock();
+    if (!plan || k < 0 || (beta != 0 && beta != 1) || opn < 0 || opn > 14) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (!(plan->sides & bm::PLAN_ROWS)) return kInvalid;
+    if (k == 0 || plan->nrows == 0) return 0;
+    if (!G || (plan->nnz > 0 && (!A || !B || (!V && !plan->pvals)))) return kInvalid;
+    hipStream_t s = as_stream(stream);
+    hipError_t err;
+    float* partial = row_partial(plan, k, s, &err);
+    if (!partial) return (int)err;
+    if ((err = bm::fused_segments(k, k, k, plan->nseg, plan->xcd_start, plan->segrow, A, B, V ? V : plan->pvals, plan->pc,
+                                  V ? plan->perm : nullptr, plan->perm, opn, plan->segstart, partial, Q, s)) != hipSuccess)
+        return (int)err;
+    return (int)bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, partial, G, beta, s);
+}
+
 API int bidmat_plan_set_values(bidmat_plan* plan, const float* Sdata, void* stream) {
     if (!plan) return kInvalid;
     auto lock = bm::device_lock();
@@ -1009,6 +1029,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_plan_builder.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "class_shift")) {
+        if (value < -1 || value > 16) return kInvalid;
+        bm::g_class_shift.store((int)value);
+        return 0;
+    }
     if (!strcmp(name, "rowsum_form")) {
         if (value != 0 && value != 2) return kInvalid;
         bm::g_rowsum_form.store((int)value);
@@ -1058,6 +1083,7 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "check_plan")) return bm::opt_check_plan();
     if (!strcmp(name, "plan_builder")) return bm::opt_plan_builder();
     if (!strcmp(name, "rowsum_form")) return bm::opt_rowsum_form();
+    if (!strcmp(name, "class_shift")) return bm::opt_class_shift();
     if (!strcmp(name, "plan_pool_mb")) return bm::opt_plan_pool_mb();
     return -2;
 }

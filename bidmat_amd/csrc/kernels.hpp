@@ -15,6 +15,7 @@ int opt_class_strip(); // columns per wave in the class-ordered DDS kernel (1..6
 int opt_plan_keep_mb(); // plan-build temporaries up to this many MiB stay allocated for the next build
 int opt_class_hot();   // hot rows per class kept in LDS by the class-ordered DDS kernel: -1 = by k_hint (default), 0 = none
 int opt_plan_pool_mb(); // MiB of freed plan blocks kept per device for the next plans
+int opt_class_shift();  // class ordering: class of row r = (r >> shift) & 7; -1 = chosen from k
 int opt_rowsum_form();  // bidmat_spsum_rows_csc: 0 = by the row count (default), 2 = always the hashed tables with global accumulators
 int opt_plan_builder(); // row side of a plan: 0 = per-panel counting sorts (default), 1 = one library radix sort
 int opt_check_plan();  // 1: plans keep a digest of their pattern and the plan-taking calls compare it
@@ -115,6 +116,13 @@ hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A
 hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, const float* A,
                               const float* vals, const int* pc, const int* perm, const int* segstart,
                               float* partial, Window cols, const int* segrow, Window rowsel, hipStream_t s);
+// Fused form: q_p = op(vals, dot(R[:, row of the segment], A[:, pc[p]])) and partial[s*k ..] = sum of q_p * A[:, pc[p]]
+// (vals through perm, or in plan order when perm == nullptr); qout (nullable) receives q_p at qperm[p] (plan order
+// when qperm == nullptr). hipErrorInvalidValue when k does not fit one pass (k > 1024, or > 256 unaligned).
+hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_start, const int* segrow,
+                          const float* R, const float* A, const float* vals, const int* pc, const int* perm,
+                          const int* qperm, int opn, const int* segstart, float* partial, float* qout,
+                          hipStream_t s);
 // C[:,r] = beta*C[:,r] + sum over q in [rowptr[r], rowptr[r+1]) of partial[rowseg[q]*k ..]
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
                            const float* partial, float* C, int beta, hipStream_t s);

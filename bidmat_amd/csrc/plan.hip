@@ -196,7 +196,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_bounds(int nseg, const unsig
 template <bool HOT>
 __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nrows, const int* __restrict__ ir,
                                                               const int* __restrict__ jc,
-                                                              const int* __restrict__ hotrank,
+                                                              const int* __restrict__ hotrank, int cshift,
                                                               int* __restrict__ cir,
                                                               int* __restrict__ cperm, int* __restrict__ cptr,
                                                               int* __restrict__ maxlen, int* __restrict__ bad) {
@@ -214,7 +214,8 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nro
         const int r = valid ? ir[j] : 0;
         if ((unsigned)r >= (unsigned)nrows) *bad = 1;           // a row outside the matrix: the build fails
         const int hr = (HOT && valid && (unsigned)r < (unsigned)nrows) ? hotrank[r] : -1;
-        const int bucket = HOT ? 2 * (r & 7) + (hr < 0 ? 1 : 0) : (r & 7);
+        const int cls = (r >> cshift) & 7;
+        const int bucket = HOT ? 2 * cls + (hr < 0 ? 1 : 0) : cls;
 #pragma unroll
         for (int x = 0; x < NB; ++x) cnt[x] += __popcll(__ballot(valid && bucket == x));
     }
@@ -240,7 +241,8 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nro
         const bool valid = j < e;
         const int r = valid ? ir[j] : 0;
         const int hr = (HOT && valid && (unsigned)r < (unsigned)nrows) ? hotrank[r] : -1;
-        const int bucket = HOT ? 2 * (r & 7) + (hr < 0 ? 1 : 0) : (r & 7);
+        const int cls = (r >> cshift) & 7;
+        const int bucket = HOT ? 2 * cls + (hr < 0 ? 1 : 0) : cls;
         int dest = -1;
 #pragma unroll
         for (int x = 0; x < NB; ++x) {
@@ -469,10 +471,10 @@ hipError_t plan_build_classes(bidmat_plan* plan, const int* ir, const int* jc, c
     if ((e = fill_i32(d_maxlen, 1, 0, s)) != hipSuccess) return e;
     const long long nblk = ((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
     if (hotrank != nullptr)
-        hipLaunchKernelGGL(k_class_partition<true>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank,
+        hipLaunchKernelGGL(k_class_partition<true>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank, plan->cshift,
                            plan->cir, plan->cperm, plan->cptr, d_maxlen, bad);
     else
-        hipLaunchKernelGGL(k_class_partition<false>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank,
+        hipLaunchKernelGGL(k_class_partition<false>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, plan->nrows, ir, jc, hotrank, plan->cshift,
                            plan->cir, plan->cperm, plan->cptr, d_maxlen, bad);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if ((e = hipMemcpy(&plan->maxlen, d_maxlen, sizeof(int), hipMemcpyDeviceToHost)) != hipSuccess) return e;
@@ -502,6 +504,7 @@ struct BuildTmp {
 hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const BuildTmp& t, hipStream_t s) {
     const int nrows = plan->nrows, ncols = plan->ncols, nnz = plan->nnz;
     const int k_hint = plan->k_hint;
+    plan->cshift = opt_class_shift() >= 0 ? opt_class_shift() : 0;
     plan->col_seglen = opt_seglen();
     {
         int* tbl = nullptr;
@@ -578,7 +581,7 @@ hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const Bui
                 std::vector<int> hotrows((size_t)(8 * hcap), -1), rows, ranks;
                 int filled[8] = {0, 0, 0, 0, 0, 0, 0, 0};
                 for (int i = 0; i < ntop; ++i) {
-                    const int r = top[i], x = r & 7;
+                    const int r = top[i], x = (r >> plan->cshift) & 7;
                     if (cnts[i] < 2 || filled[x] >= hcap) continue;      // a row used once gains nothing
                     hotrows[(size_t)x * hcap + filled[x]] = r;
                     rows.push_back(r);

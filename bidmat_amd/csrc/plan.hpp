@@ -56,6 +56,7 @@ struct bidmat_plan {
     // on XCD x only touches class-x nonzeros, so every L2 caches one eighth of the rows.
     // Built when the pattern promises a gain (plan.hip: wants_classes) or when the option says so.
     int ncls = 0;                // 0: no class ordering; otherwise 8
+    int cshift = 0;              // class of row r = (r >> cshift) & 7
     int maxlen = 0;              // longest column
     int* cir = nullptr;          // [nnz]         row of the p-th nonzero in class order
     int* cperm = nullptr;        // [nnz]         its position in the original CSC order

@@ -13,6 +13,7 @@
 // before their FMAs to keep the memory pipeline full.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "ops.hpp"
 #include "scan.hpp"
 #include "workspace.hpp"
 #include <algorithm>
@@ -45,6 +46,13 @@ struct GatherArgs {
     // CSC mode on a class-ordered pattern: the wave of column w takes the nonzeros
     // [ptr[w*pstride + poff], ptr[w*pstride + poff + pspan]) (plain CSC: 1, 0, 1)
     int pstride, poff, pspan;
+    // fused DDS + A*^S over a plan (k_fused_rows): the dense matrix whose column `row of the segment` is dotted
+    // with every gathered column, the op applied to (value, dot), where the products go (CSC order, nullable)
+    const float* R;
+    int ldr;
+    int opn;
+    float* qout;
+    const int* qperm;    // position of each product in qout (nullptr: plan order)
 };
 
 template <int V, int LPN>
@@ -259,6 +267,159 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
     }
 }
 
+// ---- DDS, the elementwise step and A*^S in one walk over a plan's segments (an NMF update's
+// G = B *^ op(V, DDS(R, B, V))): the segment's row of R stays in registers, every nonzero's column of B is
+// gathered once and serves both the dot product and the accumulation, and the products q never travel through
+// memory unless the caller asks for them. The arithmetic is that of the two kernels it replaces, step for
+// step: the dot product in the lane layout and reduction tree of the DDS kernels (dotacc over the lane's
+// vectors, butterfly over the group), the accumulation in the order of k_gather_axpy.
+template <int W, int V, int LPN, bool FULL>
+__device__ __forceinline__ float fused_chunk(const GatherArgs& a, int mycol, float myval, int rem, int g, int l,
+                                             const int (&eld)[V], const bool (&ev)[V], const Vec<W> (&rr)[V],
+                                             Vec<W> (&acc)[V]) {
+    constexpr int NG = 64 / LPN;
+    constexpr int U = Unroll<V, LPN>::U;
+    const int niter = FULL ? LPN : (rem + NG - 1) / NG;
+    float keep = 0.f;                                   // the product of the nonzero this lane loaded
+#pragma unroll 1
+    for (int it0 = 0; it0 < niter; it0 += U) {
+        Vec<W> bv[U][V];
+        float vv[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int it = it0 + u;
+            int c;
+            if constexpr (LPN == 64) {
+                c = __builtin_amdgcn_readlane(mycol, it);
+                vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myval), it));
+            } else {
+                const int src = g * LPN + it;
+                c = lane_read(mycol, src);
+                vv[u] = lane_read(myval, src);
+            }
+            ok[u] = FULL || (it * NG + g) < rem;
+            const float* bp = a.A + (size_t)c * (size_t)a.lda;
+            if (ok[u]) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) bv[u][i] = Vec<W>::load(bp + eld[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) bv[u][i] = Vec<W>::zero();
+            }
+        }
+        float qq[U];
+        if constexpr ((LPN >= 8) && (U >= 2)) {
+            // The U dot products are reduced together (group_multisum: the additions of group_allsum, shared
+            // between the lanes), which leaves the sum of slot slot_label(lane) in every lane; that lane applies
+            // the op once for its slot, and the U products are then read back from the lanes that hold them.
+            float sums[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float s = 0.f;
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    const Vec<W> x = ev[i] ? rr[i] : Vec<W>::zero();   // lanes past k contribute nothing
+                    s = x.dotacc(bv[u][i], s);
+                }
+                sums[u] = s;
+            }
+            const int label = slot_label(l) & (U - 1);
+            const float red = group_multisum<LPN, U>(sums, slot_label(l));
+            float vmine = vv[0];
+#pragma unroll
+            for (int u = 1; u < U; ++u) vmine = (label == u) ? vv[u] : vmine;
+            const bool okmine = FULL || ((it0 + label) * NG + g) < rem;
+            const float qmine = okmine ? binop_rt(a.opn, vmine, red) : 0.f;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int holder = it0 + slot_offset<U>(u, it0);        // the lane of the group that holds slot u
+                if constexpr (LPN == 64) qq[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qmine), holder));
+                else qq[u] = lane_read(qmine, g * LPN + holder);
+                keep = (l == it0 + u) ? qq[u] : keep;
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float s = 0.f;
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    const Vec<W> x = ev[i] ? rr[i] : Vec<W>::zero();   // lanes past k contribute nothing
+                    s = x.dotacc(bv[u][i], s);
+                }
+                s = group_allsum<LPN>(s);
+                qq[u] = ok[u] ? binop_rt(a.opn, vv[u], s) : 0.f;
+                keep = (l == it0 + u) ? qq[u] : keep;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i].fma(bv[u][i], qq[u]);
+        }
+    }
+    return keep;
+}
+
+template <int W, int V, int LPN>
+__global__ __launch_bounds__(BM_BLOCK) void k_fused_rows(GatherArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int g = lane / LPN, l = lane % LPN;
+    const int xcd = blockIdx.x & 7;
+    const long long wi = (long long)(blockIdx.x >> 3) * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+    const int hstart = a.xcd_start[xcd];
+    const int hcount = a.xcd_start[xcd + 1] - hstart;
+    const long long seg = wi < hcount ? hstart + wi : a.xcd_start[8] + (wi - hcount) * 8 + xcd;
+    if (seg >= a.nfirst) return;
+    const int jstart = a.ptr[seg], jend = a.ptr[seg + 1];
+    const int row = a.segrow[seg];
+    float* outp = a.out + (size_t)seg * (size_t)a.k;
+
+    int est[V], eld[V];
+    bool ev[V];
+    Vec<W> acc[V], rr[V];
+    const float* rp = a.R + (size_t)row * (size_t)a.ldr;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        est[i] = (i * LPN + l) * W;
+        ev[i] = est[i] < a.k;
+        eld[i] = ev[i] ? est[i] : 0;
+        acc[i] = Vec<W>::zero();
+        rr[i] = Vec<W>::load(rp + eld[i]);
+    }
+    const int q = l * (64 / LPN) + g;
+    int rem = jend - jstart, j0 = jstart;
+    int ccol;
+    float cval;
+    load_chunk<true>(a, j0, 0, rem, q, ccol, cval);
+    while (rem > 0) {
+        int ncol;
+        float nval;
+        load_chunk<true>(a, j0, 64, rem - 64, q, ncol, nval);
+        float keep;
+        if (rem >= 64) keep = fused_chunk<W, V, LPN, true>(a, ccol, cval, 64, g, l, eld, ev, rr, acc);
+        else keep = fused_chunk<W, V, LPN, false>(a, ccol, cval, rem, g, l, eld, ev, rr, acc);
+        if (a.qout != nullptr && q < rem) {
+            const int p = j0 + q;
+            a.qout[a.qperm != nullptr ? a.qperm[p] : p] = keep;
+        }
+        ccol = ncol;
+        cval = nval;
+        j0 += 64;
+        rem -= 64;
+    }
+#pragma unroll
+    for (int m = LPN; m < 64; m <<= 1) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] = vec_xor_add<W>(acc[i], m);
+    }
+    if (g == 0) {
+#pragma unroll
+        for (int i = 0; i < V; ++i)
+            if (ev[i]) acc[i].store(outp + est[i]);
+    }
+}
+
 // C[:,c] += sum of the overflow partials of column c, in segment order.
 __global__ __launch_bounds__(BM_BLOCK) void k_overflow_reduce(int k, int ldc, int ncols, const int* __restrict__ ovf,
                                                               const float* __restrict__ partial,
@@ -418,6 +579,7 @@ void init_args(GatherArgs& a) {
     a.segrow = nullptr; a.row_off = 0; a.row_len = 0;
     for (int x = 0; x < 9; ++x) a.xcd_start[x] = 0;
     a.pstride = 1; a.poff = 0; a.pspan = 1;
+    a.R = nullptr; a.ldr = 0; a.opn = 0; a.qout = nullptr; a.qperm = nullptr;
 }
 }  // namespace
 
@@ -525,6 +687,44 @@ hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, co
     const long long per_xcd = (long long)maxheavy + (nlight + 7) / 8;
     const long long blocks_per_xcd = (per_xcd + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
     return launch_gather<true>(sh, a, blocks_per_xcd * 8 * BM_WAVES_PER_BLOCK, s);
+}
+
+hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_start, const int* segrow,
+                          const float* R, const float* A, const float* vals, const int* pc, const int* perm,
+                          const int* qperm, int opn, const int* segstart, float* partial, float* qout,
+                          hipStream_t s) {
+    if (k <= 0 || nseg <= 0) return hipSuccess;
+    Shape sh = pick_shape(k, aligned16(A) && aligned16(R) && aligned16(partial) && lda % 4 == 0 && ldr % 4 == 0);
+    if (sh.V > 4) return hipErrorInvalidValue;          // one pass must cover k
+    GatherArgs a;
+    init_args(a);
+    a.k = k; a.lda = lda; a.ldo = k; a.nfirst = nseg; a.seglen = 0; a.beta = 0;
+    a.A = A; a.vals = vals; a.idx = pc; a.perm = perm; a.ptr = segstart; a.ovf = nullptr;
+    a.out = partial; a.partial = nullptr;
+    a.segrow = segrow;
+    a.R = R; a.ldr = ldr; a.opn = opn; a.qout = qout; a.qperm = qperm;
+    int maxheavy = 0;
+    for (int x = 0; x < 9; ++x) a.xcd_start[x] = xcd_start[x];
+    for (int x = 0; x < 8; ++x) maxheavy = std::max(maxheavy, a.xcd_start[x + 1] - a.xcd_start[x]);
+    const long long nlight = (long long)nseg - a.xcd_start[8];
+    const long long per_xcd = (long long)maxheavy + (nlight + 7) / 8;
+    const long long blocks_per_xcd = (per_xcd + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
+    const long long nblk = blocks_per_xcd * 8;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)nblk), block(BM_BLOCK);
+#define BM_CASE(W_, V_, L_)                                                              \
+    if (sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                                      \
+        hipLaunchKernelGGL((k_fused_rows<W_, V_, L_>), grid, block, 0, s, a);            \
+        return hipGetLastError();                                                        \
+    }
+#define BM_CASES(W_)                                                                     \
+    BM_CASE(W_, 1, 1) BM_CASE(W_, 1, 2) BM_CASE(W_, 1, 4) BM_CASE(W_, 1, 8) BM_CASE(W_, 1, 16) \
+    BM_CASE(W_, 1, 32) BM_CASE(W_, 1, 64) BM_CASE(W_, 2, 64) BM_CASE(W_, 4, 64)
+    BM_CASES(1)
+    BM_CASES(4)
+#undef BM_CASES
+#undef BM_CASE
+    return hipErrorInvalidValue;
 }
 
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,

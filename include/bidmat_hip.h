@@ -232,6 +232,16 @@ int bidmat_dds_plan(bidmat_plan *plan, int k, const float *A, const float *B, co
  * hipErrorInvalidValue when no values are stored. */
 int bidmat_dds_plan_stored(bidmat_plan *plan, int k, const float *A, const float *B, const int *Sir,
                            const int *Sjc, int opn, float *P, void *stream);
+/* One walk over the plan's rows for the chain Q = op(V, DDS(A, B, S)), G = beta*G + B *^ Q (the update of one
+ * factor in NMF / LDA: DDS, Arith.cu:349-389; the elementwise step, Operators.cu:86-101; A *^ S, Arith.cu:206-248;
+ * callers GSMat.scala:649-667 and GMat.scala:1082-1096).  A is k x nrows, B is k x ncols, G is k x nrows.  For
+ * every nonzero the column of B is gathered once and serves the dot product and the accumulation; Q is only
+ * written when Q != NULL (nnz values in the stored CSC order).  V == NULL: the values stored in the plan.  The
+ * results are those of bidmat_dds_plan[_stored] followed by bidmat_dsmultT_plan, bit for bit.  k must fit one pass
+ * (k <= 1024 with 16-byte aligned operands and k % 4 == 0, else k <= 256): otherwise hipErrorInvalidValue, and
+ * the two calls remain.  Needs the row side of the plan. */
+int bidmat_dds_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *B, const float *V, int opn,
+                            float *Q, float *G, int beta, void *stream);
 /* Number of extra wave segments of the plan's long columns (0: every column fits one segment). */
 int bidmat_plan_overflow_segments(const bidmat_plan *plan);
 

@@ -1,0 +1,139 @@
+"""bidmat_dds_dsmultT_plan: Q = op(V, DDS(A, B, S)) and G = B *^ Q in one walk over the plan's rows.
+
+The fused entry promises the bits of the two calls it replaces (bidmat_dds_plan with the fused elementwise
+op, then bidmat_dsmultT_plan), so the parity bar is array equality with that chain, which the other GPU
+tests hold against the oracle; one case is also checked against the oracle's float64 arbiter directly.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from bidmat_amd import hip_abi
+from util import Dev, make_plan
+
+pytestmark = pytest.mark.gpu
+
+OP_DIV = 3
+
+
+def zipf_csc(rng, nrows, ncols, mean_len, a=1.1):
+    p = 1.0 / np.arange(1, nrows + 1) ** a
+    p /= p.sum()
+    lens = rng.poisson(mean_len, size=ncols)
+    cols = []
+    for c in range(ncols):
+        cols.append(np.unique(rng.choice(nrows, size=int(lens[c]), p=p)).astype(np.int32))
+    jc = np.zeros(ncols + 1, np.int32)
+    jc[1:] = np.cumsum([x.size for x in cols])
+    ir = np.concatenate(cols) if cols else np.zeros(0, np.int32)
+    return ir.astype(np.int32), jc
+
+
+def chain(hip, plan, k, d, nnz, nrows, op, stored):
+    """The two calls: Q through the class-ordered / plain DDS with the op fused, G through the plan."""
+    d.zeros("Q1", max(nnz, 1))
+    d.zeros("G1", k * nrows)
+    if stored:
+        hip_abi.check(hip.bidmat_dds_plan_stored(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, op, d.Q1.ptr, None))
+    else:
+        hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, op, d.Q1.ptr, 0, None))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.B.ptr, d.Q1.ptr, d.G1.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    return d.Q1.numpy()[:nnz], d.G1.numpy()
+
+
+# k: a single lane group, odd, every group width, the headline's and configs[4]'s, several vectors per lane,
+# the largest that fits one pass; nrows/ncols/mean length keep every case to well under a second
+CASES = [(1, 40, 60, 8), (3, 40, 60, 8), (10, 300, 500, 20), (32, 300, 500, 20), (33, 300, 500, 20), (64, 2000, 3000, 30),
+         (100, 2000, 3000, 30), (128, 5000, 20000, 60), (256, 5000, 20000, 60), (250, 300, 500, 20), (512, 1000, 2000, 40),
+         (1024, 500, 1000, 40)]
+
+
+@pytest.mark.parametrize("k,nrows,ncols,mean_len", CASES)
+@pytest.mark.parametrize("stored", [False, True], ids=["values_passed", "values_in_plan"])
+def test_fused_chain_has_the_bits_of_the_two_calls(hip, k, nrows, ncols, mean_len, stored):
+    rng = np.random.default_rng(1000 * k + nrows)
+    ir, jc = zipf_csc(rng, nrows, ncols, mean_len)
+    nnz = ir.size
+    A = (0.01 + rng.random(k * nrows)).astype(np.float32)
+    B = (0.01 + rng.random(k * ncols)).astype(np.float32)
+    v = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+    d = Dev(A=A, B=B, v=v, ir=ir, jc=jc)
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    if stored:
+        hip_abi.check(hip.bidmat_plan_set_values(plan, d.v.ptr, None))
+    Q1, G1 = chain(hip, plan, k, d, nnz, nrows, OP_DIV, stored)
+    d.put("Q2", np.full(max(nnz, 1), -5.0, np.float32))
+    G0 = rng.standard_normal(k * nrows).astype(np.float32)
+    d.put("G2", np.zeros(k * nrows, np.float32))
+    hip_abi.check(hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, None if stored else d.v.ptr, OP_DIV, d.Q2.ptr,
+                                              d.G2.ptr, 0, None), "fused")
+    hip_abi.check(hip.bidmat_synchronize())
+    Q2, G2 = d.Q2.numpy()[:nnz], d.G2.numpy()
+    assert np.array_equal(Q2.view(np.uint32), Q1.view(np.uint32)), "Q differs in %d places" % int((Q2 != Q1).sum())
+    assert np.array_equal(G2.view(np.uint32), G1.view(np.uint32)), "G differs in %d places" % int((G2 != G1).sum())
+    # without the product output, accumulating into G
+    d.put("G3", G0)
+    hip_abi.check(hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, None if stored else d.v.ptr, OP_DIV, None,
+                                              d.G3.ptr, 1, None), "fused beta=1")
+    d.put("G4", G0)
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.B.ptr, d.Q1.ptr, d.G4.ptr, 1, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert np.array_equal(d.G3.numpy().view(np.uint32), d.G4.numpy().view(np.uint32))
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    d.free()
+
+
+def test_fused_chain_against_the_oracle(hip):
+    """Q = V ./ DDS and G = B *^ Q from the CPU restatement (oracle.dds, oracle.fsmultT), fp32 tolerance 1e-4
+    against the float64 arbiter."""
+    rng = np.random.default_rng(77)
+    k, nrows, ncols = 48, 200, 300
+    ir, jc = zipf_csc(rng, nrows, ncols, 15)
+    nnz = ir.size
+    A = (0.01 + rng.random(k * nrows)).astype(np.float32)
+    B = (0.01 + rng.random(k * ncols)).astype(np.float32)
+    v = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+    d = Dev(A=A, B=B, v=v, ir=ir, jc=jc)
+    d.zeros("Q", nnz), d.zeros("G", k * nrows)
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    hip_abi.check(hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, d.v.ptr, OP_DIV, d.Q.ptr, d.G.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    A2, B2 = A.reshape(nrows, k).astype(np.float64), B.reshape(ncols, k).astype(np.float64)
+    ic = np.repeat(np.arange(ncols), np.diff(jc))
+    dots = np.einsum("ij,ij->i", A2[ir], B2[ic])
+    q64 = v.astype(np.float64) / dots
+    assert np.allclose(d.Q.numpy(), q64, rtol=1e-4, atol=0)
+    g64 = np.zeros((nrows, k))
+    np.add.at(g64, ir, q64[:, None] * B2[ic])
+    sa = np.zeros((nrows, k))
+    np.add.at(sa, ir, np.abs(q64[:, None] * B2[ic]))
+    ok, worst = oracle.within_tolerance(d.G.numpy(), g64.ravel(), sa.ravel(), 1e-4)
+    assert ok, worst
+    # and the oracle's own fp32 chain passes the same bar
+    q32 = (v / oracle.dds(A, B, k, ir, jc)[0]).astype(np.float32)
+    assert np.allclose(q32, q64, rtol=1e-4, atol=0)
+    g32 = oracle.fsmultT(B, k, nrows, q32, ir, jc)
+    ok, worst = oracle.within_tolerance(g32, g64.ravel(), sa.ravel(), 1e-4)
+    assert ok, worst
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    d.free()
+
+
+def test_fused_chain_refuses_what_it_cannot_do(hip):
+    rng = np.random.default_rng(3)
+    nrows, ncols = 50, 80
+    ir, jc = zipf_csc(rng, nrows, ncols, 6)
+    nnz = ir.size
+    for k in (1028, 260):                       # more than one pass: aligned beyond 1024, unaligned beyond 256
+        d = Dev(A=rng.random(k * nrows).astype(np.float32), B=rng.random(k * ncols).astype(np.float32),
+                v=rng.random(nnz).astype(np.float32), ir=ir, jc=jc)
+        d.zeros("G", k * nrows)
+        plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+        off = 0 if k == 1028 else 4             # k = 260 with a misaligned B takes the scalar shape
+        rc = hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr + off, d.v.ptr, OP_DIV, None, d.G.ptr, 0, None)
+        assert rc == 1, (k, rc)
+        assert hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, d.v.ptr, 99, None, d.G.ptr, 0, None) == 1
+        assert hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, None, OP_DIV, None, d.G.ptr, 0, None) == 1  # no stored values
+        hip_abi.check(hip.bidmat_plan_destroy(plan))
+        d.free()
