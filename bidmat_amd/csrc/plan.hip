@@ -315,32 +315,63 @@ __global__ __launch_bounds__(BM_BLOCK) void k_count_bins(int nrows, const int* _
         if (lr[i]) { atomicAdd(&brows[i], lr[i]); atomicAdd(&bsum[i], ls[i]); }
     }
 }
-// out[0], out[1] = nonzeros in the n1 / n8 most frequent rows (one wave; the bins are few)
-__global__ void k_top_from_bins(const int* __restrict__ brows, const unsigned long long* __restrict__ bsum, int n1, int n8,
-                                unsigned long long* __restrict__ out) {
-    if (threadIdx.x != 0) return;
-    long long rows = 0;
-    unsigned long long sum = 0;
-    bool done1 = false;
-    out[0] = out[1] = 0;
-    for (int b = TOPBINS - 1; b >= 0; --b) {
-        const long long nr = brows[b];
-        if (nr == 0) continue;
-        const unsigned long long sb = bsum[b];
-        for (int which = done1 ? 1 : 0; which < 2; ++which) {
-            const long long want = which == 0 ? n1 : n8;
-            if (rows + nr >= want) {
-                out[which] = sum + (unsigned long long)((double)sb * (double)(want - rows) / (double)nr);
-                if (which == 0) done1 = true; else return;
-            } else {
-                break;
+// out[0], out[1] = nonzeros in the n1 / n8 most frequent rows. One workgroup: every thread takes a run of
+// bins (from the top), the runs are scanned, and the thread whose run crosses n1 (n8) rows interpolates inside
+// the bin that crosses.
+__global__ __launch_bounds__(BM_BLOCK) void k_top_from_bins(const int* __restrict__ brows,
+                                                            const unsigned long long* __restrict__ bsum, int n1, int n8,
+                                                            unsigned long long* __restrict__ out) {
+    constexpr int PER = (TOPBINS + BM_BLOCK - 1) / BM_BLOCK;
+    __shared__ long long srows[BM_BLOCK + 1];
+    __shared__ unsigned long long ssum[BM_BLOCK + 1];
+    const int t = threadIdx.x;
+    long long nr[PER];
+    unsigned long long sb[PER];
+    long long r = 0;
+    unsigned long long sm = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int b = TOPBINS - 1 - (t * PER + j);
+        nr[j] = b >= 0 ? brows[b] : 0;
+        sb[j] = b >= 0 ? bsum[b] : 0ull;
+        r += nr[j];
+        sm += sb[j];
+    }
+    srows[t] = r;
+    ssum[t] = sm;
+    if (t == 0) { out[0] = 0ull; out[1] = 0ull; }
+    __syncthreads();
+    if (t == 0) {                                   // exclusive scan of 256 pairs in LDS
+        long long ar = 0;
+        unsigned long long as = 0;
+        for (int i = 0; i < BM_BLOCK; ++i) {
+            const long long xr = srows[i];
+            const unsigned long long xs = ssum[i];
+            srows[i] = ar; ssum[i] = as;
+            ar += xr; as += xs;
+        }
+        srows[BM_BLOCK] = ar; ssum[BM_BLOCK] = as;
+    }
+    __syncthreads();
+    long long rows = srows[t];
+    unsigned long long sum = ssum[t];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        if (nr[j] > 0) {
+#pragma unroll
+            for (int which = 0; which < 2; ++which) {
+                const long long want = which == 0 ? n1 : n8;
+                if (rows < want && rows + nr[j] >= want)
+                    out[which] = sum + (unsigned long long)((double)sb[j] * (double)(want - rows) / (double)nr[j]);
             }
         }
-        rows += nr;
-        sum += sb;
+        rows += nr[j];
+        sum += sb[j];
     }
-    if (!done1) out[0] = sum;
-    out[1] = sum;
+    if (t == 0) {                                   // fewer rows than asked for: all of them
+        if (srows[BM_BLOCK] < n1) out[0] = ssum[BM_BLOCK];
+        if (srows[BM_BLOCK] < n8) out[1] = ssum[BM_BLOCK];
+    }
 }
 
 inline unsigned grid_for(long long n, int maxblocks = 16384) {
@@ -549,7 +580,7 @@ hipError_t build_cols(bidmat_plan* plan, const int* ir, const int* jc, const Bui
         PB_CHECK(fill_i32(brows, TOPBINS, 0, s));
         PB_CHECK(fill_i32(reinterpret_cast<int*>(bsum), 2 * TOPBINS, 0, s));
         hipLaunchKernelGGL(k_count_bins, dim3(grid_for(nrows, 256)), dim3(BM_BLOCK), 0, s, nrows, t.cnt, brows, bsum);
-        hipLaunchKernelGGL(k_top_from_bins, dim3(1), dim3(64), 0, s, brows, bsum, (int)(n1 < nrows ? n1 : nrows),
+        hipLaunchKernelGGL(k_top_from_bins, dim3(1), dim3(BM_BLOCK), 0, s, brows, bsum, (int)(n1 < nrows ? n1 : nrows),
                            (int)(8 * n1 < nrows ? 8 * n1 : nrows), cov);
         unsigned long long h[2] = {0, 0};
         PB_CHECK(hipMemcpy(h, cov, sizeof(h), hipMemcpyDeviceToHost));

@@ -278,7 +278,7 @@ __device__ __forceinline__ float fused_chunk(const GatherArgs& a, int mycol, flo
                                              const int (&eld)[V], const bool (&ev)[V], const Vec<W> (&rr)[V],
                                              Vec<W> (&acc)[V]) {
     constexpr int NG = 64 / LPN;
-    constexpr int U = Unroll<V, LPN>::U;
+    constexpr int U = Unroll<V, LPN>::U > 4 ? 4 : Unroll<V, LPN>::U;   // fewer registers buy a fifth wave per SIMD
     const int niter = FULL ? LPN : (rem + NG - 1) / NG;
     float keep = 0.f;                                   // the product of the nonzero this lane loaded
 #pragma unroll 1

@@ -211,6 +211,16 @@ def test_config5_nmf_step(hip):
     hip_abi.check(hip.bidmat_dds_plan(plan, k, dW.ptr, dH.ptr, dir_.ptr, djc.ptr, dv.ptr, 3, dQ2.ptr, 0, None))
     hip_abi.check(hip.bidmat_synchronize())
     assert np.array_equal(dQ2.numpy(), Q)
+    # ... and the whole chain in one walk over the plan's rows (what bench.py times for this configuration), with the
+    # stored V and with the caller's, with and without the products written: the same bits again
+    for vptr, qptr in ((None, dQ2.ptr), (dv.ptr, None)):
+        hip_abi.check(hip.bidmat_memset(dQ2.ptr, 0, dQ2.nbytes))
+        hip_abi.check(hip.bidmat_memset(dG2.ptr, 0, dG2.nbytes))
+        hip_abi.check(hip.bidmat_dds_dsmultT_plan(plan, k, dW.ptr, dH.ptr, vptr, 3, qptr, dG2.ptr, 0, None), "fused chain")
+        hip_abi.check(hip.bidmat_synchronize())
+        assert np.array_equal(dG2.numpy(), G), "bidmat_dds_dsmultT_plan differs from the two calls"
+        if qptr:
+            assert np.array_equal(dQ2.numpy(), Q)
     dQ2.free(), dG2.free()
     hip_abi.check(hip.bidmat_plan_destroy(plan))
 
