@@ -115,6 +115,16 @@ JFN(jint, spsumRowsPlan)(JNIEnv*, jclass, jlong plan, jlong Sdata, jlong out, ji
     int e = bidmat_spsum_rows_plan(P(bidmat_plan, plan), P(const float, Sdata), P(float, out), beta, nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
+JFN(jint, spsumRowsCsc)(JNIEnv*, jclass, jint nr, jint nnz, jlong Sir, jlong Sdata, jlong out, jint beta) {
+    int e = bidmat_spsum_rows_csc(nr, nnz, P(const int, Sir), P(const float, Sdata), P(float, out), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
+// Q = op(V, DDS(A, B, S)), G = beta*G + B *^ Q in one launch (V == 0: the values stored in the plan; Q == 0: not written)
+JFN(jint, ddsDsmultTPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong B, jlong V, jint opn, jlong Q, jlong G, jint beta) {
+    int e = bidmat_dds_dsmultT_plan(P(bidmat_plan, plan), k, P(const float, A), P(const float, B), P(const float, V), opn,
+                                    P(float, Q), P(float, G), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
 // S^T * A and S * A (replace the cusparseScsrmm calls of GSMat.SDTMult / SDMult, GSMat.scala:265-313)
 JFN(jint, sdtmultCsc)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jint p, jlong Sdata, jlong Sir, jlong Sjc, jlong A,
                       jint lda, jlong C, jint ldc) {
