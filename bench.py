@@ -43,9 +43,9 @@ HBM_PEAK_GBS = 8000.0
 # was taken on; it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dsmultT", 100003320): (31.6e9, "bidmat_amd/csrc/spmm.hip", "6cfa72e2052c477a",
+    ("headline", "dsmultT", 100003320): (31.6e9, "bidmat_amd/csrc/spmm.hip", "07b900239e5e9173",
                                          "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "6cfa72e2052c477a",
+    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "07b900239e5e9173",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 
@@ -149,11 +149,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs (baseline timing and verification)")
     ap.add_argument("--cpu-sample", type=float, default=1.0,
                     help="fraction of the columns timed on the CPU (1.0 = the whole workload)")
-    ap.add_argument("--sections", default="probe,shaped,operator,graph,stored",
+    ap.add_argument("--sections", default="probe,shaped,operator,graph,stored,chains",
                     help="side measurements around the timed steps, comma-separated: probe (L2-resident and streaming "
                          "rates for the bounded roofline), shaped (reference-shaped entries, repeated and fresh patterns), "
                          "operator (the GMat / GSMat operator layer), graph (HIP-graph replay), "
-                         "stored (values stored in the plan); 'none' runs the timed steps only, which keeps a profiler's "
+                         "stored (values stored in the plan), chains (the LDA / NMF factor updates as two calls and as one launch); 'none' runs the timed steps only, which keeps a profiler's "
                          "per-kernel averages clean")
     ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE",
                     help="library option set before anything runs (bidmat_set_option), repeatable")
@@ -485,6 +485,26 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
                                                                d_P, d_C, d_G)
     if name == "headline" and "operator" in sections:
         out["operator_api_ms"] = operator_layer(cfg)
+
+    if name == "headline" and "chains" in sections:
+        # The two factor updates of an LDA / NMF step on this pattern, each as the two calls the reference's
+        # operators make (DDS with the elementwise op fused, then the product) and as one launch that gathers once:
+        # E-step Q = V ./ DDS(A,B,S), C = A * Q (by columns); M-step G = B *^ Q (by the plan's rows).
+        d_Q2, d_C2, d_G2 = DeviceArray(nnz, np.float32), DeviceArray(k * ncols, np.float32), DeviceArray(k * nrows, np.float32)
+        ch = {}
+        ch["e_step_dds_op_ms"] = round(_timed(lib, lambda: lib.bidmat_dds_plan(plan, k, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_v.ptr, 3, d_Q2.ptr, 0, stream), stream, 5), 4)
+        ch["e_step_dsmult_ms"] = round(_timed(lib, lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, d_Q2.ptr, d_ir.ptr, d_jc.ptr, d_C2.ptr, 0, stream), stream, 5), 4)
+        ch["e_step_two_calls_ms"] = round(ch["e_step_dds_op_ms"] + ch["e_step_dsmult_ms"], 4)
+        ch["e_step_one_launch_ms"] = round(_timed(lib, lambda: lib.bidmat_dds_dsmult_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_v.ptr, 3, None, d_C2.ptr, 0, stream), stream, 5), 4)
+        ch["m_step_dsmultT_ms"] = round(_timed(lib, lambda: lib.bidmat_dsmultT_plan(plan, k, d_B.ptr, d_Q2.ptr, d_G2.ptr, 0, stream), stream, 5), 4)
+        ch["m_step_two_calls_ms"] = round(ch["e_step_dds_op_ms"] + ch["m_step_dsmultT_ms"], 4)
+        g_two = d_G2.numpy()
+        ch["m_step_one_launch_ms"] = round(_timed(lib, lambda: lib.bidmat_dds_dsmultT_plan(plan, k, d_A.ptr, d_B.ptr, d_v.ptr, 3, None, d_G2.ptr, 0, stream), stream, 5), 4)
+        ch["m_step_one_launch_same_bits_as_two_calls"] = bool(np.array_equal(g_two.view(np.uint32), d_G2.numpy().view(np.uint32)))
+        del g_two
+        for d in (d_Q2, d_C2, d_G2):
+            d.free()
+        out["chain_forms"] = ch
 
     if name == "headline" and "stored" in sections:
         # Callers whose values stay fixed over several calls (the data matrix of an LDA minibatch) can

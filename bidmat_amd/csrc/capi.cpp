@@ -499,6 +499,16 @@ API int bidmat_dds_csc_op(int k, int ncols, int nnz, const float* A, const float
     return (int)bm::dds_csc(k, ncols, nnz, A, B, Sir, Sjc, P, 0, as_stream(stream), V, opn);
 }
 
+API int bidmat_dds_dsmult_csc(int k, int ncols, int nnz, const float* A, const float* B, const int* Sir, const int* Sjc,
+                              const float* V, int opn, float* Q, float* C, int beta, void* stream) {
+    auto lock = bm::device_lock();
+    if (k < 0 || ncols < 0 || nnz < 0 || opn < 0 || opn > 14 || (beta != 0 && beta != 1)) return kInvalid;
+    if (k == 0 || ncols == 0) return 0;
+    if (!Sjc || !C || !A || !B || (nnz > 0 && (!Sir || !V))) return kInvalid;
+    if (Q && V != Q && ranges_overlap(V, Q, nnz)) return kInvalid;      // in place (Q == V) or apart
+    return (int)bm::fused_columns(k, ncols, nnz, A, B, V, Sir, Sjc, opn, Q, C, beta, as_stream(stream));
+}
+
 API int bidmat_dds0(int nrows, int ncols, const float* A, const float* B, const int* Cir, const int* Cjc,
                     float* P) {
     auto lock = bm::device_lock();

@@ -125,6 +125,13 @@ JFN(jint, ddsDsmultTPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong B,
                                     P(float, Q), P(float, G), beta, nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
+// Q = op(V, DDS(A, B, S)), C = beta*C + A * Q in one launch (Q == 0: not written; Q == V: in place)
+JFN(jint, ddsDsmultCsc)(JNIEnv*, jclass, jint k, jint nc, jint nnz, jlong A, jlong B, jlong Sir, jlong Sjc, jlong V, jint opn,
+                        jlong Q, jlong C, jint beta) {
+    int e = bidmat_dds_dsmult_csc(k, nc, nnz, P(const float, A), P(const float, B), P(const int, Sir), P(const int, Sjc),
+                                  P(const float, V), opn, P(float, Q), P(float, C), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
 // S^T * A and S * A (replace the cusparseScsrmm calls of GSMat.SDTMult / SDMult, GSMat.scala:265-313)
 JFN(jint, sdtmultCsc)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jint p, jlong Sdata, jlong Sir, jlong Sjc, jlong A,
                       jint lda, jlong C, jint ldc) {

@@ -123,6 +123,10 @@ hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_star
                           const float* R, const float* A, const float* vals, const int* pc, const int* perm,
                           const int* qperm, int opn, const int* segstart, float* partial, float* qout,
                           hipStream_t s);
+// The chain by columns: Q[j] = op(vals[j], dot(A[:, ir[j]], B[:, c])) (nullable output) and C[:, c] = beta*C[:, c] + sum of
+// Q[j] * A[:, ir[j]]; segments and order of additions of dsmult_csc. hipErrorInvalidValue when k does not fit one pass.
+hipError_t fused_columns(int k, int ncols, int nnz, const float* A, const float* B, const float* vals, const int* ir,
+                         const int* jc, int opn, float* Q, float* C, int beta, hipStream_t s, const ColTable* tab = nullptr);
 // C[:,r] = beta*C[:,r] + sum over q in [rowptr[r], rowptr[r+1]) of partial[rowseg[q]*k ..]
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
                            const float* partial, float* C, int beta, hipStream_t s);

@@ -420,6 +420,99 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fused_rows(GatherArgs a) {
     }
 }
 
+// The same chain by columns (an LDA E-step: Q = op(V, DDS(A, B, S)), C = beta*C + A * Q): the column of B
+// stays in registers, every nonzero's column of A is gathered once for the dot product and the accumulation.
+// Segments, overflow partials and the order of the additions are those of k_gather_axpy<..., false>; the dot
+// products are those of the DDS kernels. a.R = B (column stride a.ldr), a.A = A.
+template <int W, int V, int LPN>
+__global__ __launch_bounds__(BM_BLOCK) void k_fused_cols(GatherArgs a) {
+    const int lane = threadIdx.x & 63;
+    const long long w = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+    const int g = lane / LPN, l = lane % LPN;
+    int jstart, jend, col;
+    float* outp;
+    bool accumulate;
+    if (w < a.nfirst) {
+        const int s = a.ptr[w], e = a.ptr[w + 1];
+        col = (int)w;
+        jstart = s;
+        jend = (e - s > a.seglen) ? s + a.seglen : e;
+        outp = a.out + (size_t)w * (size_t)a.ldo;
+        accumulate = a.beta != 0;
+    } else {
+        if (a.ovf == nullptr) return;
+        const long long x = w - a.nfirst;
+        if (x >= a.ovf[a.nfirst]) return;
+        int lo = 0, hi = a.nfirst;       // ovf[lo] <= x < ovf[hi]
+        while (hi - lo > 1) {
+            const int mid = (int)(((long long)lo + hi) >> 1);
+            if (a.ovf[mid] <= x) lo = mid; else hi = mid;
+        }
+        const long long qseg = x - a.ovf[lo] + 1;
+        const long long s = (long long)a.ptr[lo] + qseg * a.seglen;
+        const long long e = a.ptr[lo + 1];
+        col = lo;
+        jstart = (int)s;
+        jend = (int)((e - s > a.seglen) ? s + a.seglen : e);
+        outp = a.partial + (size_t)x * (size_t)a.k;
+        accumulate = false;
+    }
+    int est[V], eld[V];
+    bool ev[V];
+    Vec<W> acc[V], rr[V];
+    const float* rp = a.R + (size_t)col * (size_t)a.ldr;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        est[i] = (i * LPN + l) * W;
+        ev[i] = est[i] < a.k;
+        eld[i] = ev[i] ? est[i] : 0;
+        acc[i] = Vec<W>::zero();
+        rr[i] = Vec<W>::load(rp + eld[i]);
+    }
+    constexpr bool EARLY_ADDEND = V <= 2;            // as in k_gather_axpy
+    Vec<W> addend[V];
+    if constexpr (EARLY_ADDEND) {
+#pragma unroll
+        for (int i = 0; i < V; ++i)
+            addend[i] = (accumulate && g == 0 && ev[i]) ? Vec<W>::load(outp + est[i]) : Vec<W>::zero();
+    }
+    const int q = l * (64 / LPN) + g;
+    int rem = jend - jstart, j0 = jstart;
+    int crow;
+    float cval;
+    load_chunk<false>(a, j0, 0, rem, q, crow, cval);
+    while (rem > 0) {
+        int nrow;
+        float nval;
+        load_chunk<false>(a, j0, 64, rem - 64, q, nrow, nval);
+        float keep;
+        if (rem >= 64) keep = fused_chunk<W, V, LPN, true>(a, crow, cval, 64, g, l, eld, ev, rr, acc);
+        else keep = fused_chunk<W, V, LPN, false>(a, crow, cval, rem, g, l, eld, ev, rr, acc);
+        if (a.qout != nullptr && q < rem) a.qout[j0 + q] = keep;
+        crow = nrow;
+        cval = nval;
+        j0 += 64;
+        rem -= 64;
+    }
+#pragma unroll
+    for (int m = LPN; m < 64; m <<= 1) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] = vec_xor_add<W>(acc[i], m);
+    }
+    if (g == 0) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            if (ev[i]) {
+                float* o = outp + est[i];
+                Vec<W> r = acc[i];
+                if constexpr (EARLY_ADDEND) r.add(addend[i]);
+                else if (accumulate) r.add(Vec<W>::load(o));
+                r.store(o);
+            }
+        }
+    }
+}
+
 // C[:,c] += sum of the overflow partials of column c, in segment order.
 __global__ __launch_bounds__(BM_BLOCK) void k_overflow_reduce(int k, int ldc, int ncols, const int* __restrict__ ovf,
                                                               const float* __restrict__ partial,
@@ -725,6 +818,65 @@ hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_star
 #undef BM_CASES
 #undef BM_CASE
     return hipErrorInvalidValue;
+}
+
+hipError_t fused_columns(int k, int ncols, int nnz, const float* A, const float* B, const float* vals, const int* ir,
+                         const int* jc, int opn, float* Q, float* C, int beta, hipStream_t s, const ColTable* tab) {
+    if (k <= 0 || ncols <= 0) return hipSuccess;
+    int seglen = opt_seglen();
+    int* ovf = nullptr;
+    float* partial = nullptr;
+    long long novf_max = 0;
+    hipError_t err;
+    if (tab) {
+        seglen = tab->seglen;
+        if (tab->novf > 0) {
+            ovf = const_cast<int*>(tab->ovf);
+            novf_max = tab->novf;
+        }
+    } else {
+        err = build_overflow_table(ncols, nnz, jc, seglen, &ovf, s);
+        if (err != hipSuccess) return err;
+        if (ovf) novf_max = nnz / seglen;
+    }
+    if (ovf) {
+        partial = (float*)ws_get(WS_PARTIAL, sizeof(float) * (size_t)novf_max * (size_t)k, &err, s);
+        if (!partial) return err;
+    }
+    const bool al = aligned16(A) && aligned16(B) && aligned16(C) && aligned16(partial);
+    Shape sh = pick_shape(k, al);
+    if (sh.V > 4) return hipErrorInvalidValue;          // one pass must cover k
+    GatherArgs a;
+    init_args(a);
+    a.k = k; a.lda = k; a.ldo = k; a.nfirst = ncols; a.seglen = seglen; a.beta = beta;
+    a.A = A; a.vals = vals; a.idx = ir; a.perm = nullptr; a.ptr = jc; a.ovf = ovf;
+    a.out = C; a.partial = partial;
+    a.R = B; a.ldr = k; a.opn = opn; a.qout = Q;
+    const long long nwaves = (long long)ncols + novf_max;
+    const long long nblk = (nwaves + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)nblk), block(BM_BLOCK);
+    bool launched = false;
+#define BM_CASE(W_, V_, L_)                                                              \
+    if (!launched && sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                         \
+        hipLaunchKernelGGL((k_fused_cols<W_, V_, L_>), grid, block, 0, s, a);            \
+        launched = true;                                                                 \
+    }
+#define BM_CASES(W_)                                                                     \
+    BM_CASE(W_, 1, 1) BM_CASE(W_, 1, 2) BM_CASE(W_, 1, 4) BM_CASE(W_, 1, 8) BM_CASE(W_, 1, 16) \
+    BM_CASE(W_, 1, 32) BM_CASE(W_, 1, 64) BM_CASE(W_, 2, 64) BM_CASE(W_, 4, 64)
+    BM_CASES(1)
+    BM_CASES(4)
+#undef BM_CASES
+#undef BM_CASE
+    if (!launched) return hipErrorInvalidValue;
+    if ((err = hipGetLastError()) != hipSuccess) return err;
+    if (ovf) {
+        unsigned rblk = (unsigned)(((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK);
+        hipLaunchKernelGGL(k_overflow_reduce, dim3(rblk), dim3(BM_BLOCK), 0, s, k, k, ncols, ovf, partial, C);
+        err = hipGetLastError();
+    }
+    return err;
 }
 
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,

@@ -242,6 +242,15 @@ int bidmat_dds_plan_stored(bidmat_plan *plan, int k, const float *A, const float
  * the two calls remain.  Needs the row side of the plan. */
 int bidmat_dds_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *B, const float *V, int opn,
                             float *Q, float *G, int beta, void *stream);
+/* The same chain by columns, Q = op(V, DDS(A, B, S)) and C = beta*C + A * Q (the E-step of an LDA / NMF update, where the
+ * matrix that is dotted against is also the one that is multiplied: DDS, Arith.cu:349-389; the elementwise step,
+ * Operators.cu:86-101; A * S, Arith.cu:16-60; callers GSMat.scala:649-667 and GMat.scala:1041-1074).  A is k x nrows,
+ * B and C are k x ncols.  Every nonzero's column of A is gathered once for the dot product and the accumulation; Q (nnz
+ * values in stored order) is only written when Q != NULL and may be V itself.  The results are those of
+ * bidmat_dds_csc_op followed by bidmat_dsmult_csc, bit for bit.  k must fit one pass (k <= 1024 with 16-byte aligned
+ * operands and k % 4 == 0, else k <= 256): otherwise hipErrorInvalidValue, and the two calls remain. */
+int bidmat_dds_dsmult_csc(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir, const int *Sjc,
+                          const float *V, int opn, float *Q, float *C, int beta, void *stream);
 /* Number of extra wave segments of the plan's long columns (0: every column fits one segment). */
 int bidmat_plan_overflow_segments(const bidmat_plan *plan);
 

@@ -137,3 +137,81 @@ def test_fused_chain_refuses_what_it_cannot_do(hip):
         assert hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, None, OP_DIV, None, d.G.ptr, 0, None) == 1  # no stored values
         hip_abi.check(hip.bidmat_plan_destroy(plan))
         d.free()
+
+
+# ------------------------------------------------------------------ the chain by columns
+COL_CASES = [(1, 40, 60, 8), (3, 40, 60, 8), (10, 300, 500, 20), (32, 300, 500, 20), (33, 300, 500, 20), (64, 2000, 3000, 30),
+             (100, 2000, 3000, 30), (128, 5000, 20000, 60), (256, 5000, 20000, 60), (250, 300, 500, 20), (512, 1000, 2000, 40),
+             (1024, 500, 1000, 40)]
+
+
+@pytest.mark.parametrize("k,nrows,ncols,mean_len", COL_CASES)
+@pytest.mark.parametrize("seglen", [1024, 64], ids=["whole_columns", "columns_cut_into_segments"])
+def test_column_chain_has_the_bits_of_the_two_calls(hip, k, nrows, ncols, mean_len, seglen):
+    """bidmat_dds_dsmult_csc against bidmat_dds_csc_op + bidmat_dsmult_csc; seglen = 64 cuts every longer column into
+    overflow segments with partial sums."""
+    rng = np.random.default_rng(2000 * k + nrows)
+    ir, jc = zipf_csc(rng, nrows, ncols, mean_len * (4 if seglen == 64 else 1))
+    nnz = ir.size
+    A = (0.01 + rng.random(k * nrows)).astype(np.float32)
+    B = (0.01 + rng.random(k * ncols)).astype(np.float32)
+    v = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+    C0 = rng.standard_normal(k * ncols).astype(np.float32)
+    old = hip.bidmat_get_option(b"seglen")
+    hip_abi.check(hip.bidmat_set_option(b"seglen", seglen))
+    try:
+        for beta in (0, 1):
+            d = Dev(A=A, B=B, v=v, ir=ir, jc=jc, C1=C0, C2=C0)
+            d.zeros("Q1", max(nnz, 1))
+            d.put("Q2", np.full(max(nnz, 1), -5.0, np.float32))
+            hip_abi.check(hip.bidmat_dds_csc_op(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.Q1.ptr, None))
+            hip_abi.check(hip.bidmat_dsmult_csc(k, ncols, nnz, d.A.ptr, d.Q1.ptr, d.ir.ptr, d.jc.ptr, d.C1.ptr, beta, None))
+            hip_abi.check(hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV,
+                                                    d.Q2.ptr, d.C2.ptr, beta, None), "column chain")
+            hip_abi.check(hip.bidmat_synchronize())
+            assert np.array_equal(d.Q2.numpy()[:nnz].view(np.uint32), d.Q1.numpy()[:nnz].view(np.uint32))
+            assert np.array_equal(d.C2.numpy().view(np.uint32), d.C1.numpy().view(np.uint32)), "beta %d" % beta
+            # without the products, and in place (Q == V)
+            d.put("C3", C0)
+            hip_abi.check(hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV,
+                                                    None, d.C3.ptr, beta, None))
+            hip_abi.check(hip.bidmat_synchronize())
+            assert np.array_equal(d.C3.numpy().view(np.uint32), d.C1.numpy().view(np.uint32))
+            d.put("C4", C0)
+            hip_abi.check(hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV,
+                                                    d.v.ptr, d.C4.ptr, beta, None))
+            hip_abi.check(hip.bidmat_synchronize())
+            assert np.array_equal(d.C4.numpy().view(np.uint32), d.C1.numpy().view(np.uint32))
+            assert np.array_equal(d.v.numpy()[:nnz].view(np.uint32), d.Q1.numpy()[:nnz].view(np.uint32))
+            d.free()
+    finally:
+        hip_abi.check(hip.bidmat_set_option(b"seglen", old))
+
+
+def test_column_chain_against_the_oracle_and_refusals(hip):
+    rng = np.random.default_rng(78)
+    k, nrows, ncols = 48, 200, 300
+    ir, jc = zipf_csc(rng, nrows, ncols, 15)
+    nnz = ir.size
+    A = (0.01 + rng.random(k * nrows)).astype(np.float32)
+    B = (0.01 + rng.random(k * ncols)).astype(np.float32)
+    v = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+    d = Dev(A=A, B=B, v=v, ir=ir, jc=jc)
+    d.zeros("Q", nnz), d.zeros("C", k * ncols)
+    hip_abi.check(hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.Q.ptr, d.C.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    q32 = (v / oracle.dds(A, B, k, ir, jc)[0]).astype(np.float32)
+    assert np.allclose(d.Q.numpy(), q32, rtol=2e-5, atol=0)
+    ref64, sa = oracle.fsmult_f64(A, k, q32, ir, jc)
+    ok, worst = oracle.within_tolerance(d.C.numpy(), ref64, sa, 1e-4)
+    assert ok, worst
+    # refusals: an op code outside the table, products that overlap the values at another offset, k beyond one pass
+    assert hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, 15, None, d.C.ptr, 0, None) == 1
+    assert hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.v.ptr + 4, d.C.ptr, 0, None) == 1
+    assert hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, None, d.C.ptr, 2, None) == 1
+    d.free()
+    k = 1028
+    d = Dev(A=rng.random(k * nrows).astype(np.float32), B=rng.random(k * ncols).astype(np.float32), v=v, ir=ir, jc=jc)
+    d.zeros("C", k * ncols)
+    assert hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, None, d.C.ptr, 0, None) == 1
+    d.free()
