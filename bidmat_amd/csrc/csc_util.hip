@@ -45,18 +45,31 @@ __global__ __launch_bounds__(BM_BLOCK) void k_csc_validate(int nrows, int ncols,
     if (bad) atomicOr(flags, bad);
 }
 
-// Thread j fills jc for every column that starts at position j:
-// columns ic[j-1]+1 .. ic[j] (with ic[-1] = -1 and ic[nnz] = ncols).
+// Position j closes the columns ic[j-1]+1 .. ic[j] (with ic[-1] = -1 and ic[nnz] = ncols): jc[c] = j for
+// each of them. A thread takes four consecutive positions (one 128-bit load when ic is 16-byte aligned).
 __global__ __launch_bounds__(BM_BLOCK) void k_compress_cols(int ncols, int nnz, const int* __restrict__ ic,
                                                             int* __restrict__ jc) {
-    const long long j = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    if (j > nnz) return;
-    int prev = (j == 0) ? -1 : ic[j - 1];
-    int cur = (j == nnz) ? ncols : ic[j];
-    if (prev >= ncols) prev = ncols - 1;      // malformed input: stay inside jc
-    if (prev < -1) prev = -1;
-    if (cur > ncols) cur = ncols;
-    for (int c = prev + 1; c <= cur; ++c) jc[c] = (int)j;
+    const long long j0 = 4 * ((long long)blockIdx.x * BM_BLOCK + threadIdx.x);
+    if (j0 > nnz) return;
+    int v[5];
+    v[0] = (j0 == 0) ? -1 : ic[j0 - 1];
+    if (j0 + 4 <= nnz && (reinterpret_cast<uintptr_t>(ic) & 15) == 0) {
+        const int4 q = *reinterpret_cast<const int4*>(ic + j0);
+        v[1] = q.x; v[2] = q.y; v[3] = q.z; v[4] = q.w;
+    } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u + 1] = j0 + u < nnz ? ic[j0 + u] : ncols;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const long long j = j0 + u;
+        if (j > nnz) break;
+        int prev = v[u], cur = (j == nnz) ? ncols : v[u + 1];
+        if (prev >= ncols) prev = ncols - 1;      // malformed input: stay inside jc
+        if (prev < -1) prev = -1;
+        if (cur > ncols) cur = ncols;
+        for (int c = prev + 1; c <= cur; ++c) jc[c] = (int)j;
+    }
 }
 
 template <typename T>
@@ -316,7 +329,7 @@ hipError_t csc_validate(int nrows, int ncols, int nnz, const int* ir, const int*
 
 hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStream_t s) {
     if (ncols < 0 || nnz < 0) return hipErrorInvalidValue;
-    long long nblk = ((long long)nnz + 1 + BM_BLOCK - 1) / BM_BLOCK;
+    long long nblk = ((long long)nnz / 4 + 1 + BM_BLOCK - 1) / BM_BLOCK;
     hipLaunchKernelGGL(k_compress_cols, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nnz, ic, jc);
     return hipGetLastError();
 }

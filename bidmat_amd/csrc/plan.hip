@@ -205,6 +205,81 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nro
     const long long c = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
     if (c >= ncols) return;
     const int s = jc[c], e = jc[c + 1];
+    const unsigned long long below = (1ULL << lane) - 1ULL;
+    if (e - s <= 4 * 64) {
+        // The usual column: all its row indices are requested at once and stay in registers, so the wave waits
+        // for memory once (twice with hot rows) instead of once per 64 nonzeros and per pass.
+        int r[4], hr[4], bucket[4];
+        bool valid[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = s + u * 64 + lane;
+            valid[u] = j < e;
+            r[u] = valid[u] ? ir[j] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if ((unsigned)r[u] >= (unsigned)nrows) *bad = 1;
+            hr[u] = (HOT && valid[u] && (unsigned)r[u] < (unsigned)nrows) ? hotrank[r[u]] : -1;
+        }
+        // Bucket numbers are NBITS bits wide: one ballot per bit and chunk; every bucket's lanes then follow from
+        // the ballots by scalar mask arithmetic (counts), and a lane finds the lanes before it in its own bucket
+        // by selecting each ballot or its complement.
+        constexpr int NBITS = HOT ? 4 : 3;
+        unsigned long long vm[4], bm[4][NBITS];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int cls = (r[u] >> cshift) & 7;
+            bucket[u] = HOT ? 2 * cls + (hr[u] < 0 ? 1 : 0) : cls;
+            vm[u] = __ballot(valid[u]);
+#pragma unroll
+            for (int b = 0; b < NBITS; ++b) bm[u][b] = __ballot(valid[u] && ((bucket[u] >> b) & 1));
+        }
+        int cntx[4][NB];                               // lanes of chunk u in bucket x (wave-uniform)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int x = 0; x < NB; ++x) {
+                unsigned long long m = vm[u];
+#pragma unroll
+                for (int b = 0; b < NBITS; ++b) m &= ((x >> b) & 1) ? bm[u][b] : ~bm[u][b];
+                cntx[u][x] = __popcll(m);
+            }
+        }
+        int base[NB], run = 0;
+#pragma unroll
+        for (int x = 0; x < NB; ++x) {
+            base[x] = run;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) run += cntx[u][x];
+        }
+        if (lane < 16) {
+            const int which = HOT ? lane : lane >> 1;
+            int bb = 0;
+#pragma unroll
+            for (int x = 0; x < NB; ++x) bb = (which == x) ? base[x] : bb;
+            cptr[c * 16 + lane] = s + bb;
+        }
+        if (c == ncols - 1 && lane == 0) cptr[(long long)ncols * 16] = e;
+        if (lane == 0 && e - s > __hip_atomic_load(maxlen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(maxlen, e - s);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            unsigned long long peers = vm[u];
+            int mybase = 0;
+#pragma unroll
+            for (int b = 0; b < NBITS; ++b) peers &= ((bucket[u] >> b) & 1) ? bm[u][b] : ~bm[u][b];
+#pragma unroll
+            for (int x = 0; x < NB; ++x) mybase = (bucket[u] == x) ? base[x] : mybase;
+            if (valid[u]) {
+                const int dest = s + mybase + __popcll(peers & below);
+                cir[dest] = hr[u] < 0 ? r[u] : hr[u];
+                cperm[dest] = s + u * 64 + lane;
+            }
+#pragma unroll
+            for (int x = 0; x < NB; ++x) base[x] += cntx[u][x];
+        }
+        return;
+    }
     int cnt[NB];
 #pragma unroll
     for (int x = 0; x < NB; ++x) cnt[x] = 0;
@@ -235,7 +310,6 @@ __global__ __launch_bounds__(BM_BLOCK) void k_class_partition(int ncols, int nro
     // every column would hit the same address: only columns longer than the longest seen so far do
     // (the plain read may be stale, which only costs a redundant atomic)
     if (lane == 0 && e - s > __hip_atomic_load(maxlen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(maxlen, e - s);
-    const unsigned long long below = (1ULL << lane) - 1ULL;
     for (int j0 = s; j0 < e; j0 += 64) {
         const int j = j0 + lane;
         const bool valid = j < e;

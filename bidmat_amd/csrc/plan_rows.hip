@@ -543,18 +543,32 @@ __global__ __launch_bounds__(BM_BLOCK) void k_row_segcount(int nkh, int nslots, 
     if (t < nrows && hcode[t] < 0) rowcnt[t] = segcnt[(size_t)nkh + t];
 }
 
-// rowseg: the ids of a row's segments in ascending order
+// rowseg: the ids of a row's segments in ascending order. A heavy row has one key per panel slot: a wave takes
+// the row, its lanes the slots (64 at a time, a prefix sum over the lanes gives every slot its place); a light
+// row is one thread's.
 __global__ __launch_bounds__(BM_BLOCK) void k_rowseg_fill(int nkh, int nslots, int nheavy, int nrows,
                                                           const int* __restrict__ hcode, const int* __restrict__ hrow,
                                                           const int* __restrict__ segcnt, const int* __restrict__ segbase,
                                                           const int* __restrict__ rowptr, int* __restrict__ rowseg) {
     const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    if (t < nheavy) {
-        int d = rowptr[hrow[t]];
-        for (int s = 0; s < nslots; ++s) {
-            const size_t q = (size_t)s * nheavy + t;
-            const int n = segcnt[q], base = segbase[q];
-            for (int i = 0; i < n; ++i) rowseg[d++] = base + i;
+    const long long w = t >> 6;
+    const int lane = threadIdx.x & 63;
+    if (w < nheavy) {
+        int d = rowptr[hrow[w]];
+        for (int s0 = 0; s0 < nslots; s0 += 64) {
+            const int sl = s0 + lane;
+            const size_t q = (size_t)(sl < nslots ? sl : 0) * nheavy + (size_t)w;
+            const int n = sl < nslots ? segcnt[q] : 0;
+            const int base = sl < nslots ? segbase[q] : 0;
+            int inc = n;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int y = __shfl_up(inc, o, 64);
+                if (lane >= o) inc += y;
+            }
+            const int at = d + inc - n;
+            for (int i = 0; i < n; ++i) rowseg[at + i] = base + i;
+            d += __shfl(inc, 63, 64);
         }
     }
     if (t < nrows && hcode[t] < 0) {
@@ -788,7 +802,7 @@ hipError_t build_rows_binned(bidmat_plan* plan, const int* ir, const int* jc, co
     hipLaunchKernelGGL(k_row_segcount, dim3(blocks_for(nrows > nheavy ? nrows : nheavy)), dim3(BM_BLOCK), 0, s, nkh, nslots, nheavy,
                        nrows, hcode, hrow, segcnt, rowcnt);
     RB_CHECK(scan_exclusive_i32(rowcnt, plan->rowptr, nrows, scantmp2, s));
-    hipLaunchKernelGGL(k_rowseg_fill, dim3(blocks_for(nrows > nheavy ? nrows : nheavy)), dim3(BM_BLOCK), 0, s, nkh, nslots, nheavy,
+    hipLaunchKernelGGL(k_rowseg_fill, dim3(blocks_for((long long)nrows > 64LL * nheavy ? (long long)nrows : 64LL * nheavy)), dim3(BM_BLOCK), 0, s, nkh, nslots, nheavy,
                        nrows, hcode, hrow, segcnt, segbase, plan->rowptr, plan->rowseg);
     RB_CHECK(hipGetLastError());
     RB_CHECK(hipStreamSynchronize(s));
