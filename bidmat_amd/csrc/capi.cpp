@@ -35,8 +35,16 @@ std::atomic<int> g_plan_builder{0};
 std::atomic<int> g_rowsum_form{0};
 std::atomic<int> g_class_shift{-1};
 std::atomic<int> g_plan_pool_mb{4096};
+std::atomic<int> g_dense_rows{128};
+std::atomic<int> g_dense_min_pct{15};
+std::atomic<int> g_dense_min_nnz{1 << 22};
+std::atomic<int> g_dense_cb{0};
 }  // namespace
 int opt_plan_pool_mb() { return g_plan_pool_mb.load(std::memory_order_relaxed); }
+int opt_dense_rows() { return g_dense_rows.load(std::memory_order_relaxed); }
+int opt_dense_min_pct() { return g_dense_min_pct.load(std::memory_order_relaxed); }
+int opt_dense_min_nnz() { return g_dense_min_nnz.load(std::memory_order_relaxed); }
+int opt_dense_cb() { return g_dense_cb.load(std::memory_order_relaxed); }
 int opt_plan_builder() { return g_plan_builder.load(std::memory_order_relaxed); }
 int opt_class_shift() { return g_class_shift.load(std::memory_order_relaxed); }
 int opt_rowsum_form() { return g_rowsum_form.load(std::memory_order_relaxed); }
@@ -162,8 +170,8 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
 
 // The nseg*k partial sums of one call through a plan: scratch of the stream the call runs on, so a plan holds
 // pattern data only and calls on different streams do not meet.
-float* row_partial(const bidmat_plan* plan, int k, hipStream_t s, hipError_t* err) {
-    return (float*)bm::ws_get(bm::WS_ROWPARTIAL, sizeof(float) * (size_t)plan->nseg * (size_t)k, err, s);
+float* row_partial(const bidmat_plan* plan, int k, hipStream_t s, hipError_t* err, size_t extra_floats = 0) {
+    return (float*)bm::ws_get(bm::WS_ROWPARTIAL, sizeof(float) * ((size_t)plan->nseg * (size_t)k + extra_floats), err, s);
 }
 
 // vals == nullptr: the values stored in the plan by bidmat_plan_set_values (already in plan order)
@@ -172,12 +180,27 @@ hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* va
                        hipStream_t s, hipEvent_t between = nullptr) {
     hipError_t err;
     if (!vals && !plan->pvals && plan->nnz > 0) return hipErrorInvalidValue;
-    float* partial = row_partial(plan, k, s, &err);
+    // With values of the caller's (stored order) and a k the dense product is written for, the plan's dense rows go
+    // through the matrix cores: their partial sums follow the segments' in the scratch, then the flag that tells
+    // whether A held a value that is not finite (the dense rows' segments are then gathered after all).
+    const bool dense = vals != nullptr && plan->ndense > 0 && bm::dense_rows_fit(k) && bm::opt_dense_rows() > 0;
+    const size_t dfloats = dense ? (size_t)(plan->ndblocks + bm::dense_rows_fold(plan->ndblocks)) * (size_t)plan->ndense * (size_t)k : 0;
+    float* partial = row_partial(plan, k, s, &err, dense ? dfloats + 64 : 0);
     if (!partial) return err;
+    float* dpart = partial + (size_t)plan->nseg * (size_t)k;
+    int* flag = dense ? reinterpret_cast<int*>(dpart + dfloats) : nullptr;
     if ((err = bm::gather_segments(k, plan->nseg, plan->xcd_start, A, vals ? vals : plan->pvals, plan->pc,
-                                   vals ? plan->perm : nullptr, plan->segstart, partial, s)) != hipSuccess) return err;
+                                   vals ? plan->perm : nullptr, plan->segstart, partial, s,
+                                   dense ? plan->dskip : nullptr, flag)) != hipSuccess) return err;
+    if (dense) {
+        if ((err = bm::dense_rows_stage(k, plan->ncols, plan->ndense, plan->dcb, plan->ndblocks, A, vals, plan->dpos, dpart,
+                                        flag, s)) != hipSuccess) return err;
+        if ((err = bm::gather_segments_listed(k, plan->ndseg, plan->dseglist, flag, A, vals, plan->pc, plan->perm,
+                                              plan->segstart, partial, s)) != hipSuccess) return err;
+    }
     if (between && (err = hipEventRecord(between, s)) != hipSuccess) return err;
-    return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, partial, C, beta, s);
+    return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, partial, C, beta, s,
+                               dense ? plan->rowptr2 : nullptr, dense ? plan->rowseg2 : nullptr, flag);
 }
 
 hipError_t run_spsum_rows(bidmat_plan* plan, const float* vals, float* out, int beta, hipStream_t s) {
@@ -563,6 +586,10 @@ API long long bidmat_plan_info(const bidmat_plan* plan, const char* name) {
     if (!strcmp(name, "col_classes")) return plan->ncls;
     if (!strcmp(name, "class_hot")) return plan->hcap;
     if (!strcmp(name, "longest_column")) return plan->maxlen;
+    if (!strcmp(name, "dense_rows")) return plan->ndense;
+    if (!strcmp(name, "dense_blocks")) return plan->ndblocks;
+    if (!strcmp(name, "dense_block_cols")) return plan->dcb;
+    if (!strcmp(name, "dense_segments")) return plan->ndseg;
     if (!strncmp(name, "xcd_start", 9) && name[9] >= '0' && name[9] <= '8' && !name[10]) return plan->xcd_start[name[9] - '0'];
     return -1;
 }
@@ -581,6 +608,8 @@ API int bidmat_plan_array(const bidmat_plan* plan, const char* name, const void*
         {"cir", plan->cir, cls ? plan->nnz : 0}, {"cperm", plan->cperm, cls ? plan->nnz : 0},
         {"cptr", plan->cptr, cls ? 16LL * plan->ncols + 1 : 0},
         {"ovf", plan->ovf, plan->ovf ? (long long)plan->ncols + 1 : 0},
+        {"drow", plan->drow, plan->ndense}, {"drank", plan->drank, plan->ndense > 0 ? plan->nrows : 0},
+        {"dpos", plan->dpos, (long long)plan->ndense * plan->ncols},
     };
     for (auto& t : tab)
         if (!strcmp(name, t.n)) { *dptr = t.c > 0 ? t.p : nullptr; *count = t.p ? t.c : 0; return 0; }
@@ -1074,6 +1103,26 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_col_classes.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "dense_rows")) {
+        if (value < 0 || value > bm::dense_rows_max() || value % 32 != 0) return kInvalid;
+        bm::g_dense_rows.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "dense_min_pct")) {
+        if (value < 1 || value > 100) return kInvalid;
+        bm::g_dense_min_pct.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "dense_min_nnz")) {
+        if (value < 0 || value > 0x7fffffffLL) return kInvalid;
+        bm::g_dense_min_nnz.store((int)value);
+        return 0;
+    }
+    if (!strcmp(name, "dense_cb")) {
+        if (value < 0 || value > (1 << 24)) return kInvalid;
+        bm::g_dense_cb.store((int)value);
+        return 0;
+    }
     return kInvalid;
 }
 
@@ -1095,6 +1144,10 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "rowsum_form")) return bm::opt_rowsum_form();
     if (!strcmp(name, "class_shift")) return bm::opt_class_shift();
     if (!strcmp(name, "plan_pool_mb")) return bm::opt_plan_pool_mb();
+    if (!strcmp(name, "dense_rows")) return bm::opt_dense_rows();
+    if (!strcmp(name, "dense_min_pct")) return bm::opt_dense_min_pct();
+    if (!strcmp(name, "dense_min_nnz")) return bm::opt_dense_min_nnz();
+    if (!strcmp(name, "dense_cb")) return bm::opt_dense_cb();
     return -2;
 }
 

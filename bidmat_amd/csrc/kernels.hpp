@@ -20,6 +20,10 @@ int opt_rowsum_form();  // bidmat_spsum_rows_csc: 0 = by the row count (default)
 int opt_plan_builder(); // row side of a plan: 0 = per-panel counting sorts (default), 1 = one library radix sort
 int opt_check_plan();  // 1: plans keep a digest of their pattern and the plan-taking calls compare it
 int opt_col_classes(); // row-class ordering of the columns in a plan: -1 decide from the pattern, 0 never, 1 always
+int opt_dense_rows();  // rows a plan may treat as a dense block of A *^ S (0 = none, at most 128)
+int opt_dense_min_pct(); // a row counts as dense when it has a nonzero in at least this percentage of the columns
+int opt_dense_min_nnz(); // patterns with fewer nonzeros get no dense block
+int opt_dense_cb();    // columns per block of the dense product (0 = chosen from the column count)
 
 // ---- CSC utilities (csc_util.hip)
 hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);
@@ -108,9 +112,13 @@ hipError_t dds_csc_static(int k, int ncols, int nnz, const float* A, const float
 // ---- plan stage kernels (spmm.hip): segment s gathers columns pc[p] of A scaled by
 // vals[perm[p]] for p in [segstart[s], segstart[s+1]) into partial[s*k ..].
 // xcd_start[9]: segment groups per XCD (see plan.hpp); workgroup b is assumed to run on XCD b % 8.
+// skip (nullable): a byte per segment, 1 = leave the segment out. flag (nullable): an int the launch clears.
 hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A, const float* vals,
                            const int* pc, const int* perm, const int* segstart, float* partial,
-                           hipStream_t s);
+                           hipStream_t s, const unsigned char* skip = nullptr, int* flag = nullptr);
+// The segments list[0..n) only, and only if *flag != 0 when the launch runs (its waves return at once otherwise).
+hipError_t gather_segments_listed(int k, int n, const int* list, const int* flag, const float* A, const float* vals,
+                                  const int* pc, const int* perm, const int* segstart, float* partial, hipStream_t s);
 // tile form: column stride lda of A; only nonzeros whose column lies in `cols` (rebased), only
 // segments whose row (segrow) lies in `rowsel`.
 hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, const float* A,
@@ -128,11 +136,14 @@ hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_star
 hipError_t fused_columns(int k, int ncols, int nnz, const float* A, const float* B, const float* vals, const int* ir,
                          const int* jc, int opn, float* Q, float* C, int beta, hipStream_t s, const ColTable* tab = nullptr);
 // C[:,r] = beta*C[:,r] + sum over q in [rowptr[r], rowptr[r+1]) of partial[rowseg[q]*k ..]
+// rowptr2 / rowseg2 / flag (nullable): the table to use instead while *flag == 0.
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
-                           const float* partial, float* C, int beta, hipStream_t s);
+                           const float* partial, float* C, int beta, hipStream_t s, const int* rowptr2 = nullptr,
+                           const int* rowseg2 = nullptr, const int* flag = nullptr);
 // tile form: rows [row0, row0+nrows) of the plan go to columns 0.. of C (stride ldc)
 hipError_t reduce_segments_ex(int k, int ldc, int row0, int nrows, const int* rowptr, const int* rowseg,
-                              const float* partial, float* C, int beta, hipStream_t s);
+                              const float* partial, float* C, int beta, hipStream_t s, const int* rowptr2 = nullptr,
+                              const int* rowseg2 = nullptr, const int* flag = nullptr);
 
 // ---- sums (sums.hip)
 hipError_t spsum_cols(int ncols, int nnz, const float* vals, const int* jc, float* out, int beta,

@@ -483,7 +483,7 @@ hipError_t plan_alloc(T** p, size_t bytes) {
 }
 // Frees one half of a plan and marks it absent.
 hipError_t drop_rows(bidmat_plan* p) {
-    hipError_t e = hipSuccess;
+    hipError_t e = drop_dense(p);
     free_all({&p->block_nnz, &p->block_seg, (void**)&p->pvals}, &e);
     p->pc = p->perm = p->rowptr = p->segstart = p->segrow = p->rowseg = nullptr;
     p->nseg = p->nheavy = 0;
@@ -988,6 +988,10 @@ hipError_t build_sides(bidmat_plan* plan, const int* ir, const int* jc, int side
         if (opt_plan_builder() == 0) PB_CHECK(build_rows_binned(plan, ir, jc, t.hflag, t.hrow, nheavy, p8, t.bad, &unfit, s));
         if (unfit) PB_CHECK(build_rows_sorted(plan, ir, jc, t, nheavy, p8, s));
         clock.mark(unfit ? "row side (library sort)" : "row side (counting sorts)");
+        if (opt_dense_rows() > 0 && (long long)nnz >= opt_dense_min_nnz() && dense_rows_fit(k_hint)) {
+            PB_CHECK(build_dense_rows(plan, ir, jc, t.cnt, t.sample, s));
+            clock.mark("dense rows");
+        }
     }
     PB_CHECK(hipGetLastError());
     if (t.arena_bytes > ((size_t)opt_plan_keep_mb() << 20)) PB_CHECK(ws_drop(WS_PLAN));

@@ -41,6 +41,23 @@ struct bidmat_plan {
     int* rowseg = nullptr;   // [nseg]   segment ids grouped by row, ascending within a row
     void* block_nnz = nullptr;   // owns pc, perm, rowptr
     void* block_seg = nullptr;   // owns segstart, segrow, rowseg
+    // The densest rows as a dense block of A *^ S (dense_rows.hip; optional, ndense == 0: none). The segments of
+    // these rows stay in the arrays above (row sums and the other walks over the plan use them); A *^ S leaves
+    // them out (dskip) and multiplies the rows on the matrix cores instead, one partial sum per dense row and
+    // block of dcb columns, which the second row table (rowptr2 / rowseg2) lists in place of the segments.
+    int ndense = 0;              // dense rows, a multiple of 32
+    int dcb = 0;                 // columns per block of the dense product
+    int ndblocks = 0;            // blocks of columns
+    int ndseg = 0;               // segments of the dense rows
+    int* drank = nullptr;        // [nrows]  rank of a dense row (by count, descending), -1 for every other row
+    int* drow = nullptr;         // [ndense] row of every rank
+    int* dpos = nullptr;         // [ncols*ndense] position (stored order) of column c's nonzero in dense row d, or -1
+    unsigned char* dskip = nullptr;  // [nseg] 1: segment of a dense row
+    int* dseglist = nullptr;     // [ndseg] those segments
+    int* rowptr2 = nullptr;      // [nrows+1] like rowptr / rowseg, a dense row's entries being the partial sums
+    int* rowseg2 = nullptr;      //           nseg + (ndblocks + ch)*ndense + d of the chunks ch of blocks of columns
+    void* block_dense = nullptr; // owns drank, drow, dskip, dseglist, rowptr2, rowseg2
+    size_t dense_bytes = 0;      // device bytes of the dense block's arrays (counted in row_bytes)
     // (the nseg*k partial sums of a call live in the scratch of the stream it runs on, not here)
     size_t row_bytes = 0;        // device bytes of the row side's index arrays
     size_t col_bytes = 0;        // device bytes of the column side's index arrays
@@ -92,4 +109,12 @@ hipError_t build_rows_binned(bidmat_plan* plan, const int* ir, const int* jc, co
 hipError_t plan_digest(int nnz, int ncols, const int* ir, const int* jc, unsigned long long d[2]);
 // pvals[p] = data[perm[p]] (allocates pvals on first use).
 hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s);
+// The dense block of the row side (dense_rows.hip). cnt[r]: about (nonzeros of row r) / sample.
+hipError_t build_dense_rows(bidmat_plan* plan, const int* ir, const int* jc, const int* cnt, int sample, hipStream_t s);
+hipError_t drop_dense(bidmat_plan* p);
+bool dense_rows_fit(int k);      // the dense product is written for 64 < k <= 256
+int dense_rows_max();
+int dense_rows_fold(int ndblocks);   // partial sums per dense row that reach the row reduction
+hipError_t dense_rows_stage(int k, int ncols, int nd, int cb, int ndblocks, const float* A, const float* vals,
+                            const int* dpos, float* part, int* flag, hipStream_t s);
 }  // namespace bm

@@ -53,6 +53,10 @@ struct GatherArgs {
     int opn;
     float* qout;
     const int* qperm;    // position of each product in qout (nullptr: plan order)
+    // plan mode, A *^ S with the densest rows multiplied elsewhere (dense_rows.hip)
+    const unsigned char* skip;   // a byte per segment, 1 = not this launch's (nullable)
+    int* flag;                   // cleared by the launch over all segments; the launch over `seglist` only works when it is set
+    const int* seglist;          // the launch takes segments seglist[0 .. nfirst) instead of all (nullable)
 };
 
 template <int V, int LPN>
@@ -167,12 +171,20 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
         // the light segments (every 8th one). Interleaving the two kinds, with or without
         // non-temporal loads for the light gathers, was measured slower: the light gathers miss
         // L2 and evict the panel the heavy segments are reusing.
-        const int xcd = blockIdx.x & 7;
-        const long long wi = (long long)(blockIdx.x >> 3) * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
-        const int hstart = a.xcd_start[xcd];
-        const int hcount = a.xcd_start[xcd + 1] - hstart;
-        const long long seg = wi < hcount ? hstart + wi : a.xcd_start[8] + (wi - hcount) * 8 + xcd;
-        if (seg >= a.nfirst) return;
+        long long seg;
+        if (a.seglist != nullptr) {
+            if (*a.flag == 0 || w >= a.nfirst) return;
+            seg = a.seglist[w];
+        } else {
+            if (a.flag != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *a.flag = 0;
+            const int xcd = blockIdx.x & 7;
+            const long long wi = (long long)(blockIdx.x >> 3) * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
+            const int hstart = a.xcd_start[xcd];
+            const int hcount = a.xcd_start[xcd + 1] - hstart;
+            seg = wi < hcount ? hstart + wi : a.xcd_start[8] + (wi - hcount) * 8 + xcd;
+            if (seg >= a.nfirst) return;
+            if (a.skip != nullptr && a.skip[seg]) return;
+        }
         if (a.segrow != nullptr && (unsigned)(a.segrow[seg] - a.row_off) >= (unsigned)a.row_len) return;
         jstart = a.ptr[seg];
         jend = a.ptr[seg + 1];
@@ -576,11 +588,15 @@ __global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int ldc, in
                                                               const int* __restrict__ rowptr,
                                                               const int* __restrict__ rowseg,
                                                               const float* __restrict__ partial,
-                                                              float* __restrict__ C, int beta) {
+                                                              float* __restrict__ C, int beta,
+                                                              const int* __restrict__ rowptr2,
+                                                              const int* __restrict__ rowseg2,
+                                                              const int* __restrict__ flag) {
     const long long t = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
     const long long row = t / lpr;
     const int l = (int)(t % lpr);
     if (row >= nrows) return;
+    if (rowptr2 != nullptr && *flag == 0) { rowptr = rowptr2; rowseg = rowseg2; }
     const int s = rowptr[row0 + row], e = rowptr[row0 + row + 1];
     for (int el = l * W; el < k; el += lpr * W) {
         float* o = C + (size_t)row * ldc + el;
@@ -673,6 +689,7 @@ void init_args(GatherArgs& a) {
     for (int x = 0; x < 9; ++x) a.xcd_start[x] = 0;
     a.pstride = 1; a.poff = 0; a.pspan = 1;
     a.R = nullptr; a.ldr = 0; a.opn = 0; a.qout = nullptr; a.qperm = nullptr;
+    a.skip = nullptr; a.flag = nullptr; a.seglist = nullptr;
 }
 }  // namespace
 
@@ -753,16 +770,45 @@ hipError_t dsmult_phased(int k, int ncols, const float* A, const float* vals, co
     return hipSuccess;
 }
 
+namespace {
+hipError_t gather_segments_impl(int k, int lda, int nseg, const int* xcd_start, const float* A,
+                                const float* vals, const int* pc, const int* perm, const int* segstart,
+                                float* partial, Window cols, const int* segrow, Window rowsel, hipStream_t s,
+                                const unsigned char* skip, int* flag);
+}
+
 hipError_t gather_segments(int k, int nseg, const int* xcd_start, const float* A, const float* vals,
                            const int* pc, const int* perm, const int* segstart, float* partial,
-                           hipStream_t s) {
-    return gather_segments_ex(k, k, nseg, xcd_start, A, vals, pc, perm, segstart, partial,
-                              Window{0, 0, 0}, nullptr, Window{0, 0, 0}, s);
+                           hipStream_t s, const unsigned char* skip, int* flag) {
+    return gather_segments_impl(k, k, nseg, xcd_start, A, vals, pc, perm, segstart, partial,
+                                Window{0, 0, 0}, nullptr, Window{0, 0, 0}, s, skip, flag);
+}
+
+hipError_t gather_segments_listed(int k, int n, const int* list, const int* flag, const float* A, const float* vals,
+                                  const int* pc, const int* perm, const int* segstart, float* partial, hipStream_t s) {
+    if (k <= 0 || n <= 0) return hipSuccess;
+    Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(partial)));
+    GatherArgs a;
+    init_args(a);
+    a.k = k; a.lda = k; a.ldo = k; a.nfirst = n; a.seglen = 0; a.beta = 0;
+    a.A = A; a.vals = vals; a.idx = pc; a.perm = perm; a.ptr = segstart; a.ovf = nullptr;
+    a.out = partial; a.partial = nullptr;
+    a.seglist = list; a.flag = const_cast<int*>(flag);
+    return launch_gather<true>(sh, a, n, s);
 }
 
 hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, const float* A,
                               const float* vals, const int* pc, const int* perm, const int* segstart,
                               float* partial, Window cols, const int* segrow, Window rowsel, hipStream_t s) {
+    return gather_segments_impl(k, lda, nseg, xcd_start, A, vals, pc, perm, segstart, partial, cols, segrow, rowsel, s,
+                                nullptr, nullptr);
+}
+
+namespace {
+hipError_t gather_segments_impl(int k, int lda, int nseg, const int* xcd_start, const float* A,
+                                const float* vals, const int* pc, const int* perm, const int* segstart,
+                                float* partial, Window cols, const int* segrow, Window rowsel, hipStream_t s,
+                                const unsigned char* skip, int* flag) {
     if (k <= 0 || nseg <= 0) return hipSuccess;
     Shape sh = clamp_shape(pick_shape(k, aligned16(A) && aligned16(partial) && lda % 4 == 0));
     GatherArgs a;
@@ -772,6 +818,7 @@ hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, co
     a.out = partial; a.partial = nullptr;
     a.win_on = cols.on; a.win_off = cols.off; a.win_len = cols.len;
     if (rowsel.on) { a.segrow = segrow; a.row_off = rowsel.off; a.row_len = rowsel.len; }
+    a.skip = skip; a.flag = flag;
     int maxheavy = 0;
     for (int x = 0; x < 9; ++x) a.xcd_start[x] = xcd_start[x];
     for (int x = 0; x < 8; ++x) maxheavy = std::max(maxheavy, a.xcd_start[x + 1] - a.xcd_start[x]);
@@ -781,6 +828,7 @@ hipError_t gather_segments_ex(int k, int lda, int nseg, const int* xcd_start, co
     const long long blocks_per_xcd = (per_xcd + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
     return launch_gather<true>(sh, a, blocks_per_xcd * 8 * BM_WAVES_PER_BLOCK, s);
 }
+}  // namespace
 
 hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_start, const int* segrow,
                           const float* R, const float* A, const float* vals, const int* pc, const int* perm,
@@ -880,12 +928,15 @@ hipError_t fused_columns(int k, int ncols, int nnz, const float* A, const float*
 }
 
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,
-                           const float* partial, float* C, int beta, hipStream_t s) {
-    return reduce_segments_ex(k, k, 0, nrows, rowptr, rowseg, partial, C, beta, s);
+                           const float* partial, float* C, int beta, hipStream_t s, const int* rowptr2,
+                           const int* rowseg2, const int* flag) {
+    return reduce_segments_ex(k, k, 0, nrows, rowptr, rowseg, partial, C, beta, s, rowptr2, rowseg2, flag);
 }
 
 hipError_t reduce_segments_ex(int k, int ldc, int row0, int nrows, const int* rowptr, const int* rowseg,
-                              const float* partial, float* C, int beta, hipStream_t s) {
+                              const float* partial, float* C, int beta, hipStream_t s, const int* rowptr2,
+                              const int* rowseg2, const int* flag) {
+    if (rowptr2 == nullptr || rowseg2 == nullptr || flag == nullptr) { rowptr2 = nullptr; rowseg2 = nullptr; flag = nullptr; }
     if (k <= 0 || nrows <= 0) return hipSuccess;
     const bool al = aligned16(C) && aligned16(partial) && (k % 4 == 0) && (ldc % 4 == 0);
     const int W = al ? 4 : 1;
@@ -894,8 +945,8 @@ hipError_t reduce_segments_ex(int k, int ldc, int row0, int nrows, const int* ro
     long long threads = (long long)nrows * lpr;
     long long nblk = (threads + BM_BLOCK - 1) / BM_BLOCK;
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (al) hipLaunchKernelGGL(k_reduce_segments<4>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, ldc, row0, nrows, lpr, rowptr, rowseg, partial, C, beta);
-    else hipLaunchKernelGGL(k_reduce_segments<1>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, ldc, row0, nrows, lpr, rowptr, rowseg, partial, C, beta);
+    if (al) hipLaunchKernelGGL(k_reduce_segments<4>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, ldc, row0, nrows, lpr, rowptr, rowseg, partial, C, beta, rowptr2, rowseg2, flag);
+    else hipLaunchKernelGGL(k_reduce_segments<1>, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, k, ldc, row0, nrows, lpr, rowptr, rowseg, partial, C, beta, rowptr2, rowseg2, flag);
     return hipGetLastError();
 }
 

@@ -213,6 +213,26 @@ def test_config5_nmf_step(hip):
     assert np.array_equal(dQ2.numpy(), Q)
     # ... and the whole chain in one walk over the plan's rows (what bench.py times for this configuration), with the
     # stored V and with the caller's, with and without the products written: the same bits again
+    # (the one walk adds every row's terms in the plan's order; bidmat_dsmultT_plan does so too once the plan's dense
+    # block, which reorders the sums of the most frequent rows, is switched off: that is the G the bits are held against,
+    # the G with the dense block having been checked against the oracle above, rows 0 and 1 among the sampled ones)
+    dense_rows = int(hip.bidmat_plan_info(plan, b"dense_rows"))
+    assert dense_rows >= 32, "this pattern's most frequent rows are in most columns"
+    hip_abi.check(hip.bidmat_set_option(b"dense_rows", 0))
+    try:
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, dH.ptr, dR.ptr, dG2.ptr, 0, None))
+        hip_abi.check(hip.bidmat_synchronize())
+    finally:
+        hip_abi.check(hip.bidmat_set_option(b"dense_rows", 128))
+    G_plain = dG2.numpy()
+    drow = np.empty(dense_rows, np.int32)
+    ptr, cnt = C.c_void_p(), C.c_longlong()
+    hip_abi.check(hip.bidmat_plan_array(plan, b"drow", C.byref(ptr), C.byref(cnt)))
+    hip_abi.check(hip.bidmat_memcpy_d2h(drow.ctypes.data, ptr, 4 * dense_rows))
+    others = np.ones(nrows, bool); others[drow] = False
+    assert np.array_equal(G_plain.reshape(nrows, k)[others], G.reshape(nrows, k)[others]), "rows outside the dense block changed"
+    np.testing.assert_allclose(G.reshape(nrows, k)[drow], G_plain.reshape(nrows, k)[drow], rtol=1e-5)
+    G = G_plain
     for vptr, qptr in ((None, dQ2.ptr), (dv.ptr, None)):
         hip_abi.check(hip.bidmat_memset(dQ2.ptr, 0, dQ2.nbytes))
         hip_abi.check(hip.bidmat_memset(dG2.ptr, 0, dG2.nbytes))
