@@ -290,7 +290,9 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
         workload = "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), step = DDS, A*S, A*^S"
         metric = "algorithmic GB/s (gathered operand charged once per nonzero) and nnz/s for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
         roof_op = "dsmultT"
-        roof_kernel = "k_gather_axpy<4,1,64,true> = stage 1 of A*^S, the time-dominant kernel of the step (one launch = the gathers of the whole pattern in plan order)"
+        roof_kernel = ("stage 1 of A*^S, the time-dominant part of the step: k_gather_axpy<4,1,64,true> (the gathers of the pattern in plan "
+                       "order) + k_dense_mfma<8,4> (the plan's densest rows as a dense block on the matrix cores) + k_dense_fold, "
+                       "timed as one stretch of the stream; bytes and time are those of the three launches together")
     elif name in ("C1", "C4"):
         d_A = up(cfg["A"])
         d_C = DeviceArray(k * ncols, np.float32)

@@ -183,16 +183,25 @@ long long bidmat_plan_bytes(const bidmat_plan *plan);
 int bidmat_plan_segments(const bidmat_plan *plan);
 /* Inspection (tests, tools; no counterpart in the reference).  bidmat_plan_info: a scalar of the plan by name
  * ("nrows", "ncols", "nnz", "sides" (1 row side | 2 column side), "nseg", "nheavy", "npanels", "panel_cols",
- * "seglen", "col_classes", "class_hot", "longest_column", "xcd_start0" .. "xcd_start8"); -1 for an unknown name.
+ * "seglen", "col_classes", "class_hot", "longest_column", "xcd_start0" .. "xcd_start8", "dense_rows",
+ * "dense_blocks", "dense_block_cols", "dense_segments"); -1 for an unknown name.
  * bidmat_plan_array: device address and element count (int32 each) of one of the plan's index arrays
- * ("pc", "perm", "segstart", "segrow", "rowseg", "rowptr", "cir", "cperm", "cptr", "ovf"; count 0 when the
- * plan does not hold it).  The arrays stay the plan's. */
+ * ("pc", "perm", "segstart", "segrow", "rowseg", "rowptr", "cir", "cperm", "cptr", "ovf", "drow", "drank", "dpos";
+ * count 0 when the plan does not hold it).  The arrays stay the plan's. */
 long long bidmat_plan_info(const bidmat_plan *plan, const char *name);
 int bidmat_plan_array(const bidmat_plan *plan, const char *name, const void **dptr, long long *count);
 
 /* C = beta*C + A*S^T through a plan.  A k x ncols, C k x nrows(S).  Sdata: the nnz values
  * in the original CSC order.  With beta == 0 every column of C is written (zeros for empty
- * rows of S). */
+ * rows of S).
+ * Dense block: when the pattern has rows with a nonzero in a large share of the columns (options "dense_rows",
+ * "dense_min_pct", "dense_min_nnz" below; plan info "dense_rows"), the plan ranks up to 128 of them at build time and,
+ * for 64 < k <= 256 and values passed in Sdata, their columns of C are computed as a dense product on the matrix
+ * cores (the columns of A streamed once per 32 rows, absent entries as zeros) instead of one gather per nonzero.
+ * Only the order in which those rows' terms are added changes (fixed by the pattern: same bits from run to run,
+ * within the 1e-4 tolerance of the path); every other row keeps its bits.  A value of A that is not finite makes the
+ * call compute those rows from their segments after all (decided on the device, also inside a replayed graph), so
+ * an absent entry's zero never meets an infinity. */
 int bidmat_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *Sdata, float *C,
                         int beta, void *stream);
 
@@ -237,7 +246,9 @@ int bidmat_dds_plan_stored(bidmat_plan *plan, int k, const float *A, const float
  * callers GSMat.scala:649-667 and GMat.scala:1082-1096).  A is k x nrows, B is k x ncols, G is k x nrows.  For
  * every nonzero the column of B is gathered once and serves the dot product and the accumulation; Q is only
  * written when Q != NULL (nnz values in the stored CSC order).  V == NULL: the values stored in the plan.  The
- * results are those of bidmat_dds_plan[_stored] followed by bidmat_dsmultT_plan, bit for bit.  k must fit one pass
+ * results are those of bidmat_dds_plan[_stored] followed by bidmat_dsmultT_plan, bit for bit (of bidmat_dsmultT_plan
+ * walking the segments of every row, i.e. with option "dense_rows" = 0: its dense block adds the most frequent rows'
+ * terms in another order).  k must fit one pass
  * (k <= 1024 with 16-byte aligned operands and k % 4 == 0, else k <= 256): otherwise hipErrorInvalidValue, and
  * the two calls remain.  Needs the row side of the plan. */
 int bidmat_dds_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const float *B, const float *V, int opn,
@@ -431,6 +442,14 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "plan_keep_mb" temporaries of a plan build up to this many MiB stay allocated on the device for the
  *              next build (default 4096: a 100 M-nonzero pattern needs 3.7 GB; 0 = always give them
  *              back); bidmat_release_caches frees them
+ *   "dense_rows" how many of a pattern's most frequent rows a plan may treat as a dense block of A *^ S (see
+ *              bidmat_dsmultT_plan; a multiple of 32 up to 128, default 128; 0 = none: plans made while it is 0 get no
+ *              dense block, and calls made while it is 0 walk the segments of every row whatever the plan holds)
+ *   "dense_min_pct" a row belongs to the dense block when it has a nonzero in at least this percentage of the
+ *              columns (default 15; below about 9 % a gather per nonzero is cheaper than multiplying zeros)
+ *   "dense_min_nnz" patterns with fewer nonzeros get no dense block (default 4 194 304)
+ *   "dense_cb" columns per block of the dense product, each block giving one partial sum per dense row
+ *              (default 0 = chosen from the column count so that the blocks fill the device evenly, about 330 to 400)
  * Returns 0, or hipErrorInvalidValue for an unknown name / bad value; bidmat_get_option returns -2
  * for an unknown name. */
 int bidmat_set_option(const char *name, long long value);

@@ -229,3 +229,48 @@ def test_the_other_walks_over_the_plan_are_untouched(dense_options):
         assert ok, (name, worst)
     hip_abi.check(hip.bidmat_plan_destroy(plan))
     d.free()
+
+
+def test_graph_replay_with_the_dense_block(dense_options):
+    """A *^ S with a dense block recorded into a HIP graph: every replay gives what the eager call gives, also the
+    replay whose A holds a value that is not finite (the fall-back to the segments is decided on the device)."""
+    hip = dense_options
+    nrows, ncols, k = 1200, 2000, 256
+    rng = np.random.default_rng(21)
+    ir, jc = power_law_csc(rng, nrows, ncols, 70)
+    nnz = ir.size
+    A = rng.standard_normal(k * ncols).astype(np.float32)
+    v = (1.0 - rng.random(nnz)).astype(np.float32)
+    d = Dev(ir=ir, jc=jc, A=A, v=v)
+    d.zeros("G", k * nrows); d.zeros("G2", k * nrows)
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    assert plan_info(hip, plan, "dense_rows") >= 32
+    st = C.c_void_p()
+    hip_abi.check(hip.bidmat_stream_create(C.byref(st)))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, d.v.ptr, d.G.ptr, 0, st))       # sizes the stream's scratch
+    hip_abi.check(hip.bidmat_stream_synchronize(st))
+    hip_abi.check(hip.bidmat_graph_begin_capture(st))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, d.v.ptr, d.G.ptr, 0, st))
+    gx = C.c_void_p()
+    hip_abi.check(hip.bidmat_graph_end_capture(st, C.byref(gx)))
+    for rep in range(4):
+        newA = rng.standard_normal(k * ncols).astype(np.float32)
+        if rep == 2:
+            newA[k * 5 + 3] = -np.inf
+        hip_abi.check(hip.bidmat_memcpy_h2d(d.A.ptr, newA.ctypes.data, newA.nbytes))
+        hip_abi.check(hip.bidmat_memset(d.G.ptr, 0xFF, d.G.nbytes))
+        hip_abi.check(hip.bidmat_graph_launch(gx, st))
+        hip_abi.check(hip.bidmat_stream_synchronize(st))
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, d.v.ptr, d.G2.ptr, 0, None))
+        hip_abi.check(hip.bidmat_synchronize())
+        assert np.array_equal(d.G.numpy().view(np.int32), d.G2.numpy().view(np.int32)), "replay %d" % rep
+        if rep == 2:
+            hip_abi.check(hip.bidmat_set_option(b"dense_rows", 0))
+            hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, d.v.ptr, d.G2.ptr, 0, None))
+            hip_abi.check(hip.bidmat_synchronize())
+            hip_abi.check(hip.bidmat_set_option(b"dense_rows", 128))
+            assert np.array_equal(d.G.numpy().view(np.int32), d.G2.numpy().view(np.int32)), "the replay with -inf in A"
+    hip_abi.check(hip.bidmat_graph_destroy(gx))
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    hip_abi.check(hip.bidmat_stream_destroy(st))
+    d.free()

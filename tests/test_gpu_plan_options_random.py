@@ -12,7 +12,8 @@ from bidmat_amd.device import DeviceArray
 from util import dense_full, random_csc
 
 pytestmark = pytest.mark.gpu
-TUNABLES = ("seglen", "panel_kb", "heavy_min", "col_classes", "class_hot", "class_threads", "class_strip", "class_phases")
+TUNABLES = ("seglen", "panel_kb", "heavy_min", "col_classes", "class_hot", "class_threads", "class_strip", "class_phases",
+            "dense_rows", "dense_min_pct", "dense_min_nnz", "dense_cb")
 
 
 @pytest.mark.parametrize("seed0", [11, 12])
@@ -42,7 +43,9 @@ def test_plan_forms_under_random_shapes_and_settings(hip, seed0):
             nnz = int(ir.size)
             o = dict(seglen=int(rng.choice([64, 100, 256, 1024])), panel_kb=int(rng.choice([16, 64, 3072])), heavy_min=int(rng.choice([1, 2, 8])),
                      col_classes=int(rng.choice([-1, 0, 1, 1])), class_hot=int(rng.choice([-1, 0, 1, 3, 16])), class_threads=int(rng.choice([256, 512, 1024])),
-                     class_strip=int(rng.choice([1, 3, 16, 64])), class_phases=int(rng.choice([0, 1, 2, 4, 8])))
+                     class_strip=int(rng.choice([1, 3, 16, 64])), class_phases=int(rng.choice([0, 1, 2, 4, 8])),
+                     dense_rows=int(rng.choice([0, 32, 96, 128])), dense_min_pct=int(rng.choice([2, 15, 60])),
+                     dense_min_nnz=int(rng.choice([0, 0, 1 << 22])), dense_cb=int(rng.choice([0, 16, 50])))
             for n, v in o.items(): opt(n, v)
             tag = "seed=%d k=%d %dx%d nnz=%d unique=%s sorted=%s %s" % (seed, k, nrows, ncols, nnz, unique, sort_rows, o)
             A = rng.standard_normal(k * nrows).astype(np.float32); B = rng.standard_normal(k * ncols).astype(np.float32)
@@ -89,7 +92,19 @@ def test_plan_forms_under_random_shapes_and_settings(hip, seed0):
             refG = (AT2.T @ S.T).T.ravel(); saG = (np.abs(AT2).T @ np.abs(S).T).T.ravel()
             g1, g2 = G1.numpy(), G2.numpy()
             assert np.all(np.abs(g1 - refG) <= 1e-5 * saG + 1e-30), "dsmultT vs fp64 " + tag
-            assert np.array_equal(g1, g2), "dsmultT stored != fresh " + tag
+            # values passed in take the plan's dense block (if the pattern got one and k fits it), stored values walk the
+            # segments of every row: the rows outside the block have the same bits, the others agree within the tolerance
+            nd = int(lib.bidmat_plan_info(plan, b"dense_rows"))
+            if nd > 0 and 64 < k <= 256 and o["dense_rows"] > 0:
+                drow = np.empty(nd, np.int32)
+                ptr, cnt = C.c_void_p(), C.c_longlong()
+                hip_abi.check(lib.bidmat_plan_array(plan, b"drow", C.byref(ptr), C.byref(cnt)))
+                hip_abi.check(lib.bidmat_memcpy_d2h(drow.ctypes.data, ptr, 4 * nd))
+                keep = np.ones(nrows, bool); keep[drow] = False
+                assert np.array_equal(g1.reshape(nrows, k)[keep], g2.reshape(nrows, k)[keep]), "dsmultT stored != fresh outside the dense block " + tag
+                assert np.all(np.abs(g2 - refG) <= 1e-5 * saG + 1e-30), "dsmultT stored vs fp64 " + tag
+            else:
+                assert np.array_equal(g1, g2), "dsmultT stored != fresh " + tag
             assert np.array_equal(rs1.numpy(), rs2.numpy()), "row sums stored != fresh " + tag
             assert np.allclose(rs1.numpy(), S.sum(axis=1), rtol=1e-5, atol=1e-6), "row sums " + tag
             hip_abi.check(lib.bidmat_plan_destroy(plan))
