@@ -20,7 +20,7 @@
 namespace bm {
 namespace {
 std::atomic<int> g_seglen{1024};
-std::atomic<int> g_panel_kb{3072};
+std::atomic<int> g_panel_kb{4096};
 std::atomic<int> g_heavy_min{8};
 std::atomic<int> g_col_classes{-1};
 std::atomic<int> g_class_strip{16};

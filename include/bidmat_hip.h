@@ -408,7 +408,7 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
 
 /* Tunables (process-wide, read at call time):
  *   "seglen"   nonzeros per wavefront segment when a long column / row is split (default 1024)
- *   "panel_kb" target size in KiB of one column panel of A in a plan (default 3072)
+ *   "panel_kb" target size in KiB of one column panel of A in a plan (default 4096: what one L2 holds)
  *   "heavy_min" a row is cut by column panels when it averages at least this many nonzeros
  *              per panel (default 8)
  *   "col_classes" row-class ordering of the columns inside a plan, used by bidmat_dds_plan so that the
