@@ -39,13 +39,13 @@ HBM_PEAK_GBS = 8000.0
 # and HBM together), from rocprofv3 FETCH_SIZE x 2.0 plus WRITE_SIZE x 1.0 (KiB per dispatch; the
 # factors are what the same counters read for the streaming kernel of --calibrate, which moves a
 # known 2 GiB + 1 GiB). A profiler cannot run inside this script, so each figure names the summary
-# under profiles/ it was taken from and the sha256 (first 16 hex digits) of the kernel source it
-# was taken on; it is reported only for that exact workload and dropped (null) as soon as the
+# under profiles/ it was taken from and the sha256 (first 16 hex digits) of the kernel sources it
+# was taken on (concatenated); it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dsmultT", 100003320): (31.6e9, "bidmat_amd/csrc/spmm.hip", "07b900239e5e9173",
+    ("headline", "dsmultT", 100003320): (33.9e9, ("bidmat_amd/csrc/spmm.hip", "bidmat_amd/csrc/dense_rows.hip"), "a52162aa7c6bafc6",
                                          "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, "bidmat_amd/csrc/spmm.hip", "07b900239e5e9173",
+    ("C4", "dsmult", 38900534): (163.1e9, ("bidmat_amd/csrc/spmm.hip",), "f8f54a08b059f7c2",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 
@@ -55,9 +55,12 @@ def measured_traffic(workload, op, nnz):
     rec = MEASURED_TRAFFIC.get((workload, op, nnz))
     if rec is None:
         return None, None
-    nbytes, src, sha, where = rec
+    nbytes, srcs, sha, where = rec
     try:
-        cur = hashlib.sha256(open(os.path.join(ROOT, src), "rb").read()).hexdigest()[:16]
+        m = hashlib.sha256()
+        for src in srcs:
+            m.update(open(os.path.join(ROOT, src), "rb").read())
+        cur = m.hexdigest()[:16]
     except OSError:
         return None, None
     return (nbytes, where) if cur == sha else (None, None)

@@ -154,7 +154,7 @@ __device__ __forceinline__ Vec<4> vec_xor_add<4>(Vec<4> x, int m) {
 }
 
 template <int W, int V, int LPN, bool PLAN>
-__global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
+__device__ __forceinline__ void gather_axpy_body(const GatherArgs& a) {
     constexpr int KT = W * V * LPN;      // elements of a dense column covered per pass
     const int lane = threadIdx.x & 63;
     const long long w = (long long)blockIdx.x * BM_WAVES_PER_BLOCK + wave_uniform(threadIdx.x >> 6);
@@ -277,6 +277,17 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
             }
         }
     }
+}
+
+template <int W, int V, int LPN, bool PLAN>
+__global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
+    gather_axpy_body<W, V, LPN, PLAN>(a);
+}
+// The same walk over a list of segments, launched behind the dense block of A *^ S: its waves return at once
+// unless the block met a value that is not finite (a kernel of its own so that traces tell the two apart).
+template <int W, int V, int LPN>
+__global__ __launch_bounds__(BM_BLOCK) void k_gather_listed(GatherArgs a) {
+    gather_axpy_body<W, V, LPN, true>(a);
 }
 
 // ---- DDS, the elementwise step and A*^S in one walk over a plan's segments (an NMF update's
@@ -625,7 +636,10 @@ hipError_t launch_gather(const Shape& sh, const GatherArgs& a, long long nwaves,
     dim3 grid((unsigned)nblk), block(BM_BLOCK);
 #define BM_CASE(W_, V_, L_)                                                              \
     if (sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                                      \
-        hipLaunchKernelGGL((k_gather_axpy<W_, V_, L_, PLAN>), grid, block, 0, s, a);     \
+        if (PLAN && a.seglist != nullptr)                                                \
+            hipLaunchKernelGGL((k_gather_listed<W_, V_, L_>), grid, block, 0, s, a);     \
+        else                                                                             \
+            hipLaunchKernelGGL((k_gather_axpy<W_, V_, L_, PLAN>), grid, block, 0, s, a); \
         return hipGetLastError();                                                        \
     }
 #define BM_CASES(W_)                                                                     \
