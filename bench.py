@@ -614,10 +614,19 @@ def shaped_entries(lib, k, nrows, ncols, nnz, d_ir, d_jc, d_v, d_A, d_B, d_AT, d
     for opname in ("dds", "dsmult", "dsmultT"):
         ts = []
         for r in range(4):
-            # a copy of the pattern in device arrays of its own: new addresses, so nothing cached applies
+            # another pattern of the same size and statistics in device arrays of its own (the columns rotated by a
+            # different amount every time: the cache goes by the content of the index arrays, not by their addresses);
+            # the values stay where they are - these calls are timed, not checked
+            c0 = 1000 * (len(fresh) * 4 + r + 1)
+            j0 = np.zeros(1, np.int32)
+            hip_abi.check(lib.bidmat_memcpy_d2h(j0.ctypes.data, d_jc.ptr + 4 * c0, 4))
+            j0 = int(j0[0])
             f_ir, f_ic = DeviceArray(nnz, np.int32), DeviceArray(nnz, np.int32)
-            hip_abi.check(lib.bidmat_memcpy_d2d(f_ir.ptr, d_ir.ptr, 4 * nnz))
-            hip_abi.check(lib.bidmat_memcpy_d2d(f_ic.ptr, d_ic.ptr, 4 * nnz))
+            for dst, src in ((f_ir, d_ir), (f_ic, d_ic)):
+                hip_abi.check(lib.bidmat_memcpy_d2d(dst.ptr, src.ptr + 4 * j0, 4 * (nnz - j0)))
+                hip_abi.check(lib.bidmat_memcpy_d2d(dst.ptr + 4 * (nnz - j0), src.ptr, 4 * j0))
+            hip_abi.check(lib.bidmat_index_shift(f_ic.ptr, nnz - j0, -c0, None))
+            hip_abi.check(lib.bidmat_index_shift(f_ic.ptr + 4 * (nnz - j0), j0, ncols - c0, None))
             _, outbuf, call = [c for c in calls(f_ir.ptr, f_ic.ptr) if c[0] == opname][0]
             ts.append(timed(outbuf, call, opname))
             f_ir.free(); f_ic.free()

@@ -82,7 +82,6 @@ inline int finish_blocking(hipError_t launch_err) {
 struct CacheEntry {
     int device;
     int ncols, nnz, nrows, k_hint;
-    const int *ir, *ic;                     // where the pattern lay when the entry was made
     unsigned long long fa, fb;
     int col_uses;                           // A*S / DDS calls that met this pattern
     std::shared_ptr<bidmat_plan> plan;      // callers hold a reference while they use the plan (may be empty)
@@ -132,8 +131,9 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
         // panels are sized for k_hint: a request that names k only takes a plan built for that k
         const bool k_ok = k_hint <= 0 || (it->k_hint > 0 ? it->k_hint : 256) == k_hint;
+        // (no addresses in the key: the same pattern uploaded into other buffers is the same pattern)
         if (k_ok && it->device == dev && it->ncols == ncols && it->nnz == nnz && it->nrows == nrows &&
-            it->ir == ir && it->ic == ic && it->fa == h[0] && it->fb == h[1]) {
+            it->fa == h[0] && it->fb == h[1]) {
             hit = it;
             break;
         }
@@ -141,7 +141,7 @@ hipError_t cached_plan(int ncols, int nnz, const int* ir, const int* ic, int k_h
     if (hit == g_cache.end()) {
         const size_t cap = (size_t)std::max(1, bm::g_cache_plans.load());
         while (g_cache.size() >= cap) g_cache.pop_back();           // its plan is freed when its last user lets go
-        g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, ir, ic, h[0], h[1], 0, PlanRef()});
+        g_cache.push_front(CacheEntry{dev, ncols, nnz, nrows, k_hint, h[0], h[1], 0, PlanRef()});
     } else {
         g_cache.splice(g_cache.begin(), g_cache, hit);
     }

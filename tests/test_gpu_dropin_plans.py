@@ -350,3 +350,32 @@ def test_static_dds_from_two_threads_on_one_stream(hip):
                 assert np.array_equal(o.numpy(), j["want"])
             j["d"].free()
     hip_abi.check(hip.bidmat_stream_destroy(st))
+
+
+def test_the_cache_goes_by_the_content_of_the_index_arrays(hip):
+    """The same pattern uploaded into other device arrays is the same pattern: the second bidmat_dsmult on it runs
+    through the cached plan's class order (other bits than the plain kernel's stored order), whichever arrays hold it."""
+    rng = np.random.default_rng(77)
+    k, nrows, ncols = 256, 900, 400                             # from k = 256 on A*S takes the class order in passes
+    hip_abi.check(hip.bidmat_release_caches())
+    with Options(hip, col_classes=1, cache_cols_after=2):
+        data, ir, jc = zipf_pattern(rng, nrows, ncols, 20, 80)
+        nnz = int(ir.size)
+        ic = expand_cols(jc)
+        A = rng.standard_normal(k * nrows).astype(np.float32)
+        d1 = Dev(A=A, data=data, ir=ir, ic=ic)
+        d2 = Dev(ir=ir, ic=ic)                                  # the same pattern at other addresses
+        assert d1.ir.ptr != d2.ir.ptr and d1.ic.ptr != d2.ic.ptr
+        outs = []
+        for which in (d1, d2, d1, d2):
+            Cm = DeviceArray.zeros(k * ncols)
+            hip_abi.check(hip.bidmat_dsmult(k, ncols, nnz, d1.A.ptr, d1.data.ptr, which.ir.ptr, which.ic.ptr, Cm.ptr))
+            outs.append(Cm.numpy())
+            Cm.free()
+        ref64, sa = oracle.fsmult_f64(A, k, data, ir, jc)
+        for o in outs:
+            close(o, ref64, sa, "bidmat_dsmult")
+        assert not np.array_equal(outs[0], outs[1]), "the second call (other arrays, same pattern) still ran the plain kernel"
+        assert np.array_equal(outs[1], outs[2]) and np.array_equal(outs[2], outs[3])
+        d1.free(); d2.free()
+    hip_abi.check(hip.bidmat_release_caches())
