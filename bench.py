@@ -515,7 +515,11 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
         ch["e_step_dds_op_ms"] = round(_timed(lib, lambda: lib.bidmat_dds_plan(plan, k, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_v.ptr, 3, d_Q2.ptr, 0, stream), stream, 5), 4)
         ch["e_step_dsmult_ms"] = round(_timed(lib, lambda: lib.bidmat_dsmult_plan(plan, k, d_A.ptr, d_Q2.ptr, d_ir.ptr, d_jc.ptr, d_C2.ptr, 0, stream), stream, 5), 4)
         ch["e_step_two_calls_ms"] = round(ch["e_step_dds_op_ms"] + ch["e_step_dsmult_ms"], 4)
+        c_two_plan = d_C2.numpy()              # what the two plan calls left
         ch["e_step_one_launch_ms"] = round(_timed(lib, lambda: lib.bidmat_dds_dsmult_csc(k, ncols, nnz, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_v.ptr, 3, None, d_C2.ptr, 0, stream), stream, 5), 4)
+        ch["e_step_one_launch_through_plan_ms"] = round(_timed(lib, lambda: lib.bidmat_dds_dsmult_plan(plan, k, d_A.ptr, d_B.ptr, d_ir.ptr, d_jc.ptr, d_v.ptr, 3, None, d_C2.ptr, 0, stream), stream, 5), 4)
+        ch["e_step_through_plan_same_bits_as_two_calls"] = bool(np.array_equal(c_two_plan.view(np.uint32), d_C2.numpy().view(np.uint32)))
+        del c_two_plan
         ch["m_step_dsmultT_ms"] = round(_timed(lib, lambda: lib.bidmat_dsmultT_plan(plan, k, d_B.ptr, d_Q2.ptr, d_G2.ptr, 0, stream), stream, 5), 4)
         ch["m_step_two_calls_ms"] = round(ch["e_step_dds_op_ms"] + ch["m_step_dsmultT_ms"], 4)
         g_two = _without_dense_block(lib, lambda: lib.bidmat_dsmultT_plan(plan, k, d_B.ptr, d_Q2.ptr, d_G2.ptr, 0, stream), stream, d_G2)

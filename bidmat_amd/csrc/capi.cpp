@@ -532,6 +532,30 @@ API int bidmat_dds_dsmult_csc(int k, int ncols, int nnz, const float* A, const f
     return (int)bm::fused_columns(k, ncols, nnz, A, B, V, Sir, Sjc, opn, Q, C, beta, as_stream(stream));
 }
 
+API int bidmat_dds_dsmult_plan(bidmat_plan* plan, int k, const float* A, const float* B, const int* Sir, const int* Sjc,
+                               const float* V, int opn, float* Q, float* C, int beta, void* stream) {
+    auto lock = bm::device_lock();
+    if (!plan || k < 0 || opn < 0 || opn > 14 || (beta != 0 && beta != 1)) return kInvalid;
+    if (!plan_on_current_device(plan)) return (int)hipErrorInvalidDevice;
+    if (!(plan->sides & bm::PLAN_COLS)) return kInvalid;
+    if (k == 0 || plan->ncols == 0) return 0;
+    if (!Sjc || !C || !A || !B || (plan->nnz > 0 && (!Sir || !V))) return kInvalid;
+    if (Q && V != Q && ranges_overlap(V, Q, plan->nnz)) return kInvalid;      // in place (Q == V) or apart
+    const int bad = plan_pattern_ok(plan, Sir, Sjc);
+    if (bad) return bad;
+    hipStream_t s = as_stream(stream);
+    // with a class order (and no hot-row ranks in it, no column too long for one running sum per pass): in passes
+    const int nphase = bm::opt_class_phases();
+    const bool phased = plan->ncls == 8 && plan->hcap == 0 && nphase > 0 && plan->maxlen <= kMaxPhasedColumn && plan->nnz > 0;
+    if (phased) {
+        const hipError_t e = bm::fused_columns_phased(k, plan->ncols, A, B, V, plan->cir, plan->cperm, plan->cptr, nphase, opn,
+                                                      Q, C, beta, s);
+        return (int)e;
+    }
+    const bm::ColTable tab = col_table(plan);
+    return (int)bm::fused_columns(k, plan->ncols, plan->nnz, A, B, V, Sir, Sjc, opn, Q, C, beta, s, &tab);
+}
+
 API int bidmat_dds0(int nrows, int ncols, const float* A, const float* B, const int* Cir, const int* Cjc,
                     float* P) {
     auto lock = bm::device_lock();

@@ -132,6 +132,13 @@ JFN(jint, ddsDsmultCsc)(JNIEnv*, jclass, jint k, jint nc, jint nnz, jlong A, jlo
                                   P(const float, V), opn, P(float, Q), P(float, C), beta, nullptr);
     return e ? e : bidmat_stream_synchronize(nullptr);
 }
+// the same through a plan's column side (in passes over the row classes when the plan has a class order)
+JFN(jint, ddsDsmultPlan)(JNIEnv*, jclass, jlong plan, jint k, jlong A, jlong B, jlong Sir, jlong Sjc, jlong V, jint opn, jlong Q,
+                         jlong C, jint beta) {
+    int e = bidmat_dds_dsmult_plan(P(bidmat_plan, plan), k, P(const float, A), P(const float, B), P(const int, Sir),
+                                   P(const int, Sjc), P(const float, V), opn, P(float, Q), P(float, C), beta, nullptr);
+    return e ? e : bidmat_stream_synchronize(nullptr);
+}
 // S^T * A and S * A (replace the cusparseScsrmm calls of GSMat.SDTMult / SDMult, GSMat.scala:265-313)
 JFN(jint, sdtmultCsc)(JNIEnv*, jclass, jint nr, jint nc, jint nnz, jint p, jlong Sdata, jlong Sir, jlong Sjc, jlong A,
                       jint lda, jlong C, jint ldc) {

@@ -135,6 +135,11 @@ hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_star
 // Q[j] * A[:, ir[j]]; segments and order of additions of dsmult_csc. hipErrorInvalidValue when k does not fit one pass.
 hipError_t fused_columns(int k, int ncols, int nnz, const float* A, const float* B, const float* vals, const int* ir,
                          const int* jc, int opn, float* Q, float* C, int beta, hipStream_t s, const ColTable* tab = nullptr);
+// The same over a plan's class-ordered pattern (no hot-row ranks) in nphase passes over disjoint row classes, like
+// dsmult_phased: q as above (bit for bit), C's additions pass by pass and class by class.
+hipError_t fused_columns_phased(int k, int ncols, const float* A, const float* B, const float* vals, const int* cir,
+                                const int* cperm, const int* cptr, int nphase, int opn, float* Q, float* C, int beta,
+                                hipStream_t s);
 // C[:,r] = beta*C[:,r] + sum over q in [rowptr[r], rowptr[r+1]) of partial[rowseg[q]*k ..]
 // rowptr2 / rowseg2 / flag (nullable): the table to use instead while *flag == 0.
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,

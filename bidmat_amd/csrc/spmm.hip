@@ -456,7 +456,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fused_cols(GatherArgs a) {
     float* outp;
     bool accumulate;
     if (w < a.nfirst) {
-        const int s = a.ptr[w], e = a.ptr[w + 1];
+        // (on a class-ordered pattern: the classes [poff, poff + pspan) of the column's 16 groups; plain CSC: 1, 0, 1)
+        const long long pi = w * a.pstride + a.poff;
+        const int s = a.ptr[pi], e = a.ptr[pi + a.pspan];
         col = (int)w;
         jstart = s;
         jend = (e - s > a.seglen) ? s + a.seglen : e;
@@ -511,7 +513,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fused_cols(GatherArgs a) {
         float keep;
         if (rem >= 64) keep = fused_chunk<W, V, LPN, true>(a, crow, cval, 64, g, l, eld, ev, rr, acc);
         else keep = fused_chunk<W, V, LPN, false>(a, crow, cval, rem, g, l, eld, ev, rr, acc);
-        if (a.qout != nullptr && q < rem) a.qout[j0 + q] = keep;
+        if (a.qout != nullptr && q < rem) a.qout[a.perm != nullptr ? a.perm[j0 + q] : j0 + q] = keep;
         crow = nrow;
         cval = nval;
         j0 += 64;
@@ -939,6 +941,49 @@ hipError_t fused_columns(int k, int ncols, int nnz, const float* A, const float*
         err = hipGetLastError();
     }
     return err;
+}
+
+// The chain by columns over a class-ordered pattern in `nphase` passes (see dsmult_phased): pass p takes the row
+// classes [8p/nphase, 8(p+1)/nphase) of every column, computes their products q (written through cperm) and adds their
+// share to C, so that every L2 sees 1/nphase of the rows at a time; the first pass honours beta, the others accumulate.
+hipError_t fused_columns_phased(int k, int ncols, const float* A, const float* B, const float* vals, const int* cir,
+                                const int* cperm, const int* cptr, int nphase, int opn, float* Q, float* C, int beta,
+                                hipStream_t s) {
+    if (k <= 0 || ncols <= 0) return hipSuccess;
+    if (nphase != 1 && nphase != 2 && nphase != 4 && nphase != 8) return hipErrorInvalidValue;
+    Shape sh = pick_shape(k, aligned16(A) && aligned16(B) && aligned16(C));
+    if (sh.V > 4) return hipErrorInvalidValue;          // one pass must cover k
+    GatherArgs a;
+    init_args(a);
+    a.k = k; a.lda = k; a.ldo = k; a.nfirst = ncols; a.seglen = 0x7fffffff;
+    a.A = A; a.vals = vals; a.idx = cir; a.perm = cperm; a.ptr = cptr; a.ovf = nullptr;
+    a.out = C; a.partial = nullptr;
+    a.R = B; a.ldr = k; a.opn = opn; a.qout = Q;
+    a.pstride = 16; a.pspan = 16 / nphase;
+    const long long nblk = ((long long)ncols + BM_WAVES_PER_BLOCK - 1) / BM_WAVES_PER_BLOCK;
+    if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)nblk), block(BM_BLOCK);
+    for (int p = 0; p < nphase; ++p) {
+        a.poff = p * a.pspan;
+        a.beta = p == 0 ? beta : 1;
+        bool launched = false;
+#define BM_CASE(W_, V_, L_)                                                              \
+        if (!launched && sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                     \
+            hipLaunchKernelGGL((k_fused_cols<W_, V_, L_>), grid, block, 0, s, a);        \
+            launched = true;                                                             \
+        }
+#define BM_CASES(W_)                                                                     \
+        BM_CASE(W_, 1, 1) BM_CASE(W_, 1, 2) BM_CASE(W_, 1, 4) BM_CASE(W_, 1, 8) BM_CASE(W_, 1, 16) \
+        BM_CASE(W_, 1, 32) BM_CASE(W_, 1, 64) BM_CASE(W_, 2, 64) BM_CASE(W_, 4, 64)
+        BM_CASES(1)
+        BM_CASES(4)
+#undef BM_CASES
+#undef BM_CASE
+        if (!launched) return hipErrorInvalidValue;
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return err;
+    }
+    return hipSuccess;
 }
 
 hipError_t reduce_segments(int k, int nrows, const int* rowptr, const int* rowseg,

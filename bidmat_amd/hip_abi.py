@@ -52,6 +52,7 @@ SIGNATURES = {
     "bidmat_spsum_rows_plan": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "bidmat_dds_dsmultT_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, C.c_int, vp, vp, C.c_int, vp]),
     "bidmat_dds_dsmult_csc": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp, vp, C.c_int, vp]),
+    "bidmat_dds_dsmult_plan": (C.c_int, [vp, C.c_int, vp, vp, vp, vp, vp, C.c_int, vp, vp, C.c_int, vp]),
     "bidmat_spsum_rows_csc": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, C.c_int, vp]),
     "bidmat_csc_expand_cols": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
     "bidmat_csc_implicit_rows": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),

@@ -260,6 +260,13 @@ int bidmat_dds_dsmultT_plan(bidmat_plan *plan, int k, const float *A, const floa
  * values in stored order) is only written when Q != NULL and may be V itself.  The results are those of
  * bidmat_dds_csc_op followed by bidmat_dsmult_csc, bit for bit.  k must fit one pass (k <= 1024 with 16-byte aligned
  * operands and k % 4 == 0, else k <= 256): otherwise hipErrorInvalidValue, and the two calls remain. */
+/* The same chain through a plan (column side): with a row-class ordering of the columns (and no column longer than 8192
+ * nonzeros) it runs in the passes of bidmat_dsmult_plan ("class_phases"), each pass computing the products and adding the
+ * share of its row classes, so that the L2s hold more of the rows that matter; Q has the bits of bidmat_dds_plan with
+ * the op, C those of bidmat_dsmult_plan fed with that Q (a fixed order that depends on the pattern alone).  Without a class
+ * ordering it is bidmat_dds_dsmult_csc with the plan's table of long columns.  No counterpart in the reference. */
+int bidmat_dds_dsmult_plan(bidmat_plan *plan, int k, const float *A, const float *B, const int *Sir, const int *Sjc,
+                           const float *V, int opn, float *Q, float *C, int beta, void *stream);
 int bidmat_dds_dsmult_csc(int k, int ncols, int nnz, const float *A, const float *B, const int *Sir, const int *Sjc,
                           const float *V, int opn, float *Q, float *C, int beta, void *stream);
 /* Number of extra wave segments of the plan's long columns (0: every column fits one segment). */

@@ -215,3 +215,99 @@ def test_column_chain_against_the_oracle_and_refusals(hip):
     d.zeros("C", k * ncols)
     assert hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, None, d.C.ptr, 0, None) == 1
     d.free()
+
+
+# ------------------------------------------------------------------ the chain by columns through a plan
+@pytest.mark.parametrize("k,nrows,ncols,mean_len", [(32, 300, 500, 20), (64, 2000, 3000, 30), (100, 2000, 3000, 30), (128, 3000, 5000, 60),
+                                                    (256, 5000, 20000, 60), (250, 300, 500, 20), (512, 1000, 2000, 40), (1024, 500, 1000, 40)])
+@pytest.mark.parametrize("classes,phases", [(1, 2), (1, 4), (1, 8), (1, 1), (0, 2)], ids=["2passes", "4passes", "8passes", "1pass", "no_class_order"])
+def test_column_chain_through_a_plan_has_the_bits_of_the_two_plan_calls(hip, k, nrows, ncols, mean_len, classes, phases):
+    """bidmat_dds_dsmult_plan against bidmat_dds_plan (with the op) + bidmat_dsmult_plan on the same plan: Q and C bit for bit,
+    whether the plan has a class order (then both forms add a column's terms pass by pass, class by class) or not."""
+    rng = np.random.default_rng(3000 * k + nrows + phases)
+    ir, jc = zipf_csc(rng, nrows, ncols, mean_len)
+    nnz = ir.size
+    A = (0.01 + rng.random(k * nrows)).astype(np.float32)
+    B = (0.01 + rng.random(k * ncols)).astype(np.float32)
+    v = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+    C0 = rng.standard_normal(k * ncols).astype(np.float32)
+    old = {n: hip.bidmat_get_option(n) for n in (b"col_classes", b"class_phases", b"class_hot")}
+    hip_abi.check(hip.bidmat_set_option(b"col_classes", classes))
+    hip_abi.check(hip.bidmat_set_option(b"class_phases", phases))
+    hip_abi.check(hip.bidmat_set_option(b"class_hot", 0))        # no hot-row ranks in the class order: the passes apply for every k
+    try:
+        d = Dev(A=A, B=B, v=v, ir=ir, jc=jc)
+        plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+        assert int(hip.bidmat_plan_info(plan, b"col_classes")) == (8 if classes else 0)
+        for beta in (0, 1):
+            d.put("C1", C0); d.put("C2", C0); d.put("C3", C0)
+            d.zeros("Q1", max(nnz, 1))
+            d.put("Q2", np.full(max(nnz, 1), -5.0, np.float32))
+            hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.Q1.ptr, 0, None))
+            hip_abi.check(hip.bidmat_dsmult_plan(plan, k, d.A.ptr, d.Q1.ptr, d.ir.ptr, d.jc.ptr, d.C1.ptr, beta, None))
+            hip_abi.check(hip.bidmat_dds_dsmult_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.Q2.ptr,
+                                                     d.C2.ptr, beta, None), "column chain through the plan")
+            hip_abi.check(hip.bidmat_dds_dsmult_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, None,
+                                                     d.C3.ptr, beta, None), "without the products")
+            hip_abi.check(hip.bidmat_synchronize())
+            assert np.array_equal(d.Q2.numpy()[:nnz].view(np.uint32), d.Q1.numpy()[:nnz].view(np.uint32)), "Q, beta %d" % beta
+            assert np.array_equal(d.C2.numpy().view(np.uint32), d.C1.numpy().view(np.uint32)), "C, beta %d" % beta
+            assert np.array_equal(d.C3.numpy().view(np.uint32), d.C1.numpy().view(np.uint32)), "C without Q, beta %d" % beta
+        # in place (Q == V), then against the oracle
+        vq = d.put("vq", v)
+        d.zeros("C4", k * ncols)
+        hip_abi.check(hip.bidmat_dds_dsmult_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, vq.ptr, OP_DIV, vq.ptr, d.C4.ptr, 0, None))
+        hip_abi.check(hip.bidmat_synchronize())
+        assert np.array_equal(vq.numpy()[:nnz].view(np.uint32), d.Q1.numpy()[:nnz].view(np.uint32))
+        q32 = d.Q1.numpy()[:nnz]
+        ref64, sa = oracle.fsmult_f64(A, k, q32, ir, jc, nthreads=8)
+        ok, worst = oracle.within_tolerance(d.C4.numpy(), ref64, sa, 1e-4)
+        assert ok, worst
+        r32 = oracle.dds(A, B, k, ir, jc, nthreads=8)[0]
+        assert np.allclose(q32, v / r32, rtol=2e-5, atol=0)
+        # refusals: a plan without a column side, an op code outside the table, overlapping V and Q, k beyond one pass
+        assert hip.bidmat_dds_dsmult_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, 15, None, d.C4.ptr, 0, None) == 1
+        if nnz > 1:
+            assert hip.bidmat_dds_dsmult_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.v.ptr + 4, d.C4.ptr, 0, None) == 1
+        hip_abi.check(hip.bidmat_plan_destroy(plan))
+        d.free()
+    finally:
+        for n, val in old.items():
+            hip_abi.check(hip.bidmat_set_option(n, val))
+
+
+def test_column_chain_through_a_plan_with_long_columns_and_refusals(hip):
+    """Columns longer than a wave segment (the plan's table of extra segments, no passes) and k beyond one pass."""
+    rng = np.random.default_rng(91)
+    k, nrows, ncols = 64, 3000, 200
+    ir, jc = zipf_csc(rng, nrows, ncols, 400)
+    nnz = ir.size
+    A = (0.01 + rng.random(k * nrows)).astype(np.float32)
+    B = (0.01 + rng.random(k * ncols)).astype(np.float32)
+    v = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+    old = {n: hip.bidmat_get_option(n) for n in (b"seglen", b"col_classes")}
+    hip_abi.check(hip.bidmat_set_option(b"seglen", 64))
+    hip_abi.check(hip.bidmat_set_option(b"col_classes", 0))
+    try:
+        d = Dev(A=A, B=B, v=v, ir=ir, jc=jc)
+        d.zeros("Q1", nnz); d.zeros("Q2", nnz); d.zeros("C1", k * ncols); d.zeros("C2", k * ncols)
+        plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+        assert hip.bidmat_plan_overflow_segments(plan) > 0
+        hip_abi.check(hip.bidmat_dds_dsmult_csc(k, ncols, nnz, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.Q1.ptr, d.C1.ptr, 0, None))
+        hip_abi.check(hip.bidmat_dds_dsmult_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, d.Q2.ptr, d.C2.ptr, 0, None))
+        hip_abi.check(hip.bidmat_synchronize())
+        assert np.array_equal(d.Q2.numpy().view(np.uint32), d.Q1.numpy().view(np.uint32))
+        assert np.array_equal(d.C2.numpy().view(np.uint32), d.C1.numpy().view(np.uint32))
+        hip_abi.check(hip.bidmat_plan_destroy(plan))
+        # k beyond one pass
+        d.free()
+        kk = 1028
+        d = Dev(A=rng.random(kk * nrows).astype(np.float32), B=rng.random(kk * ncols).astype(np.float32), v=v, ir=ir, jc=jc)
+        d.zeros("C", kk * ncols)
+        plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, kk)
+        assert hip.bidmat_dds_dsmult_plan(plan, kk, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, OP_DIV, None, d.C.ptr, 0, None) == 1
+        hip_abi.check(hip.bidmat_plan_destroy(plan))
+        d.free()
+    finally:
+        for n, val in old.items():
+            hip_abi.check(hip.bidmat_set_option(n, val))
