@@ -216,34 +216,52 @@ __global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int
 #pragma unroll
     for (int s = 0; s < NSW; ++s) ev[s] = s * 32 + n < k;
     unsigned worst = 0;              // largest magnitude bits of A met: not finite from 0x7f800000 on
-    auto ldpos = [&](int c) -> int { const int cc = c + half; return cc < c1 ? dpos[(size_t)cc * nd + g * 32 + n] : -1; };
-    auto ldval = [&](int p) -> float { return p >= 0 ? vals[p] : 0.f; };
-    auto ldA = [&](int c, float (&x)[NSW]) {
-        const int cc = c + half;
-        const float* p = A + (size_t)(cc < c1 ? cc : (int)c0) * (size_t)k + n;
+    // Every load is issued unconditionally, from a clamped address, and its result is masked only where it is consumed,
+    // DEPTH steps later: a branch around a load (or a select right behind it) makes the compiler wait for every load
+    // in flight before each step's matrix instructions, which takes the steps meant to be under way out of flight.
+    const int clast = c1 - 1;
+    auto rawpos = [&](int c) -> int { const int cc = c + half; return dpos[(size_t)(cc < c1 ? cc : clast) * nd + g * 32 + n]; };
+    auto rawval = [&](int p) -> float { return vals[p >= 0 ? p : 0]; };
+    int eoff[NSW];
 #pragma unroll
-        for (int s = 0; s < NSW; ++s) x[s] = (ev[s] && cc < c1) ? p[s * 32] : 0.f;
+    for (int s = 0; s < NSW; ++s) eoff[s] = ev[s] ? s * 32 : -n;          // an element past k: the column's first instead
+    auto rawA = [&](int c, float (&x)[NSW]) {
+        const int cc = c + half;
+        const float* p = A + (size_t)(cc < c1 ? cc : clast) * (size_t)k + n;
+#pragma unroll
+        for (int s = 0; s < NSW; ++s) x[s] = p[eoff[s]];
     };
     float a[DEPTH][NSW], bv[DEPTH];
-    int pos[DEPTH + 1];
+    int bp[DEPTH];                   // the position each bv was fetched from (-1: no nonzero there)
+    // the positions run two steps ahead of the values fetched through them: a wait for the load issued last would
+    // be a wait for every load in flight
+    int pos[DEPTH + 2];
 #pragma unroll
-    for (int d = 0; d < DEPTH + 1; ++d) pos[d] = ldpos((int)c0 + 2 * d);
+    for (int d = 0; d < DEPTH + 2; ++d) pos[d] = rawpos((int)c0 + 2 * d);
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) { bv[d] = ldval(pos[d]); ldA((int)c0 + 2 * d, a[d]); }
+    for (int d = 0; d < DEPTH; ++d) {
+        bp[d] = ((int)c0 + 2 * d + half < c1) ? pos[d] : -1;
+        bv[d] = rawval(bp[d]);
+        rawA((int)c0 + 2 * d, a[d]);
+    }
     for (int c = (int)c0; c < c1; c += 2 * DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             // take slot d (columns c + 2d and c + 2d + 1), refill it for the columns 2 DEPTH further on
+            const bool in = c + 2 * d + half < c1;
             float ax[NSW];
 #pragma unroll
-            for (int s = 0; s < NSW; ++s) ax[s] = a[d][s];
-            const float bx = bv[d];
-            const int pnext = pos[DEPTH];
+            for (int s = 0; s < NSW; ++s) ax[s] = (ev[s] && in) ? a[d][s] : 0.f;
+            const float bx = bp[d] >= 0 ? bv[d] : 0.f;
+            const int cn = c + 2 * (d + DEPTH);
+            const int pnext = (cn + half < c1) ? pos[DEPTH] : -1;
 #pragma unroll
-            for (int q = 0; q < DEPTH; ++q) pos[q] = pos[q + 1];
-            pos[DEPTH] = ldpos(c + 2 * (d + DEPTH + 1));
-            bv[d] = ldval(pnext);
-            ldA(c + 2 * (d + DEPTH), a[d]);
+            for (int q = 0; q < DEPTH + 1; ++q) pos[q] = pos[q + 1];
+            pos[DEPTH + 1] = rawpos(cn + 4);
+            bp[d] = pnext;
+            bv[d] = rawval(pnext);
+            rawA(cn, a[d]);
+            __builtin_amdgcn_sched_barrier(0);       // the refill is on its way before the matrix instructions start
 #pragma unroll
             for (int s = 0; s < NSW; ++s) {
                 const unsigned m = __float_as_uint(ax[s]) & 0x7fffffffu;
