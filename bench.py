@@ -43,9 +43,9 @@ HBM_PEAK_GBS = 8000.0
 # was taken on (concatenated); it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dsmultT", 100003320): (33.9e9, ("bidmat_amd/csrc/spmm.hip", "bidmat_amd/csrc/dense_rows.hip"), "a52162aa7c6bafc6",
+    ("headline", "dsmultT", 100003320): (33.9e9, ("bidmat_amd/csrc/spmm.hip", "bidmat_amd/csrc/dense_rows.hip"), "0202f393a97265ba",
                                          "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, ("bidmat_amd/csrc/spmm.hip",), "f8f54a08b059f7c2",
+    ("C4", "dsmult", 38900534): (163.1e9, ("bidmat_amd/csrc/spmm.hip",), "651845315168280a",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 
