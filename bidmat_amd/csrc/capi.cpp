@@ -39,12 +39,14 @@ std::atomic<int> g_dense_rows{128};
 std::atomic<int> g_dense_min_pct{15};
 std::atomic<int> g_dense_min_nnz{1 << 22};
 std::atomic<int> g_dense_cb{0};
+std::atomic<int> g_scalar_values{1};
 }  // namespace
 int opt_plan_pool_mb() { return g_plan_pool_mb.load(std::memory_order_relaxed); }
 int opt_dense_rows() { return g_dense_rows.load(std::memory_order_relaxed); }
 int opt_dense_min_pct() { return g_dense_min_pct.load(std::memory_order_relaxed); }
 int opt_dense_min_nnz() { return g_dense_min_nnz.load(std::memory_order_relaxed); }
 int opt_dense_cb() { return g_dense_cb.load(std::memory_order_relaxed); }
+int opt_scalar_values() { return g_scalar_values.load(std::memory_order_relaxed); }
 int opt_plan_builder() { return g_plan_builder.load(std::memory_order_relaxed); }
 int opt_class_shift() { return g_class_shift.load(std::memory_order_relaxed); }
 int opt_rowsum_form() { return g_rowsum_form.load(std::memory_order_relaxed); }
@@ -1147,6 +1149,11 @@ API int bidmat_set_option(const char* name, long long value) {
         bm::g_dense_cb.store((int)value);
         return 0;
     }
+    if (!strcmp(name, "scalar_values")) {
+        if (value != 0 && value != 1) return kInvalid;
+        bm::g_scalar_values.store((int)value);
+        return 0;
+    }
     return kInvalid;
 }
 
@@ -1172,6 +1179,7 @@ API long long bidmat_get_option(const char* name) {
     if (!strcmp(name, "dense_min_pct")) return bm::opt_dense_min_pct();
     if (!strcmp(name, "dense_min_nnz")) return bm::opt_dense_min_nnz();
     if (!strcmp(name, "dense_cb")) return bm::opt_dense_cb();
+    if (!strcmp(name, "scalar_values")) return bm::opt_scalar_values();
     return -2;
 }
 

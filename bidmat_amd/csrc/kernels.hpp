@@ -24,6 +24,7 @@ int opt_dense_rows();  // rows a plan may treat as a dense block of A *^ S (0 = 
 int opt_dense_min_pct(); // a row counts as dense when it has a nonzero in at least this percentage of the columns
 int opt_dense_min_nnz(); // patterns with fewer nonzeros get no dense block
 int opt_dense_cb();    // columns per block of the dense product (0 = chosen from the column count)
+int opt_scalar_values();   // A *^ S over a plan fetches the caller's values by scalar loads (1) or by a gather per lane (0)
 
 // ---- CSC utilities (csc_util.hip)
 hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);

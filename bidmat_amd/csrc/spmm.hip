@@ -64,7 +64,7 @@ struct Unroll { static constexpr int raw = 8 / V; static constexpr int U = raw <
 
 // Loads this lane's nonzero of a chunk: lane (g,l) holds nonzero q = l*NG + g, so group g meets
 // its nonzeros q = it*NG + g in lane l == it of its own group. Lanes past `rem` keep (0, 0).
-template <bool PLAN>
+template <bool PLAN, bool SV = false>
 __device__ __forceinline__ void load_chunk(const GatherArgs& a, int j0, int ahead, int rem, int q, int& myrow,
                                            float& myval) {
     myrow = 0;
@@ -72,11 +72,19 @@ __device__ __forceinline__ void load_chunk(const GatherArgs& a, int j0, int ahea
     if (q < rem) {
         const int p = j0 + ahead + q;
         myrow = a.idx[p];
-        myval = a.perm != nullptr ? a.vals[a.perm[p]] : a.vals[p];     // perm == nullptr: vals is in the order of idx
+        if constexpr (SV) myval = __int_as_float(a.perm[p]);          // the position only: gather_chunk fetches the value
+        else myval = a.perm != nullptr ? a.vals[a.perm[p]] : a.vals[p];     // perm == nullptr: vals is in the order of idx
     }
 }
 
-template <int W, int V, int LPN, bool FULL, bool TILE>
+// SV ("scalar values", plan order with the values in the caller's order): a nonzero's value is fetched by a scalar load
+// from its position, wave-uniform like the row index, instead of one 4-byte gather per lane and chunk. A lane-wise gather
+// of 64 values touches 64 cache lines, one look-up each in the per-CU vector cache that the row gathers already keep
+// busy (an eighth of their line requests at k = 256, a quarter at k = 128); the scalar cache is a path of its own to L2.
+// Read-only use: the values were written by earlier launches, and nothing here writes through that cache.
+typedef const float __attribute__((address_space(4))) scalar_float;
+
+template <int W, int V, int LPN, bool FULL, bool TILE, bool SV = false>
 __device__ __forceinline__ void gather_chunk(const GatherArgs& a, int myrow, float myval, int rem, int g, int l,
                                              const int (&eld)[V], Vec<W> (&acc)[V]) {
     constexpr int NG = 64 / LPN;
@@ -104,11 +112,28 @@ __device__ __forceinline__ void gather_chunk(const GatherArgs& a, int myrow, flo
             int r;
             if constexpr (LPN == 64) {
                 r = __builtin_amdgcn_readlane(myrow, it);
-                vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myval), it));
+                if constexpr (SV) {
+                    const int pp = __builtin_amdgcn_readlane(__float_as_int(myval), it);
+                    const float sv = ((scalar_float*)a.vals)[pp];
+                    vv[u] = (FULL || it < rem) ? sv : 0.f;       // a slot past the end holds position 0: not its value
+                } else {
+                    vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myval), it));
+                }
             } else {
                 const int src = g * LPN + it;
                 r = lane_read(myrow, src);
-                vv[u] = lane_read(myval, src);
+                if constexpr (SV) {
+                    float sv = 0.f;
+#pragma unroll
+                    for (int gg = 0; gg < NG; ++gg) {
+                        const int pp = __builtin_amdgcn_readlane(__float_as_int(myval), gg * LPN + it);
+                        const float x = ((scalar_float*)a.vals)[pp];
+                        sv = g == gg ? x : sv;
+                    }
+                    vv[u] = (FULL || (it * NG + g) < rem) ? sv : 0.f;
+                } else {
+                    vv[u] = lane_read(myval, src);
+                }
             }
             const float* ap = a.A + (size_t)r * (size_t)a.lda;
             if (!FULL || TILE) {
@@ -153,7 +178,7 @@ __device__ __forceinline__ Vec<4> vec_xor_add<4>(Vec<4> x, int m) {
     return x;
 }
 
-template <int W, int V, int LPN, bool PLAN>
+template <int W, int V, int LPN, bool PLAN, bool SV = false>
 __device__ __forceinline__ void gather_axpy_body(const GatherArgs& a) {
     constexpr int KT = W * V * LPN;      // elements of a dense column covered per pass
     const int lane = threadIdx.x & 63;
@@ -241,17 +266,17 @@ __device__ __forceinline__ void gather_axpy_body(const GatherArgs& a) {
         int rem = jend - jstart, j0 = jstart;
         int crow;
         float cval;
-        load_chunk<PLAN>(a, j0, 0, rem, q, crow, cval);
+        load_chunk<PLAN, SV>(a, j0, 0, rem, q, crow, cval);
         while (rem > 0) {
             int nrow;
             float nval;
-            load_chunk<PLAN>(a, j0, 64, rem - 64, q, nrow, nval);
-            if (a.win_on) {
+            load_chunk<PLAN, SV>(a, j0, 64, rem - 64, q, nrow, nval);
+            if (!SV && a.win_on) {
                 if (rem >= 64) gather_chunk<W, V, LPN, true, true>(a, crow, cval, 64, g, l, eld, acc);
                 else gather_chunk<W, V, LPN, false, true>(a, crow, cval, rem, g, l, eld, acc);
             } else {
-                if (rem >= 64) gather_chunk<W, V, LPN, true, false>(a, crow, cval, 64, g, l, eld, acc);
-                else gather_chunk<W, V, LPN, false, false>(a, crow, cval, rem, g, l, eld, acc);
+                if (rem >= 64) gather_chunk<W, V, LPN, true, false, SV>(a, crow, cval, 64, g, l, eld, acc);
+                else gather_chunk<W, V, LPN, false, false, SV>(a, crow, cval, rem, g, l, eld, acc);
             }
             crow = nrow;
             cval = nval;
@@ -288,6 +313,11 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy(GatherArgs a) {
 template <int W, int V, int LPN>
 __global__ __launch_bounds__(BM_BLOCK) void k_gather_listed(GatherArgs a) {
     gather_axpy_body<W, V, LPN, true>(a);
+}
+// The walk over all segments of a plan with the values in the caller's order: each value by a scalar load (SV above).
+template <int W, int V, int LPN>
+__global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy_sv(GatherArgs a) {
+    gather_axpy_body<W, V, LPN, true, true>(a);
 }
 
 // ---- DDS, the elementwise step and A*^S in one walk over a plan's segments (an NMF update's
@@ -630,6 +660,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int ldc, in
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// narrower groups (k <= 32 with 4 floats per lane) would need 8 and more scalar loads per step
+constexpr int kScalarValuesMinLanes = 16;
+
 template <bool PLAN>
 hipError_t launch_gather(const Shape& sh, const GatherArgs& a, long long nwaves, hipStream_t s) {
     if (nwaves <= 0) return hipSuccess;
@@ -640,6 +673,8 @@ hipError_t launch_gather(const Shape& sh, const GatherArgs& a, long long nwaves,
     if (sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                                      \
         if (PLAN && a.seglist != nullptr)                                                \
             hipLaunchKernelGGL((k_gather_listed<W_, V_, L_>), grid, block, 0, s, a);     \
+        else if (PLAN && L_ >= kScalarValuesMinLanes && a.perm != nullptr && !a.win_on && opt_scalar_values()) \
+            hipLaunchKernelGGL((k_gather_axpy_sv<W_, V_, (L_ >= kScalarValuesMinLanes ? L_ : 64)>), grid, block, 0, s, a); \
         else                                                                             \
             hipLaunchKernelGGL((k_gather_axpy<W_, V_, L_, PLAN>), grid, block, 0, s, a); \
         return hipGetLastError();                                                        \

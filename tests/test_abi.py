@@ -61,7 +61,8 @@ def test_no_compute_without_gpu_helpers_work():
     for name, good, bad in ((b"seglen", 512, 0), (b"panel_kb", 1024, 1), (b"heavy_min", 4, 0), (b"col_classes", 1, 2),
                             (b"class_hot", 16, 5000), (b"class_threads", 512, 300), (b"class_strip", 8, 65),
                             (b"class_phases", 4, 3), (b"plan_keep_mb", 0, -1), (b"dense_rows", 64, 100),
-                            (b"dense_min_pct", 30, 0), (b"dense_min_nnz", 0, -1), (b"dense_cb", 64, -1)):
+                            (b"dense_min_pct", 30, 0), (b"dense_min_nnz", 0, -1), (b"dense_cb", 64, -1),
+                            (b"scalar_values", 0, 2)):
         old = lib.bidmat_get_option(name)
         assert old != -2, name
         assert lib.bidmat_set_option(name, bad) == 1 and lib.bidmat_get_option(name) == old, name

@@ -13,7 +13,7 @@ from util import dense_full, random_csc
 
 pytestmark = pytest.mark.gpu
 TUNABLES = ("seglen", "panel_kb", "heavy_min", "col_classes", "class_hot", "class_threads", "class_strip", "class_phases",
-            "dense_rows", "dense_min_pct", "dense_min_nnz", "dense_cb")
+            "dense_rows", "dense_min_pct", "dense_min_nnz", "dense_cb", "scalar_values")
 
 
 @pytest.mark.parametrize("seed0", [11, 12])
@@ -45,7 +45,8 @@ def test_plan_forms_under_random_shapes_and_settings(hip, seed0):
                      col_classes=int(rng.choice([-1, 0, 1, 1])), class_hot=int(rng.choice([-1, 0, 1, 3, 16])), class_threads=int(rng.choice([256, 512, 1024])),
                      class_strip=int(rng.choice([1, 3, 16, 64])), class_phases=int(rng.choice([0, 1, 2, 4, 8])),
                      dense_rows=int(rng.choice([0, 32, 96, 128])), dense_min_pct=int(rng.choice([2, 15, 60])),
-                     dense_min_nnz=int(rng.choice([0, 0, 1 << 22])), dense_cb=int(rng.choice([0, 16, 50])))
+                     dense_min_nnz=int(rng.choice([0, 0, 1 << 22])), dense_cb=int(rng.choice([0, 16, 50])),
+                     scalar_values=int(rng.choice([0, 1, 1])))
             for n, v in o.items(): opt(n, v)
             tag = "seed=%d k=%d %dx%d nnz=%d unique=%s sorted=%s %s" % (seed, k, nrows, ncols, nnz, unique, sort_rows, o)
             A = rng.standard_normal(k * nrows).astype(np.float32); B = rng.standard_normal(k * ncols).astype(np.float32)

@@ -1,0 +1,101 @@
+"""A *^ S over a plan with each nonzero's value fetched by a scalar load (option "scalar_values").
+
+Where a value comes from does not change what is multiplied or the order of the additions: the results must have the
+bits of the form that gathers the values lane by lane, for every k and shape of segment (full chunks of 64 nonzeros,
+short tails, segments shorter than a round of 8, empty rows), and both must agree with the oracle's float64 arbiter
+(reference: the product of BIDMat's dsmultT, jni/src/Arith.cu:206-248).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from bidmat_amd import hip_abi
+from util import Dev, make_plan
+from test_gpu_dense_rows import power_law_csc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def options(hip):
+    names = ("scalar_values", "dense_rows", "heavy_min", "seglen")
+    before = {n: hip.bidmat_get_option(n.encode()) for n in names}
+    yield hip
+    for n, v in before.items():
+        hip_abi.check(hip.bidmat_set_option(n.encode(), v))
+
+
+def product(hip, plan, k, d, out, scalar, beta=0):
+    hip_abi.check(hip.bidmat_set_option(b"scalar_values", scalar))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, d.v.ptr, out.ptr, beta, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    return out.numpy()
+
+
+# k: every lane layout of the walk (16, 32 and 64 lanes per nonzero with 4 floats per lane, 1 to 4 vectors per lane;
+# k % 4 != 0 takes one float per lane) and both sides of the limit below which the values stay with the gather
+@pytest.mark.parametrize("k", [7, 12, 32, 33, 64, 100, 128, 130, 256, 300, 512, 1028])
+@pytest.mark.parametrize("shape", [(700, 900, 40), (90, 3000, 25), (5000, 300, 150)], ids=["700x900", "90x3000", "5000x300"])
+def test_same_bits_as_the_gathered_values(options, k, shape):
+    hip = options
+    nrows, ncols, mean_len = shape
+    rng = np.random.default_rng(1000 * k + nrows)
+    ir, jc = power_law_csc(rng, nrows, ncols, mean_len, shuffle_rows=True)
+    nnz = ir.size
+    A = rng.standard_normal(k * ncols).astype(np.float32)
+    v = (1.0 - rng.random(nnz)).astype(np.float32)
+    v[0] = np.float32(np.inf)                    # the value at position 0 must reach its own nonzero only
+    c0 = int(np.searchsorted(jc, 0, side="right")) - 1          # the column of the nonzero at position 0
+    A[k * c0:k * (c0 + 1)] = 0.5
+    d = Dev(ir=ir, jc=jc, A=A, v=v)
+    d.zeros("G1", k * nrows); d.zeros("G0", k * nrows)
+    hip_abi.check(hip.bidmat_set_option(b"heavy_min", 2))       # rows cut by panels and rows in one piece
+    hip_abi.check(hip.bidmat_set_option(b"seglen", 64 if k % 2 else 512))
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    with_scalar = product(hip, plan, k, d, d.G1, 1)
+    gathered = product(hip, plan, k, d, d.G0, 0)
+    assert np.array_equal(with_scalar.view(np.uint32), gathered.view(np.uint32)), "the two ways to fetch a value differ"
+    r0 = int(ir[0])
+    rows = with_scalar.reshape(nrows, k)
+    assert np.all(np.isinf(rows[r0])), "the infinite value belongs to row %d" % r0
+    others = np.ones(nrows, bool); others[r0] = False
+    assert np.all(np.isfinite(rows[others])), "a slot past the end of a segment took the value at position 0"
+    v[0] = 1.0
+    d.v.upload(v)
+    got = product(hip, plan, k, d, d.G1, 1)
+    ref64, sa = oracle.fsmultT_f64(A, k, nrows, v, ir, jc, nthreads=8)
+    ok, worst = oracle.within_tolerance(got, ref64, sa, 1e-4)
+    assert ok, "A *^ S with scalar loads differs from the oracle: %.3e" % worst
+    twice = product(hip, plan, k, d, d.G1, 1, beta=1)
+    ok2, worst2 = oracle.within_tolerance(twice, 2 * ref64, 2 * sa, 1e-4)
+    assert ok2, worst2
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    d.free()
+
+
+def test_with_the_dense_block(options):
+    """The dense rows' segments are skipped by the kernel that fetches its values by scalar loads too."""
+    hip = options
+    nrows, ncols, k = 2000, 3000, 256
+    rng = np.random.default_rng(77)
+    ir, jc = power_law_csc(rng, nrows, ncols, 120, shuffle_rows=True)
+    nnz = ir.size
+    A = rng.standard_normal(k * ncols).astype(np.float32)
+    v = (1.0 - rng.random(nnz)).astype(np.float32)
+    d = Dev(ir=ir, jc=jc, A=A, v=v)
+    d.zeros("G1", k * nrows); d.zeros("G0", k * nrows)
+    before = hip.bidmat_get_option(b"dense_min_nnz")
+    hip_abi.check(hip.bidmat_set_option(b"dense_min_nnz", 0))
+    try:
+        plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+        assert int(hip.bidmat_plan_info(plan, b"dense_rows")) >= 32
+        a = product(hip, plan, k, d, d.G1, 1)
+        b = product(hip, plan, k, d, d.G0, 0)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        ref64, sa = oracle.fsmultT_f64(A, k, nrows, v, ir, jc, nthreads=8)
+        ok, worst = oracle.within_tolerance(a, ref64, sa, 1e-4)
+        assert ok, worst
+        hip_abi.check(hip.bidmat_plan_destroy(plan))
+    finally:
+        hip_abi.check(hip.bidmat_set_option(b"dense_min_nnz", before))
+    d.free()
