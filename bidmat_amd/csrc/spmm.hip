@@ -660,8 +660,10 @@ __global__ __launch_bounds__(BM_BLOCK) void k_reduce_segments(int k, int ldc, in
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// narrower groups (k <= 32 with 4 floats per lane) would need 8 and more scalar loads per step
-constexpr int kScalarValuesMinLanes = 16;
+// Scalar loads of the values where a nonzero's row takes the whole wave (k > 128; k > 32 with one float per lane).
+// With two nonzeros per step (k = 128, rows of 512 bytes) the scalar cache does not keep up with the gathers: on a
+// 400 M-nonzero pattern the walk over the rows cut by panels took 4.4 ms longer with scalar loads, the rest 0.4 ms.
+constexpr int kScalarValuesMinLanes = 64;
 
 template <bool PLAN>
 hipError_t launch_gather(const Shape& sh, const GatherArgs& a, long long nwaves, hipStream_t s) {

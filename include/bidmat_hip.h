@@ -457,7 +457,7 @@ int bidmat_device_info(char *arch, int arch_len, int *compute_units, long long *
  *   "dense_min_nnz" patterns with fewer nonzeros get no dense block (default 4 194 304)
  *   "dense_cb" columns per block of the dense product, each block giving one partial sum per dense row
  *              (default 0 = chosen from the column count so that the blocks fill the device evenly, about 330 to 400)
- *   "scalar_values" 1 (default): A *^ S over a plan, with the values in the caller's order and k > 32 (k > 8 when
+ *   "scalar_values" 1 (default): A *^ S over a plan, with the values in the caller's order and k > 128 (k > 32 when
  *              k is no multiple of 4 or an operand is not 16-byte aligned), fetches each nonzero's value by a scalar
  *              load from its position; 0: by one gather per lane and chunk of 64 nonzeros. Same bits either way.
  * Returns 0, or hipErrorInvalidValue for an unknown name / bad value; bidmat_get_option returns -2

@@ -32,9 +32,9 @@ def product(hip, plan, k, d, out, scalar, beta=0):
     return out.numpy()
 
 
-# k: every lane layout of the walk (16, 32 and 64 lanes per nonzero with 4 floats per lane, 1 to 4 vectors per lane;
-# k % 4 != 0 takes one float per lane) and both sides of the limit below which the values stay with the gather
-@pytest.mark.parametrize("k", [7, 12, 32, 33, 64, 100, 128, 130, 256, 300, 512, 1028])
+# k: every layout in which a nonzero's row takes the whole wave (1 to 4 vectors of 4 floats per lane; k % 4 != 0 takes
+# one float per lane, from k = 33 on) and both sides of the limits below which the values stay with the gather
+@pytest.mark.parametrize("k", [7, 32, 33, 64, 100, 128, 130, 132, 256, 300, 512, 1028])
 @pytest.mark.parametrize("shape", [(700, 900, 40), (90, 3000, 25), (5000, 300, 150)], ids=["700x900", "90x3000", "5000x300"])
 def test_same_bits_as_the_gathered_values(options, k, shape):
     hip = options
