@@ -43,9 +43,9 @@ HBM_PEAK_GBS = 8000.0
 # was taken on (concatenated); it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dsmultT", 100003320): (33.9e9, ("bidmat_amd/csrc/spmm.hip", "bidmat_amd/csrc/dense_rows.hip"), "0202f393a97265ba",
+    ("headline", "dsmultT", 100003320): (34.5e9, ("bidmat_amd/csrc/spmm.hip", "bidmat_amd/csrc/dense_rows.hip"), "0805189534e32e7f",
                                          "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, ("bidmat_amd/csrc/spmm.hip",), "651845315168280a",
+    ("C4", "dsmult", 38900534): (163.1e9, ("bidmat_amd/csrc/spmm.hip",), "4d5d107f8310c7b8",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 
@@ -293,7 +293,7 @@ def run_workload(lib, name, steps, warmup, scale, sections, cpu, cpu_sample, cal
         workload = "configs[1]+configs[2] pattern (Zipf(1.1) rows, Poisson(200) columns), step = DDS, A*S, A*^S"
         metric = "algorithmic GB/s (gathered operand charged once per nonzero) and nnz/s for DDS + A*S + A*^S at k=256, ~100M nnz (1 GPU)"
         roof_op = "dsmultT"
-        roof_kernel = ("stage 1 of A*^S, the time-dominant part of the step: k_gather_axpy<4,1,64,true> (the gathers of the pattern in plan "
+        roof_kernel = ("stage 1 of A*^S, the time-dominant part of the step: k_gather_axpy_sv<4,1,64,true> (the gathers of the pattern in plan "
                        "order) + k_dense_mfma<8,4> (the plan's densest rows as a dense block on the matrix cores) + k_dense_fold, "
                        "timed as one stretch of the stream; bytes and time are those of the three launches together")
     elif name in ("C1", "C4"):

@@ -77,10 +77,10 @@ __device__ __forceinline__ void load_chunk(const GatherArgs& a, int j0, int ahea
     }
 }
 
-// SV ("scalar values", plan order with the values in the caller's order): a nonzero's value is fetched by a scalar load
-// from its position, wave-uniform like the row index, instead of one 4-byte gather per lane and chunk. A lane-wise gather
-// of 64 values touches 64 cache lines, one look-up each in the per-CU vector cache that the row gathers already keep
-// busy (an eighth of their line requests at k = 256, a quarter at k = 128); the scalar cache is a path of its own to L2.
+// SV ("scalar values", for walks whose values sit behind a permutation): a nonzero's value is fetched by a scalar load
+// from its position, wave-uniform like the row index, instead of one 4-byte gather per lane and chunk. In plan order a
+// lane-wise gather of 64 values touches 64 cache lines, one look-up each in the per-CU vector cache that the row gathers
+// already keep busy (an eighth of their line requests at k = 256); the scalar cache is a path of its own to L2.
 // Read-only use: the values were written by earlier launches, and nothing here writes through that cache.
 typedef const float __attribute__((address_space(4))) scalar_float;
 
@@ -314,10 +314,12 @@ template <int W, int V, int LPN>
 __global__ __launch_bounds__(BM_BLOCK) void k_gather_listed(GatherArgs a) {
     gather_axpy_body<W, V, LPN, true>(a);
 }
-// The walk over all segments of a plan with the values in the caller's order: each value by a scalar load (SV above).
-template <int W, int V, int LPN>
+// The walks whose values sit behind a permutation - all segments of a plan with the values in the caller's order
+// (PLAN), the columns of a class-ordered pattern (A * S in passes over the classes) - with each value fetched by a
+// scalar load (SV above).
+template <int W, int V, int LPN, bool PLAN>
 __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy_sv(GatherArgs a) {
-    gather_axpy_body<W, V, LPN, true, true>(a);
+    gather_axpy_body<W, V, LPN, PLAN, true>(a);
 }
 
 // ---- DDS, the elementwise step and A*^S in one walk over a plan's segments (an NMF update's
@@ -675,8 +677,8 @@ hipError_t launch_gather(const Shape& sh, const GatherArgs& a, long long nwaves,
     if (sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                                      \
         if (PLAN && a.seglist != nullptr)                                                \
             hipLaunchKernelGGL((k_gather_listed<W_, V_, L_>), grid, block, 0, s, a);     \
-        else if (PLAN && L_ >= kScalarValuesMinLanes && a.perm != nullptr && !a.win_on && opt_scalar_values()) \
-            hipLaunchKernelGGL((k_gather_axpy_sv<W_, V_, (L_ >= kScalarValuesMinLanes ? L_ : 64)>), grid, block, 0, s, a); \
+        else if (L_ >= kScalarValuesMinLanes && a.perm != nullptr && !a.win_on && opt_scalar_values())    \
+            hipLaunchKernelGGL((k_gather_axpy_sv<W_, V_, (L_ >= kScalarValuesMinLanes ? L_ : 64), PLAN>), grid, block, 0, s, a); \
         else                                                                             \
             hipLaunchKernelGGL((k_gather_axpy<W_, V_, L_, PLAN>), grid, block, 0, s, a); \
         return hipGetLastError();                                                        \
