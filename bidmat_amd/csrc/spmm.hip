@@ -328,7 +328,7 @@ __global__ __launch_bounds__(BM_BLOCK) void k_gather_axpy_sv(GatherArgs a) {
 // memory unless the caller asks for them. The arithmetic is that of the two kernels it replaces, step for
 // step: the dot product in the lane layout and reduction tree of the DDS kernels (dotacc over the lane's
 // vectors, butterfly over the group), the accumulation in the order of k_gather_axpy.
-template <int W, int V, int LPN, bool FULL>
+template <int W, int V, int LPN, bool FULL, bool SV = false>
 __device__ __forceinline__ float fused_chunk(const GatherArgs& a, int mycol, float myval, int rem, int g, int l,
                                              const int (&eld)[V], const bool (&ev)[V], const Vec<W> (&rr)[V],
                                              Vec<W> (&acc)[V]) {
@@ -347,8 +347,14 @@ __device__ __forceinline__ float fused_chunk(const GatherArgs& a, int mycol, flo
             int c;
             if constexpr (LPN == 64) {
                 c = __builtin_amdgcn_readlane(mycol, it);
-                vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myval), it));
+                if constexpr (SV) {
+                    // (a slot past the end reads position 0: its product is masked below)
+                    vv[u] = ((scalar_float*)a.vals)[__builtin_amdgcn_readlane(__float_as_int(myval), it)];
+                } else {
+                    vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myval), it));
+                }
             } else {
+                static_assert(!SV, "scalar values: a nonzero's row takes the whole wave");
                 const int src = g * LPN + it;
                 c = lane_read(mycol, src);
                 vv[u] = lane_read(myval, src);
@@ -416,8 +422,8 @@ __device__ __forceinline__ float fused_chunk(const GatherArgs& a, int mycol, flo
     return keep;
 }
 
-template <int W, int V, int LPN>
-__global__ __launch_bounds__(BM_BLOCK) void k_fused_rows(GatherArgs a) {
+template <int W, int V, int LPN, bool SV>
+__device__ __forceinline__ void fused_rows_body(const GatherArgs& a) {
     const int lane = threadIdx.x & 63;
     const int g = lane / LPN, l = lane % LPN;
     const int xcd = blockIdx.x & 7;
@@ -446,14 +452,14 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fused_rows(GatherArgs a) {
     int rem = jend - jstart, j0 = jstart;
     int ccol;
     float cval;
-    load_chunk<true>(a, j0, 0, rem, q, ccol, cval);
+    load_chunk<true, SV>(a, j0, 0, rem, q, ccol, cval);
     while (rem > 0) {
         int ncol;
         float nval;
-        load_chunk<true>(a, j0, 64, rem - 64, q, ncol, nval);
+        load_chunk<true, SV>(a, j0, 64, rem - 64, q, ncol, nval);
         float keep;
-        if (rem >= 64) keep = fused_chunk<W, V, LPN, true>(a, ccol, cval, 64, g, l, eld, ev, rr, acc);
-        else keep = fused_chunk<W, V, LPN, false>(a, ccol, cval, rem, g, l, eld, ev, rr, acc);
+        if (rem >= 64) keep = fused_chunk<W, V, LPN, true, SV>(a, ccol, cval, 64, g, l, eld, ev, rr, acc);
+        else keep = fused_chunk<W, V, LPN, false, SV>(a, ccol, cval, rem, g, l, eld, ev, rr, acc);
         if (a.qout != nullptr && q < rem) {
             const int p = j0 + q;
             a.qout[a.qperm != nullptr ? a.qperm[p] : p] = keep;
@@ -473,6 +479,16 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fused_rows(GatherArgs a) {
         for (int i = 0; i < V; ++i)
             if (ev[i]) acc[i].store(outp + est[i]);
     }
+}
+
+template <int W, int V, int LPN>
+__global__ __launch_bounds__(BM_BLOCK) void k_fused_rows(GatherArgs a) {
+    fused_rows_body<W, V, LPN, false>(a);
+}
+// V in the caller's order and a row that takes the whole wave: each value by a scalar load (SV above)
+template <int W, int V>
+__global__ __launch_bounds__(BM_BLOCK) void k_fused_rows_sv(GatherArgs a) {
+    fused_rows_body<W, V, 64, true>(a);
 }
 
 // The same chain by columns (an LDA E-step: Q = op(V, DDS(A, B, S)), C = beta*C + A * Q): the column of B
@@ -910,7 +926,10 @@ hipError_t fused_segments(int k, int ldr, int lda, int nseg, const int* xcd_star
     dim3 grid((unsigned)nblk), block(BM_BLOCK);
 #define BM_CASE(W_, V_, L_)                                                              \
     if (sh.W == W_ && sh.V == V_ && sh.LPN == L_) {                                      \
-        hipLaunchKernelGGL((k_fused_rows<W_, V_, L_>), grid, block, 0, s, a);            \
+        if (L_ >= kScalarValuesMinLanes && a.perm != nullptr && opt_scalar_values())     \
+            hipLaunchKernelGGL((k_fused_rows_sv<W_, V_>), grid, block, 0, s, a);         \
+        else                                                                             \
+            hipLaunchKernelGGL((k_fused_rows<W_, V_, L_>), grid, block, 0, s, a);        \
         return hipGetLastError();                                                        \
     }
 #define BM_CASES(W_)                                                                     \

@@ -72,6 +72,18 @@ def test_fused_chain_has_the_bits_of_the_two_calls(hip, k, nrows, ncols, mean_le
     Q2, G2 = d.Q2.numpy()[:nnz], d.G2.numpy()
     assert np.array_equal(Q2.view(np.uint32), Q1.view(np.uint32)), "Q differs in %d places" % int((Q2 != Q1).sum())
     assert np.array_equal(G2.view(np.uint32), G1.view(np.uint32)), "G differs in %d places" % int((G2 != G1).sum())
+    if not stored:
+        # the values by a gather per lane instead of scalar loads (what k <= 128 takes anyway): the same bits
+        hip_abi.check(hip.bidmat_set_option(b"scalar_values", 0))
+        try:
+            d.put("Q5", np.full(max(nnz, 1), -5.0, np.float32))
+            d.put("G5", np.zeros(k * nrows, np.float32))
+            hip_abi.check(hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, d.v.ptr, OP_DIV, d.Q5.ptr, d.G5.ptr, 0, None))
+            hip_abi.check(hip.bidmat_synchronize())
+        finally:
+            hip_abi.check(hip.bidmat_set_option(b"scalar_values", 1))
+        assert np.array_equal(d.Q5.numpy()[:nnz].view(np.uint32), Q2.view(np.uint32))
+        assert np.array_equal(d.G5.numpy().view(np.uint32), G2.view(np.uint32))
     # without the product output, accumulating into G
     d.put("G3", G0)
     hip_abi.check(hip.bidmat_dds_dsmultT_plan(plan, k, d.A.ptr, d.B.ptr, None if stored else d.v.ptr, OP_DIV, None,
