@@ -99,3 +99,49 @@ def test_with_the_dense_block(options):
     finally:
         hip_abi.check(hip.bidmat_set_option(b"dense_min_nnz", before))
     d.free()
+
+
+def test_values_written_by_the_launch_before_in_a_replayed_graph(options):
+    """Q = V ./ DDS(A, B, S) and G = B *^ Q recorded into one HIP graph: the scalar loads of the second product must
+    see what the first wrote in the same replay (the scalar cache holds nothing over from the replay before)."""
+    import ctypes as C
+    hip = options
+    nrows, ncols, k = 1500, 2500, 256
+    rng = np.random.default_rng(31)
+    ir, jc = power_law_csc(rng, nrows, ncols, 60, shuffle_rows=True)
+    nnz = ir.size
+    A = (0.01 + rng.random(k * nrows)).astype(np.float32)
+    B = (0.01 + rng.random(k * ncols)).astype(np.float32)
+    v = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+    d = Dev(ir=ir, jc=jc, A=A, B=B, v=v)
+    d.zeros("Q", nnz); d.zeros("G", k * nrows); d.zeros("Q2", nnz); d.zeros("G2", k * nrows)
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    st = C.c_void_p()
+    hip_abi.check(hip.bidmat_stream_create(C.byref(st)))
+
+    def chain(q, g, stream):
+        hip_abi.check(hip.bidmat_dds_plan(plan, k, d.A.ptr, d.B.ptr, d.ir.ptr, d.jc.ptr, d.v.ptr, 3, q.ptr, 0, stream))
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.B.ptr, q.ptr, g.ptr, 0, stream))
+
+    chain(d.Q, d.G, st)                                   # sizes the stream's scratch
+    hip_abi.check(hip.bidmat_stream_synchronize(st))
+    hip_abi.check(hip.bidmat_graph_begin_capture(st))
+    chain(d.Q, d.G, st)
+    gx = C.c_void_p()
+    hip_abi.check(hip.bidmat_graph_end_capture(st, C.byref(gx)))
+    for rep in range(4):
+        newv = rng.gamma(1.0, 1.0, size=nnz).astype(np.float32)
+        d.v.upload(newv)
+        hip_abi.check(hip.bidmat_memset(d.G.ptr, 0xFF, d.G.nbytes))
+        hip_abi.check(hip.bidmat_graph_launch(gx, st))
+        hip_abi.check(hip.bidmat_stream_synchronize(st))
+        hip_abi.check(hip.bidmat_set_option(b"scalar_values", 0))
+        chain(d.Q2, d.G2, None)
+        hip_abi.check(hip.bidmat_synchronize())
+        hip_abi.check(hip.bidmat_set_option(b"scalar_values", 1))
+        assert np.array_equal(d.Q.numpy().view(np.int32), d.Q2.numpy().view(np.int32)), "replay %d, Q" % rep
+        assert np.array_equal(d.G.numpy().view(np.int32), d.G2.numpy().view(np.int32)), "replay %d, G" % rep
+    hip_abi.check(hip.bidmat_graph_destroy(gx))
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    hip_abi.check(hip.bidmat_stream_destroy(st))
+    d.free()
