@@ -185,7 +185,7 @@ hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* va
     // With values of the caller's (stored order) and a k the dense product is written for, the plan's dense rows go
     // through the matrix cores: their partial sums follow the segments' in the scratch, then the flag that tells
     // whether A held a value that is not finite (the dense rows' segments are then gathered after all).
-    const bool dense = vals != nullptr && plan->ndense > 0 && bm::dense_rows_fit(k) && bm::opt_dense_rows() > 0;
+    const bool dense = (vals != nullptr || plan->dvals != nullptr) && plan->ndense > 0 && bm::dense_rows_fit(k) && bm::opt_dense_rows() > 0;
     const size_t dfloats = dense ? (size_t)(plan->ndblocks + bm::dense_rows_fold(plan->ndblocks)) * (size_t)plan->ndense * (size_t)k : 0;
     float* partial = row_partial(plan, k, s, &err, dense ? dfloats + 64 : 0);
     if (!partial) return err;
@@ -195,10 +195,10 @@ hipError_t run_dsmultT(bidmat_plan* plan, int k, const float* A, const float* va
                                    vals ? plan->perm : nullptr, plan->segstart, partial, s,
                                    dense ? plan->dskip : nullptr, flag)) != hipSuccess) return err;
     if (dense) {
-        if ((err = bm::dense_rows_stage(k, plan->ncols, plan->ndense, plan->dcb, plan->ndblocks, A, vals, plan->dpos, dpart,
-                                        flag, s)) != hipSuccess) return err;
-        if ((err = bm::gather_segments_listed(k, plan->ndseg, plan->dseglist, flag, A, vals, plan->pc, plan->perm,
-                                              plan->segstart, partial, s)) != hipSuccess) return err;
+        if ((err = bm::dense_rows_stage(k, plan->ncols, plan->ndense, plan->dcb, plan->ndblocks, A, vals, plan->dpos, plan->dvals,
+                                        dpart, flag, s)) != hipSuccess) return err;
+        if ((err = bm::gather_segments_listed(k, plan->ndseg, plan->dseglist, flag, A, vals ? vals : plan->pvals, plan->pc,
+                                              vals ? plan->perm : nullptr, plan->segstart, partial, s)) != hipSuccess) return err;
     }
     if (between && (err = hipEventRecord(between, s)) != hipSuccess) return err;
     return bm::reduce_segments(k, plan->nrows, plan->rowptr, plan->rowseg, partial, C, beta, s,

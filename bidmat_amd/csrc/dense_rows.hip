@@ -17,6 +17,7 @@
 // that has no nonzero in that column. The kernel therefore watches the elements of A it streams and raises a
 // flag when one is not finite; stage 1 is then run for the dense rows' segments after all (a launch whose waves
 // return at once while the flag is down), and the row reduction picks the table that matches the flag.
+#include <algorithm>
 #include "plan.hpp"
 #include "common.hpp"
 #include "kernels.hpp"
@@ -195,7 +196,9 @@ __global__ __launch_bounds__(BM_BLOCK) void k_dense_seglist(int nd, const int* _
 // row l % 32 and, in register v, element 32 s + 8 (v / 4) + 4 (l / 32) + v % 4.
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-template <int NSW, int DEPTH>
+// DIRECT: `dpos` holds the values themselves (the plan's copy in the layout of dpos, 0 where a column has no nonzero
+// in the row) instead of positions into vals.
+template <int NSW, int DEPTH, bool DIRECT>
 __global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int cb, const float* __restrict__ A,
                                                    const float* __restrict__ vals, const int* __restrict__ dpos,
                                                    float* __restrict__ part, int* __restrict__ flag) {
@@ -221,7 +224,8 @@ __global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int
     // in flight before each step's matrix instructions, which takes the steps meant to be under way out of flight.
     const int clast = c1 - 1;
     auto rawpos = [&](int c) -> int { const int cc = c + half; return dpos[(size_t)(cc < c1 ? cc : clast) * nd + g * 32 + n]; };
-    auto rawval = [&](int p) -> float { return vals[p >= 0 ? p : 0]; };
+    auto rawval = [&](int p) -> float { return DIRECT ? __int_as_float(p) : vals[p >= 0 ? p : 0]; };
+    constexpr int NONE = DIRECT ? 0 : -1;        // what stands for "no nonzero": the bits of +0.0f / no position
     int eoff[NSW];
 #pragma unroll
     for (int s = 0; s < NSW; ++s) eoff[s] = ev[s] ? s * 32 : -n;          // an element past k: the column's first instead
@@ -240,7 +244,7 @@ __global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int
     for (int d = 0; d < DEPTH + 2; ++d) pos[d] = rawpos((int)c0 + 2 * d);
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-        bp[d] = ((int)c0 + 2 * d + half < c1) ? pos[d] : -1;
+        bp[d] = ((int)c0 + 2 * d + half < c1) ? pos[d] : NONE;
         bv[d] = rawval(bp[d]);
         rawA((int)c0 + 2 * d, a[d]);
     }
@@ -252,9 +256,9 @@ __global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int
             float ax[NSW];
 #pragma unroll
             for (int s = 0; s < NSW; ++s) ax[s] = (ev[s] && in) ? a[d][s] : 0.f;
-            const float bx = bp[d] >= 0 ? bv[d] : 0.f;
+            const float bx = (DIRECT || bp[d] >= 0) ? bv[d] : 0.f;
             const int cn = c + 2 * (d + DEPTH);
-            const int pnext = (cn + half < c1) ? pos[DEPTH] : -1;
+            const int pnext = (cn + half < c1) ? pos[DEPTH] : NONE;
 #pragma unroll
             for (int q = 0; q < DEPTH + 1; ++q) pos[q] = pos[q + 1];
             pos[DEPTH + 1] = rawpos(cn + 4);
@@ -327,7 +331,7 @@ int dense_rows_fold(int ndblocks) { return ndblocks < 16 ? ndblocks : 16; }
 
 hipError_t drop_dense(bidmat_plan* p) {
     hipError_t e = hipSuccess;
-    for (void** b : {&p->block_dense, (void**)&p->dpos}) {
+    for (void** b : {&p->block_dense, (void**)&p->dpos, (void**)&p->dvals}) {
         if (*b) {
             hipError_t f = pool_free(*b);
             if (f != hipSuccess) e = f;
@@ -463,16 +467,52 @@ bool dense_rows_fit(int k) { return k > 64 && k <= 256; }
 
 // part: (ndblocks + dense_rows_fold(ndblocks)) * nd partial sums of k floats, the folded ones last. *flag (cleared by the caller's stage 1) is raised when A holds a
 // value that is not finite.
+namespace {
+__global__ __launch_bounds__(BM_BLOCK) void k_dense_values(long long n, const int* __restrict__ dpos, const float* __restrict__ data,
+                                                           float* __restrict__ dvals) {
+    const long long stride = (long long)gridDim.x * BM_BLOCK;
+    for (long long i = (long long)blockIdx.x * BM_BLOCK + threadIdx.x; i < n; i += stride) {
+        const int p = dpos[i];
+        dvals[i] = p >= 0 ? data[p] : 0.f;
+    }
+}
+}  // namespace
+
+hipError_t dense_rows_set_values(bidmat_plan* plan, const float* data, hipStream_t s) {
+    if (plan->ndense <= 0 || plan->dpos == nullptr) return hipSuccess;
+    const size_t n = (size_t)plan->ncols * (size_t)plan->ndense;
+    if (plan->dvals == nullptr) {
+        hipError_t e;
+        plan->dvals = static_cast<float*>(pool_alloc(sizeof(float) * n, &e));
+        if (plan->dvals == nullptr) {
+            (void)hipGetLastError();
+            return e == hipErrorOutOfMemory ? hipSuccess : e;       // no room: stored values go without the dense block
+        }
+        plan->dense_bytes += sizeof(float) * n;
+        plan->row_bytes += sizeof(float) * n;
+    }
+    hipLaunchKernelGGL(k_dense_values, dim3((unsigned)std::min<long long>(16384, ((long long)n + BM_BLOCK - 1) / BM_BLOCK)), dim3(BM_BLOCK), 0, s, (long long)n, plan->dpos, data, plan->dvals);
+    return hipGetLastError();
+}
+
 hipError_t dense_rows_stage(int k, int ncols, int nd, int cb, int ndblocks, const float* A, const float* vals,
-                            const int* dpos, float* part, int* flag, hipStream_t s) {
+                            const int* dpos, const float* dvals, float* part, int* flag, hipStream_t s) {
     if (nd <= 0 || ndblocks <= 0) return hipSuccess;
     const int G = nd >> 5;
     const long long nblk = (long long)((ndblocks + 7) / 8) * 8 * G;
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (k > 128)
-        hipLaunchKernelGGL((k_dense_mfma<8, 4>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
-    else
-        hipLaunchKernelGGL((k_dense_mfma<4, 4>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
+    if (vals == nullptr) {
+        if (dvals == nullptr) return hipErrorInvalidValue;
+        const int* bits = reinterpret_cast<const int*>(dvals);
+        if (k > 128)
+            hipLaunchKernelGGL((k_dense_mfma<8, 4, true>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, bits, part, flag);
+        else
+            hipLaunchKernelGGL((k_dense_mfma<4, 4, true>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, bits, part, flag);
+    } else if (k > 128) {
+        hipLaunchKernelGGL((k_dense_mfma<8, 4, false>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
+    } else {
+        hipLaunchKernelGGL((k_dense_mfma<4, 4, false>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
+    }
     const int nfold = dense_rows_fold(ndblocks);
     hipLaunchKernelGGL(k_dense_fold, dim3((unsigned)(nfold * nd)), dim3(64), 0, s, k, nd, ndblocks, (ndblocks + nfold - 1) / nfold, part,
                        part + (size_t)ndblocks * (size_t)nd * (size_t)k);

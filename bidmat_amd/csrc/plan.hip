@@ -547,6 +547,8 @@ hipError_t plan_set_values(bidmat_plan* p, const float* data, hipStream_t s) {
     if (p->sides & PLAN_ROWS) {
         if ((e = value_buffer(&p->pvals, p->nnz)) != hipSuccess) return e;
         hipLaunchKernelGGL(k_permute_values, grid, block, 0, s, (long long)p->nnz, data, p->perm, p->pvals);
+        // the dense block of A *^ S reads its values in the layout of its position table
+        if ((e = dense_rows_set_values(p, data, s)) != hipSuccess) return e;
     }
     if ((p->sides & PLAN_COLS) && p->ncls == 8) {
         // A*S in passes over row classes and the fused step of DDS read their values in class order

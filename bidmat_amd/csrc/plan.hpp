@@ -52,6 +52,8 @@ struct bidmat_plan {
     int* drank = nullptr;        // [nrows]  rank of a dense row (by count, descending), -1 for every other row
     int* drow = nullptr;         // [ndense] row of every rank
     int* dpos = nullptr;         // [ncols*ndense] position (stored order) of column c's nonzero in dense row d, or -1
+    float* dvals = nullptr;      // [ncols*ndense] the stored values at those positions, 0 where there is none (optional:
+                                 // bidmat_plan_set_values on a plan with a dense block)
     unsigned char* dskip = nullptr;  // [nseg] 1: segment of a dense row
     int* dseglist = nullptr;     // [ndseg] those segments
     int* rowptr2 = nullptr;      // [nrows+1] like rowptr / rowseg, a dense row's entries being the partial sums
@@ -115,6 +117,10 @@ hipError_t drop_dense(bidmat_plan* p);
 bool dense_rows_fit(int k);      // the dense product is written for 64 < k <= 256
 int dense_rows_max();
 int dense_rows_fold(int ndblocks);   // partial sums per dense row that reach the row reduction
+// vals == nullptr: the values come from dvals (the plan's copy in the layout of dpos) instead of vals[dpos[..]]
 hipError_t dense_rows_stage(int k, int ncols, int nd, int cb, int ndblocks, const float* A, const float* vals,
-                            const int* dpos, float* part, int* flag, hipStream_t s);
+                            const int* dpos, const float* dvals, float* part, int* flag, hipStream_t s);
+// dvals[i] = dpos[i] >= 0 ? data[dpos[i]] : 0 for the ncols*nd slots of a plan's dense block (allocates dvals on first use;
+// without memory for it the plan keeps none and calls with stored values walk the segments of every row)
+hipError_t dense_rows_set_values(bidmat_plan* plan, const float* data, hipStream_t s);
 }  // namespace bm

@@ -196,7 +196,7 @@ int bidmat_plan_array(const bidmat_plan *plan, const char *name, const void **dp
  * rows of S).
  * Dense block: when the pattern has rows with a nonzero in a large share of the columns (options "dense_rows",
  * "dense_min_pct", "dense_min_nnz" below; plan info "dense_rows"), the plan ranks up to 128 of them at build time and,
- * for 64 < k <= 256 and values passed in Sdata, their columns of C are computed as a dense product on the matrix
+ * for 64 < k <= 256 (values passed in Sdata, or stored by bidmat_plan_set_values), their columns of C are computed as a dense product on the matrix
  * cores (the columns of A streamed once per 32 rows, absent entries as zeros) instead of one gather per nonzero.
  * Only the order in which those rows' terms are added changes (fixed by the pattern: same bits from run to run,
  * within the 1e-4 tolerance of the path); every other row keeps its bits.  A value of A that is not finite makes the
@@ -214,7 +214,8 @@ int bidmat_dsmultT_plan_staged(bidmat_plan *plan, int k, const float *A, const f
  * stays in L2); the remaining nnz - heavy nonzeros are gathered once each with no reuse.  Blocking. */
 long long bidmat_plan_heavy_nnz(const bidmat_plan *plan);
 
-/* The values of the pattern in plan order, stored in the plan (nnz floats): afterwards
+/* The values of the pattern in plan order, stored in the plan (nnz floats; on a plan with a dense block also the
+ * dense rows' values in the layout of the block, ncols x dense rows floats): afterwards
  * bidmat_dsmultT_plan, bidmat_sdmult_plan and bidmat_spsum_rows_plan accept Sdata == NULL and stream
  * the stored values instead of fetching every value through the plan's permutation; so does
  * bidmat_dsmult_plan when the plan carries a row-class ordering of its columns and no column is longer

@@ -274,3 +274,58 @@ def test_graph_replay_with_the_dense_block(dense_options):
     hip_abi.check(hip.bidmat_plan_destroy(plan))
     hip_abi.check(hip.bidmat_stream_destroy(st))
     d.free()
+
+
+@pytest.mark.parametrize("k", [96, 256, 130])
+def test_values_stored_in_the_plan_take_the_dense_block_too(dense_options, k):
+    """bidmat_plan_set_values keeps the dense rows' values in the layout of the block's position table: a call without
+    Sdata multiplies the same numbers in the same order as a call that passes them, so the results agree bit for bit,
+    also after the values have been set anew, and a value of A that is not finite falls back to the segments."""
+    hip = dense_options
+    nrows, ncols = 2500, 3500
+    rng = np.random.default_rng(40 + k)
+    ir, jc = power_law_csc(rng, nrows, ncols, 90, shuffle_rows=True)
+    nnz = ir.size
+    A = rng.standard_normal(k * ncols).astype(np.float32)
+    v = rng.standard_normal(nnz).astype(np.float32)
+    d = Dev(ir=ir, jc=jc, A=A, v=v)
+    d.zeros("G", k * nrows); d.zeros("G0", k * nrows)
+    plan = make_plan(hip, nrows, ncols, nnz, d.ir, d.jc, k)
+    nd = plan_info(hip, plan, "dense_rows")
+    assert nd >= 32
+    before = hip.bidmat_plan_bytes(plan)
+    for rep in range(2):
+        passed = run(hip, plan, k, d.A, d.v, d.G)
+        hip_abi.check(hip.bidmat_plan_set_values(plan, d.v.ptr, None))
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, None, d.G0.ptr, 0, None))
+        hip_abi.check(hip.bidmat_synchronize())
+        stored = d.G0.numpy()
+        assert np.array_equal(stored.view(np.uint32), passed.view(np.uint32)), "stored and passed values differ (round %d)" % rep
+        if rep == 0:
+            assert hip.bidmat_plan_bytes(plan) >= before + 4 * nnz + 4 * ncols * nd, "the plan counts what it stores"
+            ref64, sa = oracle.fsmultT_f64(A, k, nrows, v, ir, jc, nthreads=8)
+            ok, worst = oracle.within_tolerance(stored, ref64, sa, 1e-4)
+            assert ok, worst
+            v = rng.standard_normal(nnz).astype(np.float32)         # other values: set again
+            d.v.upload(v)
+    # the stored values without the dense block (option at call time): the walk over every row's segments
+    hip_abi.check(hip.bidmat_set_option(b"dense_rows", 0))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, None, d.G.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    hip_abi.check(hip.bidmat_set_option(b"dense_rows", 128))
+    walk = d.G.numpy()
+    ref64, sa = oracle.fsmultT_f64(A, k, nrows, v, ir, jc, nthreads=8)
+    ok, worst = oracle.within_tolerance(walk, ref64, sa, 1e-4)
+    assert ok, worst
+    assert not np.array_equal(walk, stored), "the dense rows took the same path"
+    # a value of A that is not finite: the call falls back to exactly that walk
+    A2 = A.copy(); A2[k * 17 + 3] = -np.inf
+    d.A.upload(A2)
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, None, d.G0.ptr, 0, None))
+    hip_abi.check(hip.bidmat_set_option(b"dense_rows", 0))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, d.A.ptr, None, d.G.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    hip_abi.check(hip.bidmat_set_option(b"dense_rows", 128))
+    assert np.array_equal(d.G0.numpy(), d.G.numpy(), equal_nan=True)
+    hip_abi.check(hip.bidmat_plan_destroy(plan))
+    d.free()
