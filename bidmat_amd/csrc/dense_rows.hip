@@ -199,9 +199,9 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 // DIRECT: `dpos` holds the values themselves (the plan's copy in the layout of dpos, 0 where a column has no nonzero
 // in the row) instead of positions into vals.
 template <int NSW, int DEPTH, bool DIRECT>
-__global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int cb, const float* __restrict__ A,
-                                                   const float* __restrict__ vals, const int* __restrict__ dpos,
-                                                   float* __restrict__ part, int* __restrict__ flag) {
+__device__ __forceinline__ void dense_mfma_body(int k, int ncols, int nd, int cb, const float* __restrict__ A,
+                                                const float* __restrict__ vals, const int* __restrict__ dpos,
+                                                float* __restrict__ part, int* __restrict__ flag) {
     const int lane = threadIdx.x;
     const int G = nd >> 5;
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
@@ -290,6 +290,20 @@ __global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int
                     if (el + t < k) out[el + t] = acc[s][4 * v4 + t];
             }
         }
+}
+
+template <int NSW, int DEPTH>
+__global__ __launch_bounds__(64) void k_dense_mfma(int k, int ncols, int nd, int cb, const float* __restrict__ A,
+                                                   const float* __restrict__ vals, const int* __restrict__ dpos,
+                                                   float* __restrict__ part, int* __restrict__ flag) {
+    dense_mfma_body<NSW, DEPTH, false>(k, ncols, nd, cb, A, vals, dpos, part, flag);
+}
+// the same with the values stored in the plan (dvals, in the layout of dpos)
+template <int NSW, int DEPTH>
+__global__ __launch_bounds__(64) void k_dense_mfma_stored(int k, int ncols, int nd, int cb, const float* __restrict__ A,
+                                                          const float* __restrict__ dvals, float* __restrict__ part,
+                                                          int* __restrict__ flag) {
+    dense_mfma_body<NSW, DEPTH, true>(k, ncols, nd, cb, A, nullptr, reinterpret_cast<const int*>(dvals), part, flag);
 }
 
 // The partial sums of `per` consecutive blocks of columns added up, block after block: one wave per (chunk of
@@ -503,15 +517,14 @@ hipError_t dense_rows_stage(int k, int ncols, int nd, int cb, int ndblocks, cons
     if (nblk > 0x7fffffffLL) return hipErrorInvalidValue;
     if (vals == nullptr) {
         if (dvals == nullptr) return hipErrorInvalidValue;
-        const int* bits = reinterpret_cast<const int*>(dvals);
         if (k > 128)
-            hipLaunchKernelGGL((k_dense_mfma<8, 4, true>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, bits, part, flag);
+            hipLaunchKernelGGL((k_dense_mfma_stored<8, 4>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, dvals, part, flag);
         else
-            hipLaunchKernelGGL((k_dense_mfma<4, 4, true>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, bits, part, flag);
+            hipLaunchKernelGGL((k_dense_mfma_stored<4, 4>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, dvals, part, flag);
     } else if (k > 128) {
-        hipLaunchKernelGGL((k_dense_mfma<8, 4, false>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
+        hipLaunchKernelGGL((k_dense_mfma<8, 4>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
     } else {
-        hipLaunchKernelGGL((k_dense_mfma<4, 4, false>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
+        hipLaunchKernelGGL((k_dense_mfma<4, 4>), dim3((unsigned)nblk), dim3(64), 0, s, k, ncols, nd, cb, A, vals, dpos, part, flag);
     }
     const int nfold = dense_rows_fold(ndblocks);
     hipLaunchKernelGGL(k_dense_fold, dim3((unsigned)(nfold * nd)), dim3(64), 0, s, k, nd, ndblocks, (ndblocks + nfold - 1) / nfold, part,
