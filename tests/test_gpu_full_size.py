@@ -86,6 +86,22 @@ def test_headline_pattern_dds_dsmult_dsmultT(hip):
     assert float(np.max(np.abs(C2.astype(np.float64) - Cm) / np.abs(Cm))) <= 2e-5    # A*S: another fixed order of the same sums
     del C2
     dP2.free(), dC2.free()
+    # A*^S at full size by the other ways to fetch a value: a gather per lane instead of scalar loads, and the values
+    # stored in the plan (plan order, the dense rows' in the layout of the dense block): the same bits each time
+    dG2 = DeviceArray(k * nrows, np.float32)
+    assert hip.bidmat_get_option(b"scalar_values") == 1
+    hip_abi.check(hip.bidmat_set_option(b"scalar_values", 0))
+    try:
+        hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, dAT.ptr, dv.ptr, dG2.ptr, 0, None))
+        hip_abi.check(hip.bidmat_synchronize())
+    finally:
+        hip_abi.check(hip.bidmat_set_option(b"scalar_values", 1))
+    assert np.array_equal(dG2.numpy().view(np.uint32), G.view(np.uint32)), "A*^S: scalar loads and gathered values differ"
+    hip_abi.check(hip.bidmat_plan_set_values(plan, dv.ptr, None))
+    hip_abi.check(hip.bidmat_dsmultT_plan(plan, k, dAT.ptr, None, dG2.ptr, 0, None))
+    hip_abi.check(hip.bidmat_synchronize())
+    assert np.array_equal(dG2.numpy().view(np.uint32), G.view(np.uint32)), "A*^S: stored and passed values differ"
+    dG2.free()
     rng = np.random.default_rng(0)
     # --- the three products agree: <A*S, B> == sum_j v_j * DDS_j ; <B*^S, A> checked with A_T's own DDS
     f1 = np.dot(Cm.astype(np.float64), B.astype(np.float64))
