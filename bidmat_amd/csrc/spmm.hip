@@ -380,8 +380,7 @@ __device__ __forceinline__ float fused_chunk(const GatherArgs& a, int mycol, flo
                 float s = 0.f;
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
-                    const Vec<W> x = ev[i] ? rr[i] : Vec<W>::zero();   // lanes past k contribute nothing
-                    s = x.dotacc(bv[u][i], s);
+                    s = rr[i].dotacc(bv[u][i], s);                     // rr is zero in lanes past k
                 }
                 sums[u] = s;
             }
@@ -405,8 +404,7 @@ __device__ __forceinline__ float fused_chunk(const GatherArgs& a, int mycol, flo
                 float s = 0.f;
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
-                    const Vec<W> x = ev[i] ? rr[i] : Vec<W>::zero();   // lanes past k contribute nothing
-                    s = x.dotacc(bv[u][i], s);
+                    s = rr[i].dotacc(bv[u][i], s);                     // rr is zero in lanes past k
                 }
                 s = group_allsum<LPN>(s);
                 qq[u] = ok[u] ? binop_rt(a.opn, vv[u], s) : 0.f;
@@ -446,7 +444,8 @@ __device__ __forceinline__ void fused_rows_body(const GatherArgs& a) {
         ev[i] = est[i] < a.k;
         eld[i] = ev[i] ? est[i] : 0;
         acc[i] = Vec<W>::zero();
-        rr[i] = Vec<W>::load(rp + eld[i]);
+        // lanes past k hold zeros: they contribute nothing to the dot products (masked here, once, not per nonzero)
+        rr[i] = ev[i] ? Vec<W>::load(rp + eld[i]) : Vec<W>::zero();
     }
     const int q = l * (64 / LPN) + g;
     int rem = jend - jstart, j0 = jstart;
@@ -540,7 +539,8 @@ __global__ __launch_bounds__(BM_BLOCK) void k_fused_cols(GatherArgs a) {
         ev[i] = est[i] < a.k;
         eld[i] = ev[i] ? est[i] : 0;
         acc[i] = Vec<W>::zero();
-        rr[i] = Vec<W>::load(rp + eld[i]);
+        // lanes past k hold zeros: they contribute nothing to the dot products (masked here, once, not per nonzero)
+        rr[i] = ev[i] ? Vec<W>::load(rp + eld[i]) : Vec<W>::zero();
     }
     constexpr bool EARLY_ADDEND = V <= 2;            // as in k_gather_axpy
     Vec<W> addend[V];
