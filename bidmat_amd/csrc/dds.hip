@@ -58,7 +58,7 @@ __device__ __forceinline__ float dds_round(const float* __restrict__ A, int k, i
         else r = lane_read(myrow, g * LPN + it);
         if (!PRED || (it * NG + g) < rem) {
             if constexpr (LDSROWS) {
-                const float* hp = hot_lds + r * k;
+                const float* hp = hot_lds + __mul24(r, k);      // a rank times k: below the LDS size, a full-rate multiply
 #pragma unroll
                 for (int i = 0; i < V; ++i) av[u][i] = Vec<W>::load(hp + eld[i]);
             } else {
