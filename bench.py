@@ -43,9 +43,9 @@ HBM_PEAK_GBS = 8000.0
 # was taken on (concatenated); it is reported only for that exact workload and dropped (null) as soon as the
 # kernel source differs.
 MEASURED_TRAFFIC = {
-    ("headline", "dsmultT", 100003320): (34.5e9, ("bidmat_amd/csrc/spmm.hip", "bidmat_amd/csrc/dense_rows.hip"), "860826aceba394f4",
+    ("headline", "dsmultT", 100003320): (34.5e9, ("bidmat_amd/csrc/spmm.hip", "bidmat_amd/csrc/dense_rows.hip"), "3675babc718fa305",
                                          "profiles/headline_kernel_trace_and_hbm_counters.txt"),
-    ("C4", "dsmult", 38900534): (163.1e9, ("bidmat_amd/csrc/spmm.hip",), "473baee5b8087ba5",
+    ("C4", "dsmult", 38900534): (163.1e9, ("bidmat_amd/csrc/spmm.hip",), "d18cc32221214df7",
                                  "profiles/other_workloads_kernel_trace_and_hbm_counters.txt"),
 }
 
