@@ -45,6 +45,21 @@ __global__ __launch_bounds__(BM_BLOCK) void k_csc_validate(int nrows, int ncols,
     if (bad) atomicOr(flags, bad);
 }
 
+// rowptr[r] = number of entries of the sorted array a[0..n) that are smaller than r, for r = 0..nrows: one thread per r
+// and a binary search. (Closing the columns from the positions where a column starts, as k_compress_cols does, leaves a
+// run of absent columns to one thread: among the light rows of a plan the panel-cut rows are absent, with row indices ordered
+// by frequency the first several thousand, closed one store after the other in 0.2 ms.)
+__global__ __launch_bounds__(BM_BLOCK) void k_lower_bounds(int n, int nrows, const int* __restrict__ a, int* __restrict__ rowptr) {
+    const long long r = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
+    if (r > nrows) return;
+    int lo = 0, hi = n;                  // first position whose row is >= r
+    while (lo < hi) {
+        const int mid = (int)(((long long)lo + hi) >> 1);
+        if (a[mid] < (int)r) lo = mid + 1; else hi = mid;
+    }
+    rowptr[r] = lo;
+}
+
 // Position j closes the columns ic[j-1]+1 .. ic[j] (with ic[-1] = -1 and ic[nnz] = ncols): jc[c] = j for
 // each of them. A thread takes four consecutive positions (one 128-bit load when ic is 16-byte aligned).
 __global__ __launch_bounds__(BM_BLOCK) void k_compress_cols(int ncols, int nnz, const int* __restrict__ ic,
@@ -327,8 +342,17 @@ hipError_t csc_validate(int nrows, int ncols, int nnz, const int* ir, const int*
     return hipGetLastError();
 }
 
+hipError_t sorted_lower_bounds(int ncols, int nnz, const int* ic, int* jc, hipStream_t s) {
+    if (ncols < 0 || nnz < 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_lower_bounds, dim3((unsigned)(((long long)ncols + 1 + BM_BLOCK - 1) / BM_BLOCK)), dim3(BM_BLOCK), 0, s, nnz, ncols, ic, jc);
+    return hipGetLastError();
+}
+
 hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStream_t s) {
     if (ncols < 0 || nnz < 0) return hipErrorInvalidValue;
+    // few columns for the entries: a search per column costs no more than a pass over the entries, and a long run of
+    // empty columns is not left to one thread
+    if ((long long)ncols * 128 < (long long)nnz) return sorted_lower_bounds(ncols, nnz, ic, jc, s);
     long long nblk = ((long long)nnz / 4 + 1 + BM_BLOCK - 1) / BM_BLOCK;
     hipLaunchKernelGGL(k_compress_cols, dim3((unsigned)nblk), dim3(BM_BLOCK), 0, s, ncols, nnz, ic, jc);
     return hipGetLastError();

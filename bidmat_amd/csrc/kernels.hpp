@@ -29,6 +29,8 @@ int opt_scalar_values();   // A *^ S over a plan fetches the caller's values by 
 // ---- CSC utilities (csc_util.hip)
 hipError_t csc_expand_cols(int ncols, int nnz, const int* jc, int* ic, hipStream_t s);
 hipError_t coo_compress_cols(int ncols, int nnz, const int* ic, int* jc, hipStream_t s);
+// jc[c] = number of entries of the sorted ic[0..nnz) below c, c = 0..ncols, by a binary search per c
+hipError_t sorted_lower_bounds(int ncols, int nnz, const int* ic, int* jc, hipStream_t s);
 // ir[j] = j - jc[c]: the implied rows of a sparse matrix stored without row indices
 hipError_t csc_implicit_rows(int ncols, int nnz, const int* jc, int* ir, hipStream_t s);
 // *d_flags (device int) = bit set of violated rules: 1 jc[0] != 0, 2 jc decreasing or outside

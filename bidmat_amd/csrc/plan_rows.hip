@@ -417,21 +417,6 @@ __global__ __launch_bounds__(RB_FILL_THREADS) void k_fill_block(int heavy_total,
     }
 }
 
-// rowptr[r] = number of entries of the sorted rows a[0..n) that are smaller than r, for r = 0..nrows: one thread per row
-// and a binary search. (Closing the rows from the positions where a row starts, as k_compress_cols does, leaves a run of
-// absent rows to one thread: the panel-cut rows are absent here, and with row indices ordered by frequency they are the
-// first several thousand rows, closed one store after the other in 0.2 ms.)
-__global__ __launch_bounds__(BM_BLOCK) void k_lower_bounds(int n, int nrows, const int* __restrict__ a, int* __restrict__ rowptr) {
-    const long long r = (long long)blockIdx.x * BM_BLOCK + threadIdx.x;
-    if (r > nrows) return;
-    int lo = 0, hi = n;                  // first position whose row is >= r
-    while (lo < hi) {
-        const int mid = (int)(((long long)lo + hi) >> 1);
-        if (a[mid] < (int)r) lo = mid + 1; else hi = mid;
-    }
-    rowptr[r] = lo;
-}
-
 // ---- light rows: one stable pass by bits [shift, shift+bits) of the row.
 // counts go to table[bin*ntiles + tile], so that one flat exclusive scan of the table gives every
 // (bin, tile) its first output position.
@@ -775,9 +760,7 @@ hipError_t build_rows_binned(bidmat_plan* plan, const int* ir, const int* jc, co
             cur ^= 1;
         }
         // lr[cur]: the rows of the light nonzeros in plan order
-        hipLaunchKernelGGL(k_lower_bounds, dim3((unsigned)(((long long)nrows + 1 + BM_BLOCK - 1) / BM_BLOCK)), dim3(BM_BLOCK), 0, s, nlight, nrows,
-                           lr[cur], lrowptr);
-        RB_CHECK(hipGetLastError());
+        RB_CHECK(sorted_lower_bounds(nrows, nlight, lr[cur], lrowptr, s));
     } else {
         RB_CHECK(fill_i32(lrowptr, (long long)nrows + 1, 0, s));
     }
